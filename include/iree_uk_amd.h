@@ -1,0 +1,336 @@
+/*
+ * C-ABI of the MI355X (gfx950) data-tiled matmul ukernels: pack, mmt4d, unpack.
+ *
+ * The three entry points keep the argument lists, params structs, flag values,
+ * type enums and tile-size conventions of the IREE CPU ukernels so that a
+ * caller written against
+ *   runtime/src/iree/builtins/ukernel/{mmt4d.h,pack.h,unpack.h,exported_bits.h}
+ * links against this library unchanged.  Offsets and strides are counted in
+ * elements, M/N/K of mmt4d are tile counts, and only the outermost stride of
+ * each 4-D operand is free (inner dims are dense).
+ *
+ * What differs from the CPU ukernels:
+ *   - the work runs as HIP kernels on the current HIP device;
+ *   - buffers may be device memory (zero-copy, stream-ordered: the call
+ *     returns once the kernels are enqueued on the calling thread's stream,
+ *     see iree_uk_amd_set_stream / iree_uk_amd_synchronize) or host memory
+ *     (staged through the GPU; the call returns when the result is in the
+ *     host buffer);
+ *   - `cpu_data` is accepted and ignored (NULL is allowed);
+ *   - one mmt4d type value is added for f8E4M3FN x f8E4M3FN -> f32.
+ *
+ * Plain C; no HIP or torch types appear in any signature.
+ */
+#ifndef IREE_UK_AMD_H_
+#define IREE_UK_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IREE_UK_AMD_EXPORT __attribute__((visibility("default")))
+
+/* iree_uk_index_t is int64 on 64-bit targets (common.h:269-275). */
+typedef int64_t iree_uk_index_t;
+
+/*===--------------------------------------------------------------------===*/
+/* Flag values (exported_bits.h:29-83). These are shared with the compiler   */
+/* and therefore frozen.                                                     */
+/*===--------------------------------------------------------------------===*/
+
+/* mmt4d type enum, low byte of flags (exported_bits.h:29-41). */
+enum {
+  IREE_UK_FLAG_MMT4D_TYPE_MASK = 0xFF,
+  IREE_UK_FLAG_MMT4D_TYPE_NONE = 0x00,
+  IREE_UK_FLAG_MMT4D_TYPE_F32F32F32 = 0x01,
+  IREE_UK_FLAG_MMT4D_TYPE_S8S8S32 = 0x02,
+  IREE_UK_FLAG_MMT4D_TYPE_F16F16F32 = 0x03,
+  IREE_UK_FLAG_MMT4D_TYPE_F16F16F16 = 0x04,
+  IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32 = 0x05,
+  IREE_UK_FLAG_MMT4D_TYPE_BF16BF16BF16 = 0x06,
+  IREE_UK_FLAG_MMT4D_TYPE_S16S16S32 = 0x07,
+  IREE_UK_FLAG_MMT4D_TYPE_S16U4S32 = 0x08,
+  IREE_UK_FLAG_MMT4D_TYPE_S16S8S32 = 0x09,
+  IREE_UK_FLAG_MMT4D_TYPE_S8S4S32 = 0x0A,
+  IREE_UK_FLAG_MMT4D_TYPE_END = 0x0B,
+  /* The one deliberate addition: 8-bit float E4M3FN operands, f32 result.
+   * Taken outside the contiguous upstream range so that a future upstream
+   * 0x0B cannot collide. Element semantics follow
+   * runtime/src/iree/base/internal/math.h:324-362,557-560 (no Inf, NaN is
+   * S.1111.111, subnormals kept) and the f32-accumulating reference loop in
+   * tools/testing/e2e/iree-e2e-matmul-test.cc:123-142. */
+  IREE_UK_AMD_FLAG_MMT4D_TYPE_F8E4M3FNF8E4M3FNF32 = 0x80,
+};
+
+/* mmt4d bit flags (exported_bits.h:44-46). */
+enum {
+  IREE_UK_FLAG_MMT4D_ACCUMULATE = 0x100,
+  IREE_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION = 0x200,
+  IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS = 0x400,
+};
+
+/* iree_uk_mmt4d_info result bits (exported_bits.h:49). On this target the bit
+ * means "an MFMA kernel (not the scalar fallback kernel) serves this case". */
+enum {
+  IREE_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION = 0x1,
+};
+
+/* pack type enum and bit flags (exported_bits.h:56-66). */
+enum {
+  IREE_UK_FLAG_PACK_TYPE_MASK = 0xFF,
+  IREE_UK_FLAG_PACK_TYPE_NONE = 0x00,
+  IREE_UK_FLAG_PACK_TYPE_F32F32 = 0x01,
+  IREE_UK_FLAG_PACK_TYPE_I8I8 = 0x02,
+  IREE_UK_FLAG_PACK_TYPE_I32I32 = 0x03,
+  IREE_UK_FLAG_PACK_TYPE_F16F16 = 0x04,
+  IREE_UK_FLAG_PACK_TYPE_BF16BF16 = 0x05,
+  IREE_UK_FLAG_PACK_TRANSPOSE_INNER = 0x100,
+  IREE_UK_FLAG_PACK_TRANSPOSE_OUTER = 0x200,
+};
+
+/* unpack type enum and bit flags (exported_bits.h:73-83). There is no 1-byte
+ * unpack type upstream (0x02 is reserved). */
+enum {
+  IREE_UK_FLAG_UNPACK_TYPE_MASK = 0xFF,
+  IREE_UK_FLAG_UNPACK_TYPE_NONE = 0x00,
+  IREE_UK_FLAG_UNPACK_TYPE_F32F32 = 0x01,
+  IREE_UK_FLAG_UNPACK_TYPE_I32I32 = 0x03,
+  IREE_UK_FLAG_UNPACK_TYPE_F16F16 = 0x04,
+  IREE_UK_FLAG_UNPACK_TYPE_BF16BF16 = 0x05,
+  IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER = 0x100,
+  IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER = 0x200,
+};
+
+/* query_tile_sizes flags (exported_bits.h:91-107). */
+enum {
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK = 0xFF,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_LHS = 0x01,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RHS = 0x02,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT = 0x03,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK = 0xFF00,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F32F32F32 = 0x0100,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32 = 0x0200,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32 = 0x0300,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F16 = 0x0400,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16F32 = 0x0500,
+  IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16BF16 = 0x0600,
+};
+
+/*===--------------------------------------------------------------------===*/
+/* Params structs. Field order equals the entry-point argument order.        */
+/*===--------------------------------------------------------------------===*/
+
+/* Replaces iree_uk_mmt4d_params_t (mmt4d_internal.h:14-32). */
+typedef struct iree_uk_mmt4d_params_t {
+  const void* lhs_buffer; /* [M][K][M0][K0], outer stride lhs_stride0 */
+  iree_uk_index_t lhs_offset;
+  iree_uk_index_t lhs_stride0;
+  const void* rhs_buffer; /* [N][K][N0][K0], outer stride rhs_stride0 */
+  iree_uk_index_t rhs_offset;
+  iree_uk_index_t rhs_stride0;
+  void* out_buffer; /* [M][N][M0][N0], outer stride out_stride0 */
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t M;
+  iree_uk_index_t N;
+  iree_uk_index_t K;
+  int32_t M0;
+  int32_t N0;
+  int32_t K0;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_mmt4d_params_t;
+
+/* Replaces iree_uk_pack_params_t (pack_internal.h:12-30). */
+typedef struct iree_uk_pack_params_t {
+  const void* in_buffer; /* 2-D, strides in_stride0 / in_stride1 */
+  iree_uk_index_t in_offset;
+  iree_uk_index_t in_stride0;
+  iree_uk_index_t in_stride1;
+  void* out_buffer; /* 4-D [out_size0][out_size1][out_size2][out_size3] */
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t out_stride1; /* must equal out_size2*out_size3 (pack.c:72) */
+  iree_uk_index_t in_size0;
+  iree_uk_index_t in_size1;
+  iree_uk_index_t out_size0;
+  iree_uk_index_t out_size1;
+  iree_uk_index_t out_size2;
+  iree_uk_index_t out_size3;
+  uint64_t padding_value; /* low elem_size bytes are used (pack.h:16-25) */
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_pack_params_t;
+
+/* Replaces iree_uk_unpack_params_t (unpack_internal.h:12-29). */
+typedef struct iree_uk_unpack_params_t {
+  const void* in_buffer; /* 4-D [in_size0][in_size1][in_size2][in_size3] */
+  iree_uk_index_t in_offset;
+  iree_uk_index_t in_stride0;
+  iree_uk_index_t in_stride1; /* must equal in_size2*in_size3 (unpack.c:49) */
+  void* out_buffer; /* 2-D, strides out_stride0 / out_stride1 */
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t out_stride1;
+  iree_uk_index_t in_size0;
+  iree_uk_index_t in_size1;
+  iree_uk_index_t in_size2;
+  iree_uk_index_t in_size3;
+  iree_uk_index_t out_size0;
+  iree_uk_index_t out_size1;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_unpack_params_t;
+
+/* Replaces iree_uk_query_tile_sizes_2d_params_t / _out_params_t
+ * (query_tile_sizes.h:16-26). */
+typedef struct iree_uk_query_tile_sizes_2d_params_t {
+  uint32_t flags;
+  iree_uk_index_t size0;
+  iree_uk_index_t size1;
+  const uint64_t* cpu_data;
+} iree_uk_query_tile_sizes_2d_params_t;
+
+typedef struct iree_uk_query_tile_sizes_2d_out_params_t {
+  iree_uk_index_t tile_size0;
+  iree_uk_index_t tile_size1;
+} iree_uk_query_tile_sizes_2d_out_params_t;
+
+/*===--------------------------------------------------------------------===*/
+/* Entry points.                                                             */
+/*===--------------------------------------------------------------------===*/
+
+/* Replaces iree_uk_mmt4d (mmt4d.h:14-21, mmt4d.c:152-178).
+ * For every i<M, j<N, i0<M0, j0<N0:
+ *   OUT[i][j][i0][j0] = (ACCUMULATE ? OUT[i][j][i0][j0] : 0)
+ *                     + sum_{k<K} sum_{k0<K0} LHS[i][k][i0][k0]*RHS[j][k][j0][k0]
+ * Returns without touching OUT when M==0, N==0, or K==0 with ACCUMULATE
+ * (mmt4d.c:106-114). Bytes of OUT outside the M0xN0 tiles are never written. */
+IREE_UK_AMD_EXPORT void iree_uk_mmt4d(
+    const void* lhs_buffer, iree_uk_index_t lhs_offset,
+    iree_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0, void* out_buffer,
+    iree_uk_index_t out_offset, iree_uk_index_t out_stride0, iree_uk_index_t M,
+    iree_uk_index_t N, iree_uk_index_t K, int32_t M0, int32_t N0, int32_t K0,
+    uint32_t flags, const uint64_t* cpu_data);
+
+/* Replaces iree_uk_mmt4d_p (mmt4d_internal.h:35, mmt4d.c:116-142). */
+IREE_UK_AMD_EXPORT void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params);
+
+/* Replaces iree_uk_mmt4d_info (mmt4d.h:25-27, mmt4d.c:180-186) and
+ * iree_uk_mmt4d_info_p (mmt4d_internal.h:40, mmt4d.c:144-150). */
+IREE_UK_AMD_EXPORT uint32_t iree_uk_mmt4d_info(int32_t M0, int32_t N0,
+                                               int32_t K0, uint32_t flags,
+                                               const uint64_t* cpu_data);
+IREE_UK_AMD_EXPORT uint32_t
+iree_uk_mmt4d_info_p(const iree_uk_mmt4d_params_t* params);
+
+/* Replaces iree_uk_pack (pack.h:26-34, pack.c:325-352). Writes every element
+ * of every output tile, using the low elem_size bytes of padding_value where
+ * the source index falls outside in_size0 x in_size1. */
+IREE_UK_AMD_EXPORT void iree_uk_pack(
+    const void* in_buffer, iree_uk_index_t in_offset,
+    iree_uk_index_t in_stride0, iree_uk_index_t in_stride1, void* out_buffer,
+    iree_uk_index_t out_offset, iree_uk_index_t out_stride0,
+    iree_uk_index_t out_stride1, iree_uk_index_t in_size0,
+    iree_uk_index_t in_size1, iree_uk_index_t out_size0,
+    iree_uk_index_t out_size1, iree_uk_index_t out_size2,
+    iree_uk_index_t out_size3, uint64_t padding_value, uint32_t flags,
+    const uint64_t* cpu_data);
+
+/* Replaces iree_uk_pack_p (pack_internal.h:32, pack.c:315-323). */
+IREE_UK_AMD_EXPORT void iree_uk_pack_p(const iree_uk_pack_params_t* params);
+
+/* Replaces iree_uk_unpack (unpack.h:17-25, unpack.c:259-285). Writes only
+ * elements inside out_size0 x out_size1. */
+IREE_UK_AMD_EXPORT void iree_uk_unpack(
+    const void* in_buffer, iree_uk_index_t in_offset,
+    iree_uk_index_t in_stride0, iree_uk_index_t in_stride1, void* out_buffer,
+    iree_uk_index_t out_offset, iree_uk_index_t out_stride0,
+    iree_uk_index_t out_stride1, iree_uk_index_t in_size0,
+    iree_uk_index_t in_size1, iree_uk_index_t in_size2,
+    iree_uk_index_t in_size3, iree_uk_index_t out_size0,
+    iree_uk_index_t out_size1, uint32_t flags, const uint64_t* cpu_data);
+
+/* Replaces iree_uk_unpack_p (unpack_internal.h:31, unpack.c:249-257). */
+IREE_UK_AMD_EXPORT void iree_uk_unpack_p(const iree_uk_unpack_params_t* params);
+
+/* Replaces iree_uk_query_tile_sizes_2d (query_tile_sizes.h:28-30,
+ * query_tile_sizes.c:65-75): returns the (M0,K0) / (N0,K0) / (M0,N0) tile for
+ * the operand role and matmul type in `flags`, chosen for the gfx950 MFMA
+ * kernels instead of a CPU ISA. */
+IREE_UK_AMD_EXPORT void iree_uk_query_tile_sizes_2d(
+    const iree_uk_query_tile_sizes_2d_params_t* params,
+    iree_uk_query_tile_sizes_2d_out_params_t* out_params);
+
+/*===--------------------------------------------------------------------===*/
+/* Contract-violation hook.                                                  */
+/*===--------------------------------------------------------------------===*/
+
+/* Replaces the embedder-provided iree_uk_assert_fail (common.h:307-308).
+ * The entry points return void; contract violations (unknown flags or types,
+ * negative sizes, out_stride1 != out_size2*out_size3, ...) are reported
+ * through this hook and the call then returns without doing any work.
+ * The default handler prints "file:line: function: assertion failed: cond"
+ * to stderr and aborts, like tools/util.c:21-31. */
+typedef void (*iree_uk_amd_assert_handler_t)(const char* file, int line,
+                                             const char* function,
+                                             const char* condition);
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_assert_handler(
+    iree_uk_amd_assert_handler_t handler); /* NULL restores the default */
+
+/*===--------------------------------------------------------------------===*/
+/* Device control: has no counterpart in the reference, whose ukernels run   */
+/* synchronously on the calling CPU thread.                                  */
+/*===--------------------------------------------------------------------===*/
+
+/* Status of the most recent entry-point call on this thread: 0 = OK, else a
+ * hipError_t value (launch or staging failure) or -1 (contract violation). */
+IREE_UK_AMD_EXPORT int iree_uk_amd_last_status(void);
+IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_status_string(void);
+
+/* Stream (a hipStream_t passed as void*) that this thread's calls enqueue on.
+ * NULL (the default) is the null stream. */
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_stream(void* hip_stream);
+IREE_UK_AMD_EXPORT void* iree_uk_amd_get_stream(void);
+
+/* Blocks until this thread's stream has drained. Returns 0 or a hipError_t. */
+IREE_UK_AMD_EXPORT int iree_uk_amd_synchronize(void);
+
+/* How buffer pointers are classified, per thread.
+ *   AUTO  : ask the HIP runtime about the first byte each operand touches;
+ *           host memory is staged through the GPU.
+ *   DEVICE: the caller promises device-accessible memory; no query is made
+ *           (saves ~1 us per operand on small problems). */
+enum {
+  IREE_UK_AMD_POINTER_MODE_AUTO = 0,
+  IREE_UK_AMD_POINTER_MODE_DEVICE = 1,
+};
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_pointer_mode(int mode);
+
+/* Kernel selection override for testing and benchmarking, per thread.
+ *   AUTO    : fastest kernel that serves the case.
+ *   GENERIC : always the scalar any-shape kernels. */
+enum {
+  IREE_UK_AMD_KERNEL_MODE_AUTO = 0,
+  IREE_UK_AMD_KERNEL_MODE_GENERIC = 1,
+};
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_kernel_mode(int mode);
+
+/* Name of the kernel variant the most recent call on this thread launched
+ * ("" if it returned early). Static storage; never NULL. */
+IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_kernel_name(void);
+
+/* Number of devices visible to HIP (0 when there is none or no driver). */
+IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);
+
+/* Library version, "major.minor". */
+IREE_UK_AMD_EXPORT const char* iree_uk_amd_version(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* IREE_UK_AMD_H_ */

@@ -1,0 +1,31 @@
+// mmt4d kernel selection: MFMA kernels where one covers (type, M0, N0, K0),
+// otherwise the any-shape scalar kernel.
+#include <hip/hip_runtime.h>
+
+#include "uk_hip_abi.h"
+
+extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
+    const iree_uk_mmt4d_params_t* p, void* stream);
+extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(
+    const iree_uk_mmt4d_params_t* p, void* stream, const char** kernel_name);
+extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
+                                                    int32_t K0, uint32_t flags);
+
+extern "C" int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0,
+                                                     int32_t K0,
+                                                     uint32_t flags) {
+  return iree_uk_amd_hip_mmt4d_mfma_supported(M0, N0, K0, flags);
+}
+
+extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
+                                            void* stream, int kernel_mode,
+                                            const char** kernel_name) {
+  if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC &&
+      iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) {
+    int st = iree_uk_amd_hip_launch_mmt4d_mfma(p, stream, kernel_name);
+    // A negative status means "shape not served after all"; fall through.
+    if (st >= 0) return st;
+  }
+  *kernel_name = "mmt4d_generic";
+  return iree_uk_amd_hip_launch_mmt4d_generic(p, stream);
+}

@@ -1,0 +1,682 @@
+// pack / unpack for gfx950: HBM-bound byte movement between a 2-D matrix and
+// its 4-D tiled form.
+//
+// Index algebra (runtime/src/iree/builtins/ukernel/tools/pack_test.c:13-71,
+// unpack_test.c:13-58): with (outer0, outer1, tile0, tile1) the stored 4-D
+// shape after undoing TRANSPOSE_OUTER / TRANSPOSE_INNER, matrix element
+// (a0*tile0 + b0, a1*tile1 + b1) lives at tiled offset
+//   a0*sl0 + a1*sl1 + b0*sl2 + b1*sl3.
+//
+// Two kernel families serve each op:
+//   *_generic : one thread per destination element, any shape/stride/type.
+//   *_tiled   : a workgroup stages a G0 x G1 block of tiles through LDS, held
+//               in LDS as the row-major 2-D matrix block. Global reads and
+//               writes are both contiguous runs of >= 256 bytes moved with up
+//               to 16-byte vectors; the tile regrouping (and the transposes)
+//               happens in the LDS addressing. Needs a unit inner stride on
+//               the 2-D side and 4-byte alignment on the tiled side.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <utility>
+
+#include "uk_device_common.h"
+#include "uk_hip_abi.h"
+
+namespace {
+
+using uk::FastDiv;
+
+constexpr int kThreads = 256;
+
+//===----------------------------------------------------------------------===//
+// Logical view shared by pack and unpack.
+//===----------------------------------------------------------------------===//
+
+struct TiledView {
+  int64_t outer0, outer1, tile0, tile1;  // after undoing the transposes
+  int64_t sl0, sl1, sl2, sl3;            // tiled-side strides, elements
+  int64_t size0, size1;                  // stored 4-D outer shape
+  int64_t size2, size3;                  // stored tile shape
+  int64_t stride0;                       // stored outer stride, elements
+};
+
+TiledView make_view(int64_t size0, int64_t size1, int64_t size2, int64_t size3,
+                    int64_t stride0, bool transpose_inner,
+                    bool transpose_outer) {
+  TiledView v;
+  v.size0 = size0; v.size1 = size1; v.size2 = size2; v.size3 = size3;
+  v.stride0 = stride0;
+  v.outer0 = size0; v.outer1 = size1; v.tile0 = size2; v.tile1 = size3;
+  v.sl0 = stride0; v.sl1 = size2 * size3; v.sl2 = size3; v.sl3 = 1;
+  if (transpose_outer) { std::swap(v.outer0, v.outer1); std::swap(v.sl0, v.sl1); }
+  if (transpose_inner) { std::swap(v.tile0, v.tile1); std::swap(v.sl2, v.sl3); }
+  return v;
+}
+
+//===----------------------------------------------------------------------===//
+// Generic kernels.
+//===----------------------------------------------------------------------===//
+
+struct GenericArgs {
+  const char* src;
+  char* dst;
+  int64_t mat_stride0, mat_stride1;  // 2-D side strides, elements
+  int64_t mat_size0, mat_size1;      // 2-D side sizes
+  int64_t tile0, tile1;
+  int64_t sl0, sl1, sl2, sl3;
+  int64_t size1, size2, size3, stride0;  // stored 4-D shape (size0 implied)
+  int64_t total;                         // number of destination elements
+  uint64_t pad;
+  int transpose_inner, transpose_outer;
+};
+
+// One thread per element of the tiled destination.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void pack_generic_kernel(GenericArgs a) {
+  const int64_t tile_elems = a.size2 * a.size3;
+  const int64_t row_elems = a.size1 * tile_elems;
+  for (int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x; idx < a.total;
+       idx += (int64_t)gridDim.x * kThreads) {
+    const int64_t o0 = idx / row_elems;
+    const int64_t rem = idx - o0 * row_elems;
+    const int64_t o1 = rem / tile_elems;
+    const int64_t t = rem - o1 * tile_elems;
+    const int64_t o2 = t / a.size3;
+    const int64_t o3 = t - o2 * a.size3;
+    const int64_t a0 = a.transpose_outer ? o1 : o0;
+    const int64_t a1 = a.transpose_outer ? o0 : o1;
+    const int64_t b0 = a.transpose_inner ? o3 : o2;
+    const int64_t b1 = a.transpose_inner ? o2 : o3;
+    const int64_t i0 = a0 * a.tile0 + b0;
+    const int64_t i1 = a1 * a.tile1 + b1;
+    T v;
+    if (i0 < a.mat_size0 && i1 < a.mat_size1) {
+      v = reinterpret_cast<const T*>(a.src)[i0 * a.mat_stride0 + i1 * a.mat_stride1];
+    } else {
+      v = (T)a.pad;
+    }
+    reinterpret_cast<T*>(a.dst)[o0 * a.stride0 + rem] = v;
+  }
+}
+
+// One thread per element of the 2-D destination.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void unpack_generic_kernel(GenericArgs a) {
+  for (int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x; idx < a.total;
+       idx += (int64_t)gridDim.x * kThreads) {
+    const int64_t i0 = idx / a.mat_size1;
+    const int64_t i1 = idx - i0 * a.mat_size1;
+    const int64_t a0 = i0 / a.tile0, b0 = i0 - a0 * a.tile0;
+    const int64_t a1 = i1 / a.tile1, b1 = i1 - a1 * a.tile1;
+    const T v = reinterpret_cast<const T*>(
+        a.src)[a0 * a.sl0 + a1 * a.sl1 + b0 * a.sl2 + b1 * a.sl3];
+    reinterpret_cast<T*>(a.dst)[i0 * a.mat_stride0 + i1 * a.mat_stride1] = v;
+  }
+}
+
+int grid_for(int64_t total) {
+  int64_t blocks = uk::ceil_div(total, kThreads);
+  const int64_t cap = 256 * 64;  // grid-stride beyond this
+  return (int)(blocks < cap ? blocks : cap);
+}
+
+//===----------------------------------------------------------------------===//
+// Tiled kernels.
+//===----------------------------------------------------------------------===//
+
+struct TiledArgs {
+  const char* src;
+  char* dst;
+  int64_t mat_stride0_bytes;        // 2-D side row pitch
+  int64_t sl0_bytes, sl1_bytes;     // tiled side: byte step of a0 / a1
+  uint32_t mat_size0, mat_size1;    // 2-D side sizes, elements
+  uint32_t outer0, outer1;          // tile counts (logical)
+  uint32_t tile0, tile1;            // logical tile shape, elements
+  uint32_t G0, G1;                  // tiles per block along each dim
+  uint32_t nblk1;                   // blocks along dim 1
+  uint32_t lds_pitch;               // bytes per LDS row
+  uint32_t lds_piece;               // largest aligned LDS access on a row, bytes
+  uint32_t elem_bytes;
+  uint32_t block_rows;              // G0*tile0
+  uint32_t block_row_bytes;         // G1*tile1*elem_bytes
+  uint32_t mat_vec;                 // 2-D side global vector width, bytes
+  uint32_t transpose_inner, transpose_outer;
+  uint32_t pad32;                   // padding element replicated to 32 bits
+  uint32_t tile_bytes;              // tile0*tile1*elem_bytes
+  uint32_t run_tiles;               // tiles per contiguous tiled-side run
+  uint32_t num_runs;                // runs per block
+  uint32_t run_vecs;                // tiled-side vectors per run
+  uint32_t tile_row_grans;          // granules per logical tile row (non-TI)
+  FastDiv div_row_vecs;             // 2-D side vectors per block row
+  FastDiv div_run_vecs;
+  FastDiv div_tile_grans;           // granules per tile
+  FastDiv div_tile_row_grans;
+  FastDiv div_tile0;
+};
+
+template <int N> struct Bytes;
+template <> struct Bytes<1> { using type = uint8_t; };
+template <> struct Bytes<2> { using type = uint16_t; };
+template <> struct Bytes<4> { using type = uint32_t; };
+template <> struct Bytes<8> { using type = uint2; };
+template <> struct Bytes<16> { using type = uint4; };
+
+template <int N>
+__device__ __forceinline__ void copy_bytes(void* dst, const void* src) {
+  using T = typename Bytes<N>::type;
+  *reinterpret_cast<T*>(dst) = *reinterpret_cast<const T*>(src);
+}
+
+// Copies n = VEC bytes between a register buffer and memory using accesses of
+// `piece` bytes (piece divides VEC, wave-uniform).
+template <int VEC>
+__device__ __forceinline__ void store_pieces(char* dst, const char* reg,
+                                             uint32_t piece) {
+  if (piece >= VEC) {
+    copy_bytes<VEC>(dst, reg);
+  } else if (VEC > 8 && piece == 8) {
+#pragma unroll
+    for (int i = 0; i < VEC; i += 8) copy_bytes<8>(dst + i, reg + i);
+  } else if (VEC > 4 && piece == 4) {
+#pragma unroll
+    for (int i = 0; i < VEC; i += 4) copy_bytes<4>(dst + i, reg + i);
+  } else if (VEC > 2 && piece == 2) {
+#pragma unroll
+    for (int i = 0; i < VEC; i += 2) copy_bytes<2>(dst + i, reg + i);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) dst[i] = reg[i];
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_pieces(char* reg, const char* src,
+                                            uint32_t piece) {
+  if (piece >= VEC) {
+    copy_bytes<VEC>(reg, src);
+  } else if (VEC > 8 && piece == 8) {
+#pragma unroll
+    for (int i = 0; i < VEC; i += 8) copy_bytes<8>(reg + i, src + i);
+  } else if (VEC > 4 && piece == 4) {
+#pragma unroll
+    for (int i = 0; i < VEC; i += 4) copy_bytes<4>(reg + i, src + i);
+  } else if (VEC > 2 && piece == 2) {
+#pragma unroll
+    for (int i = 0; i < VEC; i += 2) copy_bytes<2>(reg + i, src + i);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) reg[i] = src[i];
+  }
+}
+
+// LDS byte offset of the granule that starts at logical (tl0, tl1, b0, b1) of
+// the block held row-major in LDS.
+__device__ __forceinline__ uint32_t lds_offset(const TiledArgs& a, uint32_t tl0,
+                                               uint32_t tl1, uint32_t b0,
+                                               uint32_t b1) {
+  return (tl0 * a.tile0 + b0) * a.lds_pitch +
+         (tl1 * a.tile1 + b1) * a.elem_bytes;
+}
+
+// Walks the granules of one tiled-side vector. `pos` is the byte position of
+// the vector inside its run. Calls f(i, lds_byte_offset) for granule i.
+template <int G, int VEC, typename F>
+__device__ __forceinline__ void for_each_granule(const TiledArgs& a, uint32_t run,
+                                                 uint32_t t, uint32_t in_tile_byte,
+                                                 F f) {
+  const uint32_t tl0 = a.transpose_outer ? t : run;
+  const uint32_t tl1 = a.transpose_outer ? run : t;
+  uint32_t qg = in_tile_byte / G;  // granule index inside the tile
+  uint32_t b0, b1;
+  if (a.transpose_inner) {
+    // Stored tile is [b1][b0]; a granule is one element.
+    a.div_tile0.divmod(qg, b1, b0);
+  } else {
+    uint32_t b1g;
+    a.div_tile_row_grans.divmod(qg, b0, b1g);
+    b1 = b1g * (G / a.elem_bytes);
+  }
+#pragma unroll
+  for (int i = 0; i < VEC / G; ++i) {
+    f(i, lds_offset(a, tl0, tl1, b0, b1));
+    if (a.transpose_inner) {
+      if (++b0 == a.tile0) { b0 = 0; ++b1; }
+    } else {
+      b1 += G / a.elem_bytes;
+      if (b1 == a.tile1) { b1 = 0; ++b0; }
+    }
+  }
+}
+
+// pack: 2-D rows -> LDS (phase 1, contiguous), LDS -> tiled runs (phase 2,
+// gather by granules of G bytes into VEC-byte vectors).
+template <int G, int VEC>
+__global__ __launch_bounds__(kThreads) void pack_tiled_kernel(TiledArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const uint32_t blk0 = blockIdx.x / a.nblk1;
+  const uint32_t blk1 = blockIdx.x - blk0 * a.nblk1;
+  const uint32_t row_base = blk0 * a.block_rows;
+  const uint32_t col_base_bytes = blk1 * a.block_row_bytes;
+  const uint32_t es = a.elem_bytes;
+  const uint32_t size1_bytes = a.mat_size1 * es;
+
+  // Phase 1.
+  {
+    const uint32_t mv = a.mat_vec;
+    const uint32_t row_vecs = a.div_row_vecs.d;
+    const uint32_t total = a.block_rows * row_vecs;
+    const uint32_t piece = a.lds_piece < mv ? a.lds_piece : mv;
+    for (uint32_t idx = threadIdx.x; idx < total; idx += kThreads) {
+      uint32_t r, v;
+      a.div_row_vecs.divmod(idx, r, v);
+      const uint32_t grow = row_base + r;
+      const uint32_t cb = col_base_bytes + v * mv;  // byte column in the matrix
+      __attribute__((aligned(16))) char reg[16];
+      const bool row_ok = grow < a.mat_size0;
+      const char* gp = a.src + (int64_t)grow * a.mat_stride0_bytes + cb;
+      if (row_ok && cb + mv <= size1_bytes) {
+        switch (mv) {
+          case 16: copy_bytes<16>(reg, gp); break;
+          case 8: copy_bytes<8>(reg, gp); break;
+          case 4: copy_bytes<4>(reg, gp); break;
+          case 2: copy_bytes<2>(reg, gp); break;
+          default: reg[0] = gp[0]; break;
+        }
+      } else {
+        // Edge: element-wise, padding outside the matrix.
+        for (uint32_t b = 0; b < mv; b += es) {
+          const bool ok = row_ok && (cb + b) < size1_bytes;
+          if (es == 4) {
+            uint32_t w = ok ? *reinterpret_cast<const uint32_t*>(gp + b) : a.pad32;
+            *reinterpret_cast<uint32_t*>(reg + b) = w;
+          } else if (es == 2) {
+            uint16_t w = ok ? *reinterpret_cast<const uint16_t*>(gp + b)
+                            : (uint16_t)a.pad32;
+            *reinterpret_cast<uint16_t*>(reg + b) = w;
+          } else {
+            reg[b] = ok ? gp[b] : (char)a.pad32;
+          }
+        }
+      }
+      char* lp = lds + r * a.lds_pitch + v * mv;
+      switch (mv) {
+        case 16: store_pieces<16>(lp, reg, piece); break;
+        case 8: store_pieces<8>(lp, reg, piece); break;
+        case 4: store_pieces<4>(lp, reg, piece); break;
+        case 2: store_pieces<2>(lp, reg, piece); break;
+        default: lp[0] = reg[0]; break;
+      }
+    }
+  }
+  __syncthreads();
+
+  // Phase 2.
+  {
+    const uint32_t total = a.num_runs * a.run_vecs;
+    for (uint32_t idx = threadIdx.x; idx < total; idx += kThreads) {
+      uint32_t run, v;
+      a.div_run_vecs.divmod(idx, run, v);
+      const uint32_t pos = v * VEC;
+      const uint32_t t = pos / a.tile_bytes;  // tile inside the run
+      const uint32_t in_tile = pos - t * a.tile_bytes;
+      const uint32_t tl0 = a.transpose_outer ? t : run;
+      const uint32_t tl1 = a.transpose_outer ? run : t;
+      const uint32_t a0 = blk0 * a.G0 + tl0;
+      const uint32_t a1 = blk1 * a.G1 + tl1;
+      if (a0 >= a.outer0 || a1 >= a.outer1) continue;
+      __attribute__((aligned(16))) char reg[VEC];
+      for_each_granule<G, VEC>(a, run, t, in_tile, [&](int i, uint32_t off) {
+        copy_bytes<G>(reg + i * G, lds + off);
+      });
+      char* gp = a.dst + (int64_t)a0 * a.sl0_bytes + (int64_t)a1 * a.sl1_bytes + in_tile;
+      copy_bytes<VEC>(gp, reg);
+    }
+  }
+}
+
+// unpack: tiled runs -> LDS (phase 1, scatter by granules), LDS rows -> 2-D
+// rows (phase 2, contiguous, clipped to the matrix bounds).
+template <int G, int VEC>
+__global__ __launch_bounds__(kThreads) void unpack_tiled_kernel(TiledArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const uint32_t blk0 = blockIdx.x / a.nblk1;
+  const uint32_t blk1 = blockIdx.x - blk0 * a.nblk1;
+  const uint32_t row_base = blk0 * a.block_rows;
+  const uint32_t col_base_bytes = blk1 * a.block_row_bytes;
+  const uint32_t es = a.elem_bytes;
+  const uint32_t size1_bytes = a.mat_size1 * es;
+
+  // Phase 1.
+  {
+    const uint32_t total = a.num_runs * a.run_vecs;
+    for (uint32_t idx = threadIdx.x; idx < total; idx += kThreads) {
+      uint32_t run, v;
+      a.div_run_vecs.divmod(idx, run, v);
+      const uint32_t pos = v * VEC;
+      const uint32_t t = pos / a.tile_bytes;
+      const uint32_t in_tile = pos - t * a.tile_bytes;
+      const uint32_t tl0 = a.transpose_outer ? t : run;
+      const uint32_t tl1 = a.transpose_outer ? run : t;
+      const uint32_t a0 = blk0 * a.G0 + tl0;
+      const uint32_t a1 = blk1 * a.G1 + tl1;
+      if (a0 >= a.outer0 || a1 >= a.outer1) continue;
+      __attribute__((aligned(16))) char reg[VEC];
+      const char* gp =
+          a.src + (int64_t)a0 * a.sl0_bytes + (int64_t)a1 * a.sl1_bytes + in_tile;
+      copy_bytes<VEC>(reg, gp);
+      for_each_granule<G, VEC>(a, run, t, in_tile, [&](int i, uint32_t off) {
+        copy_bytes<G>(lds + off, reg + i * G);
+      });
+    }
+  }
+  __syncthreads();
+
+  // Phase 2.
+  {
+    const uint32_t mv = a.mat_vec;
+    const uint32_t row_vecs = a.div_row_vecs.d;
+    const uint32_t total = a.block_rows * row_vecs;
+    const uint32_t piece = a.lds_piece < mv ? a.lds_piece : mv;
+    for (uint32_t idx = threadIdx.x; idx < total; idx += kThreads) {
+      uint32_t r, v;
+      a.div_row_vecs.divmod(idx, r, v);
+      const uint32_t grow = row_base + r;
+      const uint32_t cb = col_base_bytes + v * mv;
+      if (grow >= a.mat_size0 || cb >= size1_bytes) continue;
+      __attribute__((aligned(16))) char reg[16];
+      const char* lp = lds + r * a.lds_pitch + v * mv;
+      switch (mv) {
+        case 16: load_pieces<16>(reg, lp, piece); break;
+        case 8: load_pieces<8>(reg, lp, piece); break;
+        case 4: load_pieces<4>(reg, lp, piece); break;
+        case 2: load_pieces<2>(reg, lp, piece); break;
+        default: reg[0] = lp[0]; break;
+      }
+      char* gp = a.dst + (int64_t)grow * a.mat_stride0_bytes + cb;
+      if (cb + mv <= size1_bytes) {
+        switch (mv) {
+          case 16: copy_bytes<16>(gp, reg); break;
+          case 8: copy_bytes<8>(gp, reg); break;
+          case 4: copy_bytes<4>(gp, reg); break;
+          case 2: copy_bytes<2>(gp, reg); break;
+          default: gp[0] = reg[0]; break;
+        }
+      } else {
+        for (uint32_t b = 0; b < mv && cb + b < size1_bytes; b += es) {
+          if (es == 4) copy_bytes<4>(gp + b, reg + b);
+          else if (es == 2) copy_bytes<2>(gp + b, reg + b);
+          else gp[b] = reg[b];
+        }
+      }
+    }
+  }
+}
+
+//===----------------------------------------------------------------------===//
+// Host-side planning.
+//===----------------------------------------------------------------------===//
+
+struct TiledPlan {
+  bool ok = false;
+  TiledArgs args;
+  int G = 0, VEC = 0;
+  uint32_t grid = 0;
+  uint32_t lds_bytes = 0;
+};
+
+// Chooses block shape, vector widths and LDS pitch. `mat` is the 2-D side
+// (source of pack, destination of unpack), `tiled` the 4-D side.
+TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
+                     int64_t mat_stride0, int64_t mat_stride1, int64_t mat_size0,
+                     int64_t mat_size1, const char* tiled_ptr, bool ti, bool to) {
+  TiledPlan plan;
+  if (mat_stride1 != 1) return plan;
+  const int64_t tile_elems = v.tile0 * v.tile1;
+  const int64_t tile_bytes = tile_elems * es;
+  if (tile_bytes == 0 || tile_bytes > 16384) return plan;
+  if (v.outer0 >= (1ll << 24) || v.outer1 >= (1ll << 24)) return plan;
+  if (mat_size0 >= (1ll << 31) || mat_size1 * es >= (1ll << 31)) return plan;
+  // Tiled-side vector width: alignment of base, outer stride and tile size.
+  const int64_t tiled_align = std::min(
+      {uk::pow2_divisor((int64_t)(uintptr_t)tiled_ptr, 16),
+       uk::pow2_divisor(v.stride0 * es, 16), uk::pow2_divisor(tile_bytes, 16)});
+  if (tiled_align < 4) return plan;
+  const int VEC = tiled_align >= 16 ? 16 : 4;
+  // Granule: bytes contiguous on both sides.
+  int G = ti ? es : (int)uk::pow2_divisor(v.tile1 * es, 16);
+  if (G > VEC) G = VEC;
+
+  // Block shape. A run is the contiguous tiled-side span of one block.
+  const int64_t kMinSpan = 256;    // bytes, both sides
+  const int64_t kTarget = 16384;   // LDS bytes per block, about
+  int64_t G0 = 1, G1 = uk::ceil_div(kMinSpan, v.tile1 * es);
+  if (to) {
+    G0 = uk::ceil_div(kMinSpan, tile_bytes);
+    // widen along dim 1 (more, longer 2-D row segments) up to the target
+    while (G0 * G1 * tile_bytes * 2 <= kTarget) G1 *= 2;
+  } else {
+    while (G0 * G1 * tile_bytes * 2 <= kTarget) G0 *= 2;
+  }
+  G0 = std::min<int64_t>(G0, std::max<int64_t>(v.outer0, 1));
+  G1 = std::min<int64_t>(G1, std::max<int64_t>(v.outer1, 1));
+  const int64_t block_rows = G0 * v.tile0;
+  const int64_t block_row_bytes = G1 * v.tile1 * es;
+
+  // LDS pitch: rows that consecutive lanes touch in the granule phase should
+  // start in different banks. Consecutive lanes sweep one tile row
+  // (tile1*es bytes) and then move one LDS row down, or move one row down per
+  // element when the inner transpose is on; so the pitch is made congruent to
+  // that sweep width modulo the 256-byte bank span.
+  int64_t sweep = ti ? es : v.tile1 * es;
+  if (sweep < 4) sweep = 4;
+  int64_t pitch = block_row_bytes;
+  if (sweep < 256) {
+    int64_t pad = ((sweep - block_row_bytes) % 256 + 256) % 256;
+    pitch = block_row_bytes + pad;
+  }
+  pitch = uk::ceil_div(pitch, G) * G;
+  const int64_t lds_bytes = block_rows * pitch;
+  if (lds_bytes > 64 * 1024) return plan;
+
+  // 2-D side vector width.
+  const int64_t mat_vec = std::min(
+      {uk::pow2_divisor((int64_t)(uintptr_t)mat_ptr, 16),
+       uk::pow2_divisor(mat_stride0 * es, 16),
+       uk::pow2_divisor(block_row_bytes, 16)});
+  if (mat_vec < es) return plan;
+
+  const int64_t nblk0 = uk::ceil_div(v.outer0, G0);
+  const int64_t nblk1 = uk::ceil_div(v.outer1, G1);
+  if (nblk0 * nblk1 >= (1ll << 31)) return plan;
+
+  TiledArgs& a = plan.args;
+  a.mat_stride0_bytes = mat_stride0 * es;
+  a.sl0_bytes = v.sl0 * es;
+  a.sl1_bytes = v.sl1 * es;
+  a.mat_size0 = (uint32_t)mat_size0;
+  a.mat_size1 = (uint32_t)mat_size1;
+  a.outer0 = (uint32_t)v.outer0;
+  a.outer1 = (uint32_t)v.outer1;
+  a.tile0 = (uint32_t)v.tile0;
+  a.tile1 = (uint32_t)v.tile1;
+  a.G0 = (uint32_t)G0;
+  a.G1 = (uint32_t)G1;
+  a.nblk1 = (uint32_t)nblk1;
+  a.lds_pitch = (uint32_t)pitch;
+  a.lds_piece = (uint32_t)uk::pow2_divisor(pitch, 16);
+  a.elem_bytes = (uint32_t)es;
+  a.block_rows = (uint32_t)block_rows;
+  a.block_row_bytes = (uint32_t)block_row_bytes;
+  a.mat_vec = (uint32_t)mat_vec;
+  a.transpose_inner = ti;
+  a.transpose_outer = to;
+  a.tile_bytes = (uint32_t)tile_bytes;
+  a.run_tiles = (uint32_t)(to ? G0 : G1);
+  a.num_runs = (uint32_t)(to ? G1 : G0);
+  a.run_vecs = (uint32_t)(a.run_tiles * tile_bytes / VEC);
+  a.tile_row_grans = ti ? 1 : (uint32_t)(v.tile1 * es / G);
+  a.div_row_vecs = FastDiv((uint32_t)(block_row_bytes / mat_vec));
+  a.div_run_vecs = FastDiv(a.run_vecs);
+  a.div_tile_grans = FastDiv((uint32_t)(tile_bytes / G));
+  a.div_tile_row_grans = FastDiv(a.tile_row_grans);
+  a.div_tile0 = FastDiv((uint32_t)v.tile0);
+  plan.G = G;
+  plan.VEC = VEC;
+  plan.grid = (uint32_t)(nblk0 * nblk1);
+  plan.lds_bytes = (uint32_t)lds_bytes;
+  plan.ok = true;
+  return plan;
+}
+
+template <template <int, int> class Launcher>
+bool dispatch_gv(int G, int VEC, const TiledPlan& plan, hipStream_t stream) {
+#define UK_CASE(g, vv)                              \
+  if (G == g && VEC == vv) {                        \
+    Launcher<g, vv>::launch(plan, stream);          \
+    return true;                                    \
+  }
+  UK_CASE(16, 16) UK_CASE(8, 16) UK_CASE(4, 16) UK_CASE(2, 16) UK_CASE(1, 16)
+  UK_CASE(4, 4) UK_CASE(2, 4) UK_CASE(1, 4)
+#undef UK_CASE
+  return false;
+}
+
+template <int G, int VEC>
+struct PackLauncher {
+  static void launch(const TiledPlan& plan, hipStream_t stream) {
+    hipLaunchKernelGGL((pack_tiled_kernel<G, VEC>), dim3(plan.grid),
+                       dim3(kThreads), plan.lds_bytes, stream, plan.args);
+  }
+};
+
+template <int G, int VEC>
+struct UnpackLauncher {
+  static void launch(const TiledPlan& plan, hipStream_t stream) {
+    hipLaunchKernelGGL((unpack_tiled_kernel<G, VEC>), dim3(plan.grid),
+                       dim3(kThreads), plan.lds_bytes, stream, plan.args);
+  }
+};
+
+uint32_t replicate_pad(uint64_t pad, int es) {
+  if (es == 1) return (uint32_t)(pad & 0xFF) * 0x01010101u;
+  if (es == 2) return (uint32_t)(pad & 0xFFFF) * 0x00010001u;
+  return (uint32_t)pad;
+}
+
+int elem_bytes_of(uint32_t flags) {
+  switch (flags & 0xFF) {
+    case IREE_UK_FLAG_PACK_TYPE_F32F32: return 4;
+    case IREE_UK_FLAG_PACK_TYPE_I8I8: return 1;
+    case IREE_UK_FLAG_PACK_TYPE_I32I32: return 4;
+    case IREE_UK_FLAG_PACK_TYPE_F16F16: return 2;
+    case IREE_UK_FLAG_PACK_TYPE_BF16BF16: return 2;
+    default: return 0;
+  }
+}
+
+}  // namespace
+
+extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
+                                           void* stream_v, int kernel_mode,
+                                           const char** kernel_name) {
+  hipStream_t stream = (hipStream_t)stream_v;
+  const int es = elem_bytes_of(p->flags);
+  if (!es) return (int)hipErrorInvalidValue;
+  const bool ti = p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
+  const bool to = p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_OUTER;
+  const TiledView v = make_view(p->out_size0, p->out_size1, p->out_size2,
+                                p->out_size3, p->out_stride0, ti, to);
+  const char* src = (const char*)p->in_buffer + p->in_offset * es;
+  char* dst = (char*)p->out_buffer + p->out_offset * es;
+
+  if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC) {
+    TiledPlan plan = plan_tiled(v, es, src, p->in_stride0, p->in_stride1,
+                                p->in_size0, p->in_size1, dst, ti, to);
+    if (plan.ok) {
+      plan.args.src = src;
+      plan.args.dst = dst;
+      plan.args.pad32 = replicate_pad(p->padding_value, es);
+      if (dispatch_gv<PackLauncher>(plan.G, plan.VEC, plan, stream)) {
+        *kernel_name = "pack_tiled";
+        return (int)hipGetLastError();
+      }
+    }
+  }
+
+  GenericArgs a;
+  a.src = src;
+  a.dst = dst;
+  a.mat_stride0 = p->in_stride0;
+  a.mat_stride1 = p->in_stride1;
+  a.mat_size0 = p->in_size0;
+  a.mat_size1 = p->in_size1;
+  a.tile0 = v.tile0; a.tile1 = v.tile1;
+  a.sl0 = v.sl0; a.sl1 = v.sl1; a.sl2 = v.sl2; a.sl3 = v.sl3;
+  a.size1 = p->out_size1; a.size2 = p->out_size2; a.size3 = p->out_size3;
+  a.stride0 = p->out_stride0;
+  a.total = p->out_size0 * p->out_size1 * p->out_size2 * p->out_size3;
+  a.pad = p->padding_value;
+  a.transpose_inner = ti;
+  a.transpose_outer = to;
+  const int grid = grid_for(a.total);
+  switch (es) {
+    case 1: hipLaunchKernelGGL(pack_generic_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    case 2: hipLaunchKernelGGL(pack_generic_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    default: hipLaunchKernelGGL(pack_generic_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+  }
+  *kernel_name = "pack_generic";
+  return (int)hipGetLastError();
+}
+
+extern "C" int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* p,
+                                             void* stream_v, int kernel_mode,
+                                             const char** kernel_name) {
+  hipStream_t stream = (hipStream_t)stream_v;
+  const int es = elem_bytes_of(p->flags);
+  if (!es) return (int)hipErrorInvalidValue;
+  const bool ti = p->flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER;
+  const bool to = p->flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER;
+  const TiledView v = make_view(p->in_size0, p->in_size1, p->in_size2,
+                                p->in_size3, p->in_stride0, ti, to);
+  const char* src = (const char*)p->in_buffer + p->in_offset * es;
+  char* dst = (char*)p->out_buffer + p->out_offset * es;
+
+  if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC) {
+    TiledPlan plan = plan_tiled(v, es, dst, p->out_stride0, p->out_stride1,
+                                p->out_size0, p->out_size1, src, ti, to);
+    if (plan.ok) {
+      plan.args.src = src;
+      plan.args.dst = dst;
+      plan.args.pad32 = 0;
+      if (dispatch_gv<UnpackLauncher>(plan.G, plan.VEC, plan, stream)) {
+        *kernel_name = "unpack_tiled";
+        return (int)hipGetLastError();
+      }
+    }
+  }
+
+  GenericArgs a;
+  a.src = src;
+  a.dst = dst;
+  a.mat_stride0 = p->out_stride0;
+  a.mat_stride1 = p->out_stride1;
+  a.mat_size0 = p->out_size0;
+  a.mat_size1 = p->out_size1;
+  a.tile0 = v.tile0; a.tile1 = v.tile1;
+  a.sl0 = v.sl0; a.sl1 = v.sl1; a.sl2 = v.sl2; a.sl3 = v.sl3;
+  a.size1 = p->in_size1; a.size2 = p->in_size2; a.size3 = p->in_size3;
+  a.stride0 = p->in_stride0;
+  a.total = p->out_size0 * p->out_size1;
+  a.pad = 0;
+  a.transpose_inner = ti;
+  a.transpose_outer = to;
+  const int grid = grid_for(a.total);
+  switch (es) {
+    case 2: hipLaunchKernelGGL(unpack_generic_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    case 1: hipLaunchKernelGGL(unpack_generic_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    default: hipLaunchKernelGGL(unpack_generic_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+  }
+  *kernel_name = "unpack_generic";
+  return (int)hipGetLastError();
+}

@@ -1,0 +1,59 @@
+/*
+ * Internal C-ABI between the plain-C host layer (uk_host.c) and the HIP
+ * translation units. Everything the host layer needs from HIP goes through
+ * these functions: kernel launchers and a handful of runtime wrappers. No HIP
+ * type appears here, so the host layer compiles with any C compiler.
+ *
+ * Every function returns 0 on success or a hipError_t value.
+ */
+#ifndef IREE_UK_AMD_HIP_ABI_H_
+#define IREE_UK_AMD_HIP_ABI_H_
+
+#include "iree_uk_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Launchers. `params` has been validated and is not an early-return case; its
+ * buffer pointers are device-accessible. `stream` is a hipStream_t.
+ * `kernel_mode` is an IREE_UK_AMD_KERNEL_MODE_* value. `*kernel_name` receives
+ * a static string naming the variant that was launched. */
+int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* params,
+                                void* stream, int kernel_mode,
+                                const char** kernel_name);
+int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* params,
+                                  void* stream, int kernel_mode,
+                                  const char** kernel_name);
+int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* params,
+                                 void* stream, int kernel_mode,
+                                 const char** kernel_name);
+
+/* 1 when an MFMA kernel serves (M0,N0,K0,type) regardless of M,N,K. */
+int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0, int32_t K0,
+                                          uint32_t flags);
+
+/* Runtime wrappers. */
+int iree_uk_amd_hip_device_count(void);
+/* *is_device = 1 if `ptr` is device-accessible memory known to HIP (device,
+ * managed, or registered/pinned host memory), 0 for ordinary host memory. */
+int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device);
+int iree_uk_amd_hip_malloc(void** ptr, int64_t bytes);
+int iree_uk_amd_hip_free(void* ptr);
+/* 2-D copies of `height` rows of `width` bytes; pitches in bytes. Synchronous
+ * with respect to the host; ordered after prior work on `stream`. */
+int iree_uk_amd_hip_copy2d_to_device(void* dst, int64_t dst_pitch,
+                                     const void* src, int64_t src_pitch,
+                                     int64_t width, int64_t height,
+                                     void* stream);
+int iree_uk_amd_hip_copy2d_to_host(void* dst, int64_t dst_pitch,
+                                   const void* src, int64_t src_pitch,
+                                   int64_t width, int64_t height, void* stream);
+int iree_uk_amd_hip_stream_synchronize(void* stream);
+const char* iree_uk_amd_hip_error_string(int status);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* IREE_UK_AMD_HIP_ABI_H_ */

@@ -1,0 +1,84 @@
+// Thin C-ABI wrappers over the HIP runtime for the plain-C host layer.
+#include <hip/hip_runtime.h>
+
+#include "uk_hip_abi.h"
+
+extern "C" {
+
+int iree_uk_amd_hip_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device) {
+  hipPointerAttribute_t attr;
+  hipError_t err = hipPointerGetAttributes(&attr, ptr);
+  if (err != hipSuccess) {
+    // Memory HIP has never seen is ordinary host memory; the runtime reports
+    // it as an invalid value. Clear the sticky error.
+    (void)hipGetLastError();
+    *is_device = 0;
+    return 0;
+  }
+  switch (attr.type) {
+    case hipMemoryTypeDevice:
+    case hipMemoryTypeManaged:
+    case hipMemoryTypeArray:
+      *is_device = 1;
+      break;
+    case hipMemoryTypeHost:
+      // Pinned host memory is device-accessible through its device alias.
+      *is_device = attr.devicePointer != nullptr;
+      break;
+    default:  // hipMemoryTypeUnregistered
+      *is_device = 0;
+      break;
+  }
+  return 0;
+}
+
+int iree_uk_amd_hip_malloc(void** ptr, int64_t bytes) {
+  return (int)hipMalloc(ptr, (size_t)bytes);
+}
+
+int iree_uk_amd_hip_free(void* ptr) { return (int)hipFree(ptr); }
+
+int iree_uk_amd_hip_copy2d_to_device(void* dst, int64_t dst_pitch,
+                                     const void* src, int64_t src_pitch,
+                                     int64_t width, int64_t height,
+                                     void* stream) {
+  hipError_t err =
+      hipMemcpy2DAsync(dst, (size_t)dst_pitch, src, (size_t)src_pitch,
+                       (size_t)width, (size_t)height, hipMemcpyHostToDevice,
+                       (hipStream_t)stream);
+  if (err != hipSuccess) return (int)err;
+  // Pageable host memory: the caller may reuse or free `src` right after the
+  // entry point returns, so wait for the copy.
+  return (int)hipStreamSynchronize((hipStream_t)stream);
+}
+
+int iree_uk_amd_hip_copy2d_to_host(void* dst, int64_t dst_pitch,
+                                   const void* src, int64_t src_pitch,
+                                   int64_t width, int64_t height,
+                                   void* stream) {
+  hipError_t err =
+      hipMemcpy2DAsync(dst, (size_t)dst_pitch, src, (size_t)src_pitch,
+                       (size_t)width, (size_t)height, hipMemcpyDeviceToHost,
+                       (hipStream_t)stream);
+  if (err != hipSuccess) return (int)err;
+  return (int)hipStreamSynchronize((hipStream_t)stream);
+}
+
+int iree_uk_amd_hip_stream_synchronize(void* stream) {
+  return (int)hipStreamSynchronize((hipStream_t)stream);
+}
+
+const char* iree_uk_amd_hip_error_string(int status) {
+  return hipGetErrorString((hipError_t)status);
+}
+
+}  // extern "C"

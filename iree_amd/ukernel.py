@@ -1,0 +1,217 @@
+"""ctypes binding of libiree_uk_amd.so: the gfx950 pack / mmt4d / unpack ukernels.
+
+The functions keep the names, positional argument order and meaning of the
+reference C entry points (runtime/src/iree/builtins/ukernel/mmt4d.h:14-21,
+pack.h:26-34, unpack.h:17-25); buffers are passed as integer addresses
+(``tensor.data_ptr()`` of a device tensor, or a host address), offsets and
+strides in elements.
+
+There is no fallback: if the shared library has not been built, importing the
+binding raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libiree_uk_amd.so")
+
+# --- flag values (runtime/src/iree/builtins/ukernel/exported_bits.h:29-83) ---
+MMT4D_TYPE_F32F32F32 = 0x01
+MMT4D_TYPE_S8S8S32 = 0x02
+MMT4D_TYPE_F16F16F32 = 0x03
+MMT4D_TYPE_F16F16F16 = 0x04
+MMT4D_TYPE_BF16BF16F32 = 0x05
+MMT4D_TYPE_BF16BF16BF16 = 0x06
+MMT4D_TYPE_S16S16S32 = 0x07
+MMT4D_TYPE_S16U4S32 = 0x08
+MMT4D_TYPE_S16S8S32 = 0x09
+MMT4D_TYPE_S8S4S32 = 0x0A
+MMT4D_TYPE_F8E4M3FNF8E4M3FNF32 = 0x80  # extension of this library
+MMT4D_ACCUMULATE = 0x100
+MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION = 0x200
+MMT4D_SKIP_INTERMEDIATE_ROUNDINGS = 0x400
+MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION = 0x1
+
+PACK_TYPE_F32F32 = 0x01
+PACK_TYPE_I8I8 = 0x02
+PACK_TYPE_I32I32 = 0x03
+PACK_TYPE_F16F16 = 0x04
+PACK_TYPE_BF16BF16 = 0x05
+PACK_TRANSPOSE_INNER = 0x100
+PACK_TRANSPOSE_OUTER = 0x200
+
+UNPACK_TYPE_F32F32 = 0x01
+UNPACK_TYPE_I32I32 = 0x03
+UNPACK_TYPE_F16F16 = 0x04
+UNPACK_TYPE_BF16BF16 = 0x05
+UNPACK_TRANSPOSE_INNER = 0x100
+UNPACK_TRANSPOSE_OUTER = 0x200
+
+POINTER_MODE_AUTO = 0
+POINTER_MODE_DEVICE = 1
+KERNEL_MODE_AUTO = 0
+KERNEL_MODE_GENERIC = 1
+
+# (lhs bits, rhs bits, out bits) per mmt4d type value.
+MMT4D_TYPE_BITS = {
+    MMT4D_TYPE_F32F32F32: (32, 32, 32),
+    MMT4D_TYPE_S8S8S32: (8, 8, 32),
+    MMT4D_TYPE_F16F16F32: (16, 16, 32),
+    MMT4D_TYPE_F16F16F16: (16, 16, 16),
+    MMT4D_TYPE_BF16BF16F32: (16, 16, 32),
+    MMT4D_TYPE_BF16BF16BF16: (16, 16, 16),
+    MMT4D_TYPE_S16S16S32: (16, 16, 32),
+    MMT4D_TYPE_S16U4S32: (16, 4, 32),
+    MMT4D_TYPE_S16S8S32: (16, 8, 32),
+    MMT4D_TYPE_S8S4S32: (8, 4, 32),
+    MMT4D_TYPE_F8E4M3FNF8E4M3FNF32: (8, 8, 32),
+}
+PACK_TYPE_BYTES = {PACK_TYPE_F32F32: 4, PACK_TYPE_I8I8: 1, PACK_TYPE_I32I32: 4,
+                   PACK_TYPE_F16F16: 2, PACK_TYPE_BF16BF16: 2}
+
+_i64 = ctypes.c_int64
+_i32 = ctypes.c_int32
+_u32 = ctypes.c_uint32
+_u64 = ctypes.c_uint64
+_vp = ctypes.c_void_p
+
+ASSERT_HANDLER = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_int,
+                                  ctypes.c_char_p, ctypes.c_char_p)
+
+
+class ContractViolation(RuntimeError):
+    """Raised by the Python-side assert handler (see raise_on_violation)."""
+
+
+class UKernelLibrary:
+    """The loaded shared library with typed entry points."""
+
+    def __init__(self, path: str = LIB_PATH):
+        if not os.path.exists(path):
+            raise ImportError(
+                f"{path} is missing: build it with `python -m iree_amd.build` "
+                "(there is no CPU or PyTorch fallback for these kernels)")
+        self.path = path
+        self.lib = ctypes.CDLL(path)
+        L = self.lib
+        L.iree_uk_mmt4d.argtypes = [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64,
+                                    _i64, _i64, _i64, _i64, _i32, _i32, _i32,
+                                    _u32, _vp]
+        L.iree_uk_mmt4d.restype = None
+        L.iree_uk_mmt4d_info.argtypes = [_i32, _i32, _i32, _u32, _vp]
+        L.iree_uk_mmt4d_info.restype = _u32
+        L.iree_uk_pack.argtypes = [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
+                                   _i64, _i64, _i64, _i64, _i64, _i64, _u64,
+                                   _u32, _vp]
+        L.iree_uk_pack.restype = None
+        L.iree_uk_unpack.argtypes = [_vp, _i64, _i64, _i64, _vp, _i64, _i64,
+                                     _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                     _u32, _vp]
+        L.iree_uk_unpack.restype = None
+        L.iree_uk_amd_last_status.restype = ctypes.c_int
+        L.iree_uk_amd_last_status_string.restype = ctypes.c_char_p
+        L.iree_uk_amd_last_kernel_name.restype = ctypes.c_char_p
+        L.iree_uk_amd_set_stream.argtypes = [_vp]
+        L.iree_uk_amd_get_stream.restype = _vp
+        L.iree_uk_amd_synchronize.restype = ctypes.c_int
+        L.iree_uk_amd_set_pointer_mode.argtypes = [ctypes.c_int]
+        L.iree_uk_amd_set_kernel_mode.argtypes = [ctypes.c_int]
+        L.iree_uk_amd_device_count.restype = ctypes.c_int
+        L.iree_uk_amd_version.restype = ctypes.c_char_p
+        L.iree_uk_amd_set_assert_handler.argtypes = [_vp]
+        self._handler_ref = None
+        self._violations: list[str] = []
+
+    # ----------------------------------------------------------------- entry
+    def mmt4d(self, lhs, lhs_offset, lhs_stride0, rhs, rhs_offset, rhs_stride0,
+              out, out_offset, out_stride0, M, N, K, M0, N0, K0, flags,
+              cpu_data=None):
+        self.lib.iree_uk_mmt4d(lhs, lhs_offset, lhs_stride0, rhs, rhs_offset,
+                               rhs_stride0, out, out_offset, out_stride0, M, N,
+                               K, M0, N0, K0, flags, cpu_data)
+        self._check()
+
+    def mmt4d_info(self, M0, N0, K0, flags, cpu_data=None) -> int:
+        return int(self.lib.iree_uk_mmt4d_info(M0, N0, K0, flags, cpu_data))
+
+    def pack(self, inp, in_offset, in_stride0, in_stride1, out, out_offset,
+             out_stride0, out_stride1, in_size0, in_size1, out_size0, out_size1,
+             out_size2, out_size3, padding_value, flags, cpu_data=None):
+        self.lib.iree_uk_pack(inp, in_offset, in_stride0, in_stride1, out,
+                              out_offset, out_stride0, out_stride1, in_size0,
+                              in_size1, out_size0, out_size1, out_size2,
+                              out_size3, padding_value, flags, cpu_data)
+        self._check()
+
+    def unpack(self, inp, in_offset, in_stride0, in_stride1, out, out_offset,
+               out_stride0, out_stride1, in_size0, in_size1, in_size2, in_size3,
+               out_size0, out_size1, flags, cpu_data=None):
+        self.lib.iree_uk_unpack(inp, in_offset, in_stride0, in_stride1, out,
+                                out_offset, out_stride0, out_stride1, in_size0,
+                                in_size1, in_size2, in_size3, out_size0,
+                                out_size1, flags, cpu_data)
+        self._check()
+
+    # --------------------------------------------------------------- control
+    def _check(self):
+        if self._violations:
+            msg = "; ".join(self._violations)
+            self._violations.clear()
+            raise ContractViolation(msg)
+        st = self.lib.iree_uk_amd_last_status()
+        if st not in (0,):
+            raise RuntimeError(
+                f"iree_uk_amd: status {st}: "
+                f"{self.lib.iree_uk_amd_last_status_string().decode()}")
+
+    def raise_on_violation(self, enable: bool = True):
+        """Routes contract violations to ContractViolation instead of the
+        default print-and-abort handler."""
+        if not enable:
+            self.lib.iree_uk_amd_set_assert_handler(None)
+            self._handler_ref = None
+            return
+
+        def handler(file, line, function, condition):
+            self._violations.append(
+                f"{function.decode()}: assertion failed: {condition.decode()}")
+
+        self._handler_ref = ASSERT_HANDLER(handler)
+        self.lib.iree_uk_amd_set_assert_handler(
+            ctypes.cast(self._handler_ref, _vp))
+
+    def set_stream(self, hip_stream: int | None):
+        self.lib.iree_uk_amd_set_stream(hip_stream)
+
+    def synchronize(self):
+        st = self.lib.iree_uk_amd_synchronize()
+        if st:
+            raise RuntimeError(f"iree_uk_amd_synchronize: status {st}")
+
+    def set_pointer_mode(self, mode: int):
+        self.lib.iree_uk_amd_set_pointer_mode(mode)
+
+    def set_kernel_mode(self, mode: int):
+        self.lib.iree_uk_amd_set_kernel_mode(mode)
+
+    def last_kernel_name(self) -> str:
+        return self.lib.iree_uk_amd_last_kernel_name().decode()
+
+    def device_count(self) -> int:
+        return int(self.lib.iree_uk_amd_device_count())
+
+    def version(self) -> str:
+        return self.lib.iree_uk_amd_version().decode()
+
+
+_lib: UKernelLibrary | None = None
+
+
+def load() -> UKernelLibrary:
+    """Loads the library once per process; raises ImportError if it is not built."""
+    global _lib
+    if _lib is None:
+        _lib = UKernelLibrary()
+    return _lib

@@ -1,0 +1,147 @@
+"""GPU parity of iree_uk_mmt4d against the CPU oracle, through the C-ABI.
+Integer types: bit-exact. Float types: bit-exact on the small-integer inputs
+of the reference's own tests (every partial sum is exact, so the summation
+order does not matter), and within the stated tolerance on N(0,1) inputs:
+max|gpu-ref| / max|ref| <= 1e-2 for f16/bf16 and <= 2e-2 for f8, against the
+f32-accumulating oracle."""
+import numpy as np
+import pytest
+
+import uk_testing as T
+from golden import make_golden as G
+from iree_amd import ukernel as uk
+
+pytestmark = pytest.mark.gpu
+
+TOL = {uk.MMT4D_TYPE_F16F16F32: 1e-2, uk.MMT4D_TYPE_BF16BF16F32: 1e-2,
+       uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32: 2e-2, uk.MMT4D_TYPE_F32F32F32: 1e-5}
+
+
+@pytest.fixture(autouse=True)
+def _reset_modes(lib):
+    yield
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lib.set_pointer_mode(uk.POINTER_MODE_AUTO)
+
+
+@pytest.mark.parametrize("mode", [uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_GENERIC])
+@pytest.mark.parametrize("n", range(len(G.MMT4D_TILES)))
+def test_mmt4d_reference_test_grid(gpu, oracle, n, mode):
+    """tools/mmt4d_test.c's grid: every type triple, odd tile shapes,
+    degenerate M/N/K, ACCUMULATE on/off, loose strides, non-zero offsets;
+    memcmp over the whole output buffer."""
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    tf, M0, N0, K0, extra = G.MMT4D_TILES[n]
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=13000 + n, extra_flags=extra)):
+        rng = np.random.default_rng(ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+
+
+# (type, M0, N0, K0) served by the MFMA kernels, with tile-count shapes that
+# cover: single tile, ragged against the workgroup tile in M and N, K both
+# below and above one pipeline step, and a several-workgroup case.
+MFMA_TILES = [
+    (uk.MMT4D_TYPE_S8S8S32, 16, 16, 2), (uk.MMT4D_TYPE_S8S8S32, 32, 16, 8),
+    (uk.MMT4D_TYPE_S8S8S32, 16, 16, 16), (uk.MMT4D_TYPE_S8S8S32, 16, 16, 64),
+    (uk.MMT4D_TYPE_S8S8S32, 16, 16, 4), (uk.MMT4D_TYPE_S8S8S32, 16, 16, 8),
+    (uk.MMT4D_TYPE_S8S8S32, 16, 16, 32), (uk.MMT4D_TYPE_S8S8S32, 8, 8, 2),
+    (uk.MMT4D_TYPE_S8S8S32, 8, 32, 4), (uk.MMT4D_TYPE_S8S8S32, 64, 16, 1),
+    (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16), (uk.MMT4D_TYPE_F16F16F32, 16, 16, 1),
+    (uk.MMT4D_TYPE_F16F16F32, 16, 16, 8), (uk.MMT4D_TYPE_F16F16F32, 8, 16, 4),
+    (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 2), (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
+    (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 32),
+    (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
+    (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 16),
+    (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 128),
+]
+
+
+def _mfma_shapes(M0, N0, K0, bits):
+    kb = K0 * bits // 8  # bytes of K per tile row
+    k_small = max(1, 32 // kb)
+    k_big = max(3, 700 // kb)
+    m_wg = max(1, 256 // M0)
+    n_wg = max(1, 256 // N0)
+    return ((1, 1, 1), (1, 1, k_small), (2, 3, k_big), (m_wg + 1, 1, k_small + 1),
+            (1, n_wg + 3, 5), (m_wg + 2, n_wg + 1, k_big // 2 + 1), (0, 2, 2),
+            (2, 2, 0))
+
+
+@pytest.mark.parametrize("n", range(len(MFMA_TILES)))
+def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n):
+    lib, torch = gpu
+    tf, M0, N0, K0 = MFMA_TILES[n]
+    if not lib.mmt4d_info(M0, N0, K0, tf):
+        pytest.skip("no MFMA kernel for this tile shape; covered by the generic kernel")
+    bits = uk.MMT4D_TYPE_BITS[tf][0]
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=14000 + n,
+                                         shapes=_mfma_shapes(M0, N0, K0, bits))):
+        rng = np.random.default_rng(ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        # No generic-fallback flag: only an MFMA kernel may serve these calls.
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        if c.M and c.N and not (c.K == 0 and c.flags & uk.MMT4D_ACCUMULATE):
+            assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
+
+
+def _normal_operand(rng, kind, n, scale=1.0):
+    x = (rng.standard_normal(n) * scale).astype(np.float32)
+    if kind == "f16":
+        return x.astype(np.float16).view(np.uint16)
+    if kind == "bf16":
+        return T.f32_to_bf16_bits(x)
+    if kind == "f8":
+        x = x * (448.0 / np.abs(x).max())
+        return T.f32_to_f8e4m3fn_bits(x)
+    return x
+
+
+@pytest.mark.parametrize("tf,M0,N0,K0", [
+    (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16), (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 2),
+    (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
+    (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
+    (uk.MMT4D_TYPE_F32F32F32, 8, 8, 4)])
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_mmt4d_float_tolerance_on_normal_inputs(gpu, oracle, tf, M0, N0, K0, accumulate):
+    lib, torch = gpu
+    lk = T.MMT4D_KINDS[tf][0]
+    rng = np.random.default_rng(21)
+    M, N, K = 9, 11, max(1, 2048 // K0)
+    lhs = _normal_operand(rng, lk, M * K * M0 * K0)
+    rhs = _normal_operand(rng, lk, N * K * N0 * K0)
+    out0 = rng.standard_normal(M * N * M0 * N0).astype(np.float32) * 10
+    flags = tf | 0x200 | (uk.MMT4D_ACCUMULATE if accumulate else 0)
+    want = out0.copy()
+    oracle.mmt4d(lhs, 0, K * M0 * K0, rhs, 0, K * N0 * K0, want, 0, N * M0 * N0,
+                 M, N, K, M0, N0, K0, flags)
+    d = [T.DeviceBytes(torch, a) for a in (lhs, rhs, out0)]
+    lib.mmt4d(d[0].ptr, 0, K * M0 * K0, d[1].ptr, 0, K * N0 * K0, d[2].ptr, 0,
+              N * M0 * N0, M, N, K, M0, N0, K0, flags)
+    lib.synchronize()
+    got = d[2].numpy().view(np.float32)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err <= TOL[tf], (err, lib.last_kernel_name())
+
+
+def test_mmt4d_host_pointers_are_staged(gpu, oracle):
+    lib, torch = gpu
+    for ci, c in enumerate(T.mmt4d_cases(uk.MMT4D_TYPE_S8S8S32, 16, 16, 2, seed=41,
+                                         shapes=((2, 3, 5), (1, 1, 0), (5, 7, 13)))):
+        rng = np.random.default_rng(ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = out0.copy()
+        lib.mmt4d(lhs.ctypes.data - c.lhs_offset, c.lhs_offset, c.lhs_stride0,
+                  rhs.ctypes.data - c.rhs_offset, c.rhs_offset, c.rhs_stride0,
+                  got.ctypes.data - c.out_offset * 4, c.out_offset, c.out_stride0,
+                  c.M, c.N, c.K, c.M0, c.N0, c.K0, c.flags | 0x200)
+        assert np.array_equal(got, want), c.label()

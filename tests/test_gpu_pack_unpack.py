@@ -1,0 +1,192 @@
+"""GPU parity of iree_uk_pack / iree_uk_unpack against the CPU oracle, through
+the C-ABI. Bit-exact over the whole destination buffer (stride gaps must stay
+untouched)."""
+import numpy as np
+import pytest
+
+import uk_testing as T
+from golden import make_golden as G
+from iree_amd import ukernel as uk
+
+pytestmark = pytest.mark.gpu
+
+MODES = [uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_GENERIC]
+
+
+@pytest.fixture(autouse=True)
+def _reset_modes(lib):
+    yield
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lib.set_pointer_mode(uk.POINTER_MODE_AUTO)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("n", range(len(G.PACK_TILES)))
+def test_pack_reference_test_grid(gpu, oracle, n, mode):
+    """tools/pack_test.c's grid: degenerate and small outer shapes x both
+    transposes x padding variants, random strides/offsets/padding value."""
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    tf, t0, t1 = G.PACK_TILES[n]
+    for ci, c in enumerate(T.pack_cases(tf, t0, t1, seed=11000 + n)):
+        rng = np.random.default_rng(ci)
+        inp, out0 = T.make_pack_buffers(c, rng)
+        want = out0.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        got = T.gpu_pack(lib, torch, c, inp, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("n", range(len(G.UNPACK_TILES)))
+def test_unpack_reference_test_grid(gpu, oracle, n, mode):
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    tf, t0, t1 = G.UNPACK_TILES[n]
+    for ci, c in enumerate(T.unpack_cases(tf, t0, t1, seed=12000 + n)):
+        rng = np.random.default_rng(ci)
+        inp, out0 = T.make_unpack_buffers(c, rng)
+        want = out0.copy()
+        G.run_unpack_case(oracle, c, inp, want)
+        got = T.gpu_unpack(lib, torch, c, inp, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+
+
+# Shapes large enough to span several workgroup blocks of the tiled kernels,
+# with ragged edges, all-padding tiles, loose strides and shifted bases.
+TILED_SHAPES = [
+    # (type, tile0, tile1, in0, in1)
+    (uk.PACK_TYPE_F16F16, 16, 16, 300, 270),
+    (uk.PACK_TYPE_F16F16, 16, 16, 256, 256),
+    (uk.PACK_TYPE_I8I8, 16, 32, 130, 515),
+    (uk.PACK_TYPE_I8I8, 32, 8, 16, 1024),
+    (uk.PACK_TYPE_I8I8, 16, 2, 200, 301),
+    (uk.PACK_TYPE_I8I8, 16, 8, 257, 259),
+    (uk.PACK_TYPE_F32F32, 16, 1, 259, 263),
+    (uk.PACK_TYPE_F32F32, 16, 16, 100, 333),
+    (uk.PACK_TYPE_I32I32, 8, 4, 77, 130),
+    (uk.PACK_TYPE_BF16BF16, 16, 2, 130, 258),
+    (uk.PACK_TYPE_F16F16, 1, 16, 37, 400),
+    (uk.PACK_TYPE_F32F32, 3, 5, 200, 200),
+    (uk.PACK_TYPE_F16F16, 6, 7, 200, 200),
+]
+
+
+def _tiled_pack_cases():
+    g = T.Lcg(77)
+    for (tf, t0, t1, in0, in1) in TILED_SHAPES:
+        for ti in (0, 1):
+            for to in (0, 1):
+                for variant in range(3):
+                    a0, a1 = (t1, t0) if ti else (t0, t1)  # extent along matrix dims
+                    o0 = -(-in0 // a0) + (1 if variant == 2 else 0)
+                    o1 = -(-in1 // a1) + (2 if variant == 2 else 0)
+                    flags = tf | (0x100 if ti else 0) | (0x200 if to else 0)
+                    os0, os1 = (o1, o0) if to else (o0, o1)
+                    loose = (0, 4, 1)[variant]
+                    yield T.PackCase(flags, in0, in1, os0, os1, t0, t1,
+                                     in1 + (0, 8, 3)[variant], 1,
+                                     os1 * t0 * t1 + loose,
+                                     (0, 16, 5)[variant], (0, 32, 3)[variant], g.u64())
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_pack_block_spanning_shapes(gpu, oracle, mode):
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    tiled = 0
+    for ci, c in enumerate(_tiled_pack_cases()):
+        rng = np.random.default_rng(500 + ci)
+        inp, out0 = T.make_pack_buffers(c, rng)
+        want = out0.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        got = T.gpu_pack(lib, torch, c, inp, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        tiled += lib.last_kernel_name() == "pack_tiled"
+    if mode == uk.KERNEL_MODE_AUTO:
+        assert tiled >= 60, tiled  # the LDS-staged kernel is the one under test
+    else:
+        assert tiled == 0
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_unpack_block_spanning_shapes(gpu, oracle, mode):
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    tiled = 0
+    for ci, pc in enumerate(_tiled_pack_cases()):
+        if pc.elem_bytes == 1:
+            continue  # unpack has no 1-byte type (exported_bits.h:76)
+        c = T.UnpackCase(pc.flags, pc.out_size0, pc.out_size1, pc.out_size2,
+                         pc.out_size3, pc.in_size0, pc.in_size1, pc.out_stride0,
+                         pc.in_stride0, 1, pc.out_offset, pc.in_offset)
+        rng = np.random.default_rng(900 + ci)
+        inp, out0 = T.make_unpack_buffers(c, rng)
+        want = out0.copy()
+        G.run_unpack_case(oracle, c, inp, want)
+        got = T.gpu_unpack(lib, torch, c, inp, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        tiled += lib.last_kernel_name() == "unpack_tiled"
+    if mode == uk.KERNEL_MODE_AUTO:
+        assert tiled >= 40, tiled
+
+
+def test_pack_unpack_round_trip_and_numpy_identity(gpu):
+    """Size-independent properties at a size the oracle would be slow on:
+    pack == pad+reshape+transpose, unpack(pack(x)) == x."""
+    lib, torch = gpu
+    rng = np.random.default_rng(1)
+    for (dtype, tf, t0, t1, ti, to, shape) in (
+            (np.float32, uk.PACK_TYPE_F32F32, 16, 1, False, True, (1537, 1030)),
+            (np.float16, uk.PACK_TYPE_F16F16, 16, 16, False, False, (2047, 2049)),
+            (np.int32, uk.PACK_TYPE_I32I32, 16, 16, True, True, (1000, 999))):
+        x = rng.integers(-30000, 30000, shape).astype(dtype)
+        pad_val = dtype(-1)
+        pad_bits = int(np.array([pad_val]).view({2: np.uint16, 4: np.uint32}[x.itemsize])[0])
+        want4 = T.numpy_pack(x, t0, t1, ti, to, pad_val)
+        o0, o1, o2, o3 = want4.shape
+        d_x = torch.from_numpy(x).cuda()
+        d_p = torch.zeros(want4.size * x.itemsize, dtype=torch.uint8, device="cuda")
+        flags = tf | (0x100 if ti else 0) | (0x200 if to else 0)
+        lib.pack(d_x.data_ptr(), 0, shape[1], 1, d_p.data_ptr(), 0, o1 * o2 * o3,
+                 o2 * o3, shape[0], shape[1], o0, o1, o2, o3, pad_bits, flags)
+        assert lib.last_kernel_name() == "pack_tiled"
+        got4 = d_p.cpu().numpy().view(dtype).reshape(want4.shape)
+        assert np.array_equal(got4, want4)
+        d_y = torch.full((x.size * x.itemsize,), 0x5A, dtype=torch.uint8, device="cuda")
+        lib.unpack(d_p.data_ptr(), 0, o1 * o2 * o3, o2 * o3, d_y.data_ptr(), 0,
+                   shape[1], 1, o0, o1, o2, o3, shape[0], shape[1], flags)
+        assert lib.last_kernel_name() == "unpack_tiled"
+        assert np.array_equal(d_y.cpu().numpy().view(dtype).reshape(shape), x)
+
+
+def test_host_pointers_are_staged(gpu, oracle):
+    """Ordinary host memory works through the same entry points (staged through
+    the GPU) and leaves stride gaps of the destination untouched."""
+    lib, torch = gpu
+    for ci, c in enumerate(T.pack_cases(uk.PACK_TYPE_F16F16, 6, 7, seed=31,
+                                        outer_shapes=((3, 2), (9, 33)), max_offset=64)):
+        rng = np.random.default_rng(ci)
+        inp, out0 = T.make_pack_buffers(c, rng)
+        want = out0.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        got = out0.copy()
+        es = c.elem_bytes
+        lib.pack(inp.ctypes.data - c.in_offset * es, c.in_offset, c.in_stride0,
+                 c.in_stride1, got.ctypes.data - c.out_offset * es, c.out_offset,
+                 c.out_stride0, c.out_stride1, c.in_size0, c.in_size1, c.out_size0,
+                 c.out_size1, c.out_size2, c.out_size3, c.padding_value, c.flags)
+        assert np.array_equal(got, want), c.label()
+    for ci, c in enumerate(T.unpack_cases(uk.UNPACK_TYPE_I32I32, 3, 4, seed=32,
+                                          outer_shapes=((3, 2), (9, 33)), max_offset=64)):
+        rng = np.random.default_rng(ci)
+        inp, out0 = T.make_unpack_buffers(c, rng)
+        want = out0.copy()
+        G.run_unpack_case(oracle, c, inp, want)
+        got = out0.copy()
+        es = c.elem_bytes
+        lib.unpack(inp.ctypes.data - c.in_offset * es, c.in_offset, c.in_stride0,
+                   c.in_stride1, got.ctypes.data - c.out_offset * es, c.out_offset,
+                   c.out_stride0, c.out_stride1, c.in_size0, c.in_size1, c.in_size2,
+                   c.in_size3, c.out_size0, c.out_size1, c.flags)
+        assert np.array_equal(got, want), c.label()
