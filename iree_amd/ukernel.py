@@ -85,6 +85,32 @@ class ContractViolation(RuntimeError):
     """Raised by the Python-side assert handler (see raise_on_violation)."""
 
 
+def _share_hip_runtime_with_torch():
+    """A process must hold ONE HIP runtime, or device pointers made by one copy
+    are unknown to the other. PyTorch wheels bundle their own libamdhip64.so
+    (soname libamdhip64.so.7) and load it by file name, so it has to be in the
+    process before this library's NEEDED entry of the same soname is resolved;
+    then both share it. Without PyTorch the system runtime is used."""
+    import importlib.util
+    import sys
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.origin:
+        return
+    libdir = os.path.join(os.path.dirname(spec.origin), "lib")
+    for name in ("libhsa-runtime64.so", "libamdhip64.so"):
+        cand = os.path.join(libdir, name)
+        if os.path.exists(cand):
+            try:
+                ctypes.CDLL(cand, mode=ctypes.RTLD_GLOBAL)
+            except OSError:
+                return
+
+
 class UKernelLibrary:
     """The loaded shared library with typed entry points."""
 
@@ -94,6 +120,7 @@ class UKernelLibrary:
                 f"{path} is missing: build it with `python -m iree_amd.build` "
                 "(there is no CPU or PyTorch fallback for these kernels)")
         self.path = path
+        _share_hip_runtime_with_torch()
         self.lib = ctypes.CDLL(path)
         L = self.lib
         L.iree_uk_mmt4d.argtypes = [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64,
