@@ -79,7 +79,10 @@ def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n):
     if not lib.mmt4d_info(M0, N0, K0, tf):
         pytest.skip("no MFMA kernel for this tile shape; covered by the generic kernel")
     bits = uk.MMT4D_TYPE_BITS[tf][0]
-    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=14000 + n,
+    # Loose strides and offsets in steps of 16 elements: the MFMA kernels need
+    # 16-byte aligned panels (anything else goes to the generic kernel, which
+    # the reference-grid test above exercises with 1-element slack).
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=14000 + n, slack=16,
                                          shapes=_mfma_shapes(M0, N0, K0, bits))):
         rng = np.random.default_rng(ci)
         lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)

@@ -315,10 +315,11 @@ def _round_up_whole_bytes(v: int, bits: int) -> int:
 
 
 def mmt4d_cases(type_flag: int, M0: int, N0: int, K0: int, seed: int,
-                shapes=MMT4D_TEST_SHAPES, extra_flags: int = 0):
+                shapes=MMT4D_TEST_SHAPES, extra_flags: int = 0, slack: int = 1):
     """The case grid of tools/mmt4d_test.c:354-404,448-506: shapes x ACCUMULATE
-    off/on, strides tight or one element loose, offsets 0 or 1 (rounded up to
-    whole bytes for 4-bit types)."""
+    off/on, strides tight or `slack` elements loose, offsets 0 or `slack`
+    (rounded up to whole bytes for 4-bit types). slack=1 is the reference's
+    choice; slack=16 keeps operands 16-byte aligned."""
     g = Lcg(seed)
     lb, rb, ob = uk.MMT4D_TYPE_BITS[type_flag]
     for (m, n, k) in shapes:
@@ -326,12 +327,12 @@ def mmt4d_cases(type_flag: int, M0: int, N0: int, K0: int, seed: int,
             k = 100  # tools/mmt4d_test.c:456-458
         for acc in (0, 1):
             flags = type_flag | extra_flags | (uk.MMT4D_ACCUMULATE if acc else 0)
-            ls = _round_up_whole_bytes(k * M0 * K0 + g.bit(), lb)
-            rs = _round_up_whole_bytes(k * N0 * K0 + g.bit(), rb)
-            os_ = _round_up_whole_bytes(n * M0 * N0 + g.bit(), ob)
-            lo = _round_up_whole_bytes(g.bit(), lb)
-            ro = _round_up_whole_bytes(g.bit(), rb)
-            oo = _round_up_whole_bytes(g.bit(), ob)
+            ls = _round_up_whole_bytes(k * M0 * K0 + slack * g.bit(), lb)
+            rs = _round_up_whole_bytes(k * N0 * K0 + slack * g.bit(), rb)
+            os_ = _round_up_whole_bytes(n * M0 * N0 + slack * g.bit(), ob)
+            lo = _round_up_whole_bytes(slack * g.bit(), lb)
+            ro = _round_up_whole_bytes(slack * g.bit(), rb)
+            oo = _round_up_whole_bytes(slack * g.bit(), ob)
             yield Mmt4dCase(flags, m, n, k, M0, N0, K0, ls, rs, os_, lo, ro, oo)
 
 
