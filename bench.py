@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 pack / mmt4d / unpack ukernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+                    [--no-extra] [--no-cpu]
+
+A step is one pass of the workload's whole chain over one batch of seeded
+synthetic tensors that are already resident in HBM. The default workload is
+the f16 pack -> mmt4d -> unpack chain at M=N=K=4096 with 16x16x16 tiles. One
+JSON line is printed; `roofline` describes the dominant kernel (mmt4d),
+`cpu_baseline` the same chain on the host cores, and `extra` carries the other
+benchmark configurations (kernel-level event timings).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+EXTRA_WORKLOADS = [
+    "s8_mmt4d_8192_k2", "s8_mmt4d_8192_k16", "s8_mmt4d_8192_k64", "s8_mmt4d_1024_k2",
+    "c2_f16_chain_ragged", "c3_s8_decode", "c4_f8_prefill",
+    "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8",
+    "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288",
+]
+
+
+def cpu_threads() -> int:
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    for var in ("OMP_NUM_THREADS",):
+        if os.environ.get(var, "").isdigit():
+            n = min(n, int(os.environ[var]))
+    return max(1, min(n, 16))
+
+
+def cpu_baseline_c2(keep: dict, target_seconds: float = 12.0) -> dict:
+    """The f16 chain on the host: the compiled reference C ukernels when
+    oracle/_ref holds them (kind "reference"), else the C restatement (kind
+    "port"). pack of both operands runs in full; mmt4d and unpack run on a slab
+    of M tile-rows sized for about `target_seconds`, split over threads through
+    the offset/stride parameters, and are extrapolated to the whole problem."""
+    import numpy as np
+    from oracle import uk_oracle
+    from iree_amd import ukernel as uk
+
+    kind = "reference" if uk_oracle.Checker.reference_available() else "port"
+    chk = uk_oracle.Checker("reference" if kind == "reference" else "oracle")
+    chk.use_host_cpu_features(True)
+    T = cpu_threads()
+    M, N, K = keep["M"], keep["N"], keep["K"]
+    M0, N0, K0 = keep["M0"], keep["N0"], keep["K0"]
+    M1, N1, K1 = -(-M // M0), -(-N // N0), K // K0
+    a = keep["a"].cpu().numpy().view(np.uint16)
+    bt = keep["bt"].cpu().numpy().view(np.uint16)
+    lhs4 = np.zeros(M1 * K1 * M0 * K0, np.uint16)
+    rhs4 = np.zeros(N1 * K1 * N0 * K0, np.uint16)
+    t0 = time.perf_counter()
+    chk.pack(a, 0, K, 1, lhs4, 0, K1 * M0 * K0, M0 * K0, M, K, M1, K1, M0, K0, 0, uk.PACK_TYPE_F16F16)
+    chk.pack(bt, 0, K, 1, rhs4, 0, K1 * N0 * K0, N0 * K0, N, K, N1, K1, N0, K0, 0, uk.PACK_TYPE_F16F16)
+    t_pack = time.perf_counter() - t0
+    flags = uk.MMT4D_TYPE_F16F16F32 | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
+    # Calibrate on one tile-row per thread, then size the slab.
+    out4 = np.zeros(M1 * N1 * M0 * N0, np.float32)
+    t0 = time.perf_counter()
+    chk.mmt4d_threaded(T, lhs4, K1 * M0 * K0, rhs4, K1 * N0 * K0, out4, N1 * M0 * N0,
+                       T, N1, K1, M0, N0, K0, flags)
+    t_cal = time.perf_counter() - t0
+    slab = int(max(T, min(M1, T * round(target_seconds / max(t_cal, 1e-3)))))
+    slab -= slab % T
+    t0 = time.perf_counter()
+    chk.mmt4d_threaded(T, lhs4, K1 * M0 * K0, rhs4, K1 * N0 * K0, out4, N1 * M0 * N0,
+                       slab, N1, K1, M0, N0, K0, flags)
+    t_mm = time.perf_counter() - t0
+    out = np.zeros(M * N, np.float32)
+    rows = min(M, slab * M0)
+    t0 = time.perf_counter()
+    chk.unpack(out4, 0, N1 * M0 * N0, M0 * N0, out, 0, N, 1, slab, N1, M0, N0, rows, N,
+               uk.UNPACK_TYPE_F32F32)
+    t_un = time.perf_counter() - t0
+    total = t_pack + (t_mm + t_un) * (M1 / slab)
+    return {
+        "value": round(2.0 * M * N * K / total / 1e12, 6), "unit": "TFLOP/s", "cores": T,
+        "kind": kind,
+        "sample": (f"pack of both operands in full (1 thread, {t_pack:.2f} s); mmt4d on "
+                   f"{slab}/{M1} M tile-rows over {T} threads ({t_mm:.2f} s, generic f16 tile "
+                   f"function: no x86 tile exists for 16x16x16) and unpack of those rows "
+                   f"({t_un:.2f} s), extrapolated x{M1 / slab:.1f}"),
+    }, out4, slab
+
+
+def verify_c2(runner, keep, cpu_out4, slab) -> dict:
+    """GPU result of the timed chain against the CPU checker on the slab the
+    baseline computed: max|gpu-ref|/max|ref| must be <= 1e-2 (f16 inputs, f32
+    accumulation in a different order)."""
+    import numpy as np
+    M0, N0 = keep["M0"], keep["N0"]
+    N1 = -(-keep["N"] // N0)
+    n = slab * N1 * M0 * N0
+    got = keep["out4"][:n].cpu().numpy()
+    want = cpu_out4[:n]
+    err = float(np.abs(got - want).max() / np.abs(want).max())
+    return {"checked_tile_rows": slab, "max_err_over_max_ref": err, "tolerance": 1e-2,
+            "ok": bool(err <= 1e-2)}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2_f16_chain_4096")
+    ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--extra-iters", type=int, default=20)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path shards by tile rows with no "
+              "exchange step, but no multi-GPU figure is produced); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from iree_amd import runner as rn
+
+    torch.cuda.set_device(0)
+    R = rn.Runner(seed=0)
+    wl = R.workload(args.workload)
+    dominant = "mmt4d" if any(o.name == "mmt4d" for o in wl.ops) else wl.ops[0].name
+    sec_per_step, dom_us = R.run_steps(wl, args.steps, args.warmup, dominant)
+    dom = next(o for o in wl.ops if o.name == dominant)
+    roof = R.roofline(dom, dom_us)
+    roof["kernel"] = dom.kernel
+    roof["avg_us"] = round(dom_us, 2)
+
+    per_kernel = {}
+    for op in wl.ops:
+        avg, mn, med = R.time_op(op, max(5, min(args.steps, 30)))
+        r = R.roofline(op, avg)
+        per_kernel[op.name] = {"kernel": op.kernel, "avg_us": round(avg, 2), "min_us": round(mn, 2),
+                               "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"]}
+
+    if wl.flops:
+        metric, unit = "mmt4d TFLOP/s over the pack->mmt4d->unpack chain", "TFLOP/s"
+        value = wl.flops / sec_per_step / 1e12
+    else:
+        metric, unit = "pack/unpack HBM GB/s", "GB/s"
+        value = wl.bytes / sec_per_step / 1e9
+
+    result = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype,
+        "data": "synthetic (seeded, generated in HBM)",
+        "config": {"workload": wl.name, "description": wl.description},
+        "roofline": roof, "kernels": per_kernel,
+        "measured_copy_GBps": round(R.measured_copy_gbps(), 1),
+    }
+
+    if not args.no_cpu and args.workload.startswith("c2_f16_chain"):
+        base, cpu_out4, slab = cpu_baseline_c2(wl.keep)
+        result["cpu_baseline"] = base
+        result["parity"] = verify_c2(R, wl.keep, cpu_out4, slab)
+    else:
+        result["cpu_baseline"] = None
+
+    if not args.no_extra:
+        extra = {}
+        del wl
+        for name in EXTRA_WORKLOADS:
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            w = R.workload(name)
+            entry = {"description": w.description, "kernels": {}}
+            total_us = 0.0
+            for op in w.ops:
+                avg, mn, med = R.time_op(op, args.extra_iters)
+                r = R.roofline(op, avg)
+                total_us += avg
+                entry["kernels"][op.name] = {
+                    "kernel": op.kernel, "avg_us": round(avg, 2), "min_us": round(mn, 2),
+                    "bound": r["bound"], "achieved": r["achieved"], "unit": r["unit"],
+                    "frac": r["frac"]}
+            if w.flops:
+                entry["chain_TFLOPs"] = round(w.flops / (total_us * 1e-6) / 1e12, 3)
+            extra[name] = entry
+            del w
+        result["extra"] = extra
+
+    R.close()
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

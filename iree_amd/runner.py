@@ -1,0 +1,336 @@
+"""One-GPU runner for the pack / mmt4d / unpack ukernels: builds the benchmark
+workloads from seeded synthetic tensors resident in HBM, times each kernel with
+HIP events on the stream the kernels are launched on, and reports TOPS /
+TFLOP/s and GB/s next to the MI355X roofline.
+
+Conventions follow the reference's own benchmarks with one stated difference:
+  * mmt4d work = 2*M*N*K on the logical (unpadded) sizes
+    (runtime/src/iree/builtins/ukernel/tools/mmt4d_benchmark.c:82-84);
+  * pack/unpack bytes = bytes that must be read + bytes that must be written
+    (the reference counts the output buffer only,
+    tools/pack_benchmark.c:97-101; read+write is what bounds an HBM kernel).
+
+PyTorch is used for device memory, streams and events only.
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Callable
+
+from . import ukernel as uk
+
+# Published MI355X peaks (dense).
+PEAK_HBM_GBPS = 8000.0
+PEAK_TFLOPS = {"s8": 5000.0, "f8": 5000.0, "f16": 2500.0, "bf16": 2500.0}
+
+
+@dataclasses.dataclass
+class Op:
+    name: str                 # e.g. "mmt4d", "pack_lhs"
+    launch: Callable[[], None]
+    flops: float = 0.0        # algorithmic ops per launch
+    bytes: float = 0.0        # algorithmic HBM bytes per launch (read + write)
+    bound: str = "hbm"        # "hbm" | "mfma"
+    dtype: str = ""
+    kernel: str = ""          # filled after the first launch
+
+
+@dataclasses.dataclass
+class Workload:
+    name: str
+    description: str
+    ops: list
+    flops: float              # logical 2*M*N*K of the whole step (0 for pure movement)
+    bytes: float              # algorithmic bytes of the whole step
+    dtype: str
+    keep: dict                # tensors and sizes for verification
+
+
+def _torch():
+    import torch
+    return torch
+
+
+class Runner:
+    def __init__(self, seed: int = 0):
+        torch = _torch()
+        if not torch.cuda.is_available():
+            raise RuntimeError("the runner needs a GPU")
+        self.torch = torch
+        self.lib = uk.load()
+        self.stream = torch.cuda.Stream()
+        self.seed = seed
+        self.lib.set_stream(self.stream.cuda_stream)
+        self.lib.set_pointer_mode(uk.POINTER_MODE_DEVICE)
+
+    def close(self):
+        self.lib.set_stream(None)
+        self.lib.set_pointer_mode(uk.POINTER_MODE_AUTO)
+
+    # ------------------------------------------------------------ generators
+    def _gen(self, tensor_id: int):
+        g = self.torch.Generator(device="cuda")
+        g.manual_seed((self.seed << 8) ^ tensor_id)
+        return g
+
+    def normal(self, shape, dtype, tensor_id, scale=1.0):
+        t = self.torch.randn(shape, generator=self._gen(tensor_id), device="cuda",
+                             dtype=self.torch.float32)
+        if scale != 1.0:
+            t *= scale
+        return t.to(dtype)
+
+    def normal_f8(self, shape, tensor_id):
+        """N(0,1) scaled so that the sample maximum maps to 448, cast to
+        E4M3FN with round-to-nearest-even; stored as bytes."""
+        torch = self.torch
+        t = torch.randn(shape, generator=self._gen(tensor_id), device="cuda",
+                        dtype=torch.float32)
+        t *= 448.0 / t.abs().max()
+        return t.to(torch.float8_e4m3fn).view(torch.uint8)
+
+    def uniform_s8(self, shape, tensor_id):
+        return self.torch.randint(-128, 128, shape, generator=self._gen(tensor_id),
+                                  device="cuda", dtype=self.torch.int8)
+
+    def clipped_normal_s8(self, shape, tensor_id, sigma):
+        t = self.torch.randn(shape, generator=self._gen(tensor_id), device="cuda",
+                             dtype=self.torch.float32) * sigma
+        return t.round().clamp(-128, 127).to(self.torch.int8)
+
+    def empty(self, n, dtype):
+        return self.torch.empty(n, device="cuda", dtype=dtype)
+
+    # -------------------------------------------------------------- op makers
+    def _pack_op(self, name, src, rows, cols, dst, tile0, tile1, type_flag, es,
+                 pad=0, transpose_outer=False):
+        o0, o1 = -(-rows // tile0), -(-cols // tile1)
+        flags = type_flag | (uk.PACK_TRANSPOSE_OUTER if transpose_outer else 0)
+        s0, s1 = (o1, o0) if transpose_outer else (o0, o1)
+        lib = self.lib
+        sp, dp = src.data_ptr(), dst.data_ptr()
+
+        def launch():
+            lib.pack(sp, 0, cols, 1, dp, 0, s1 * tile0 * tile1, tile0 * tile1, rows,
+                     cols, s0, s1, tile0, tile1, pad, flags)
+        return Op(name, launch, 0.0, float(rows * cols * es + o0 * o1 * tile0 * tile1 * es),
+                  "hbm")
+
+    def _unpack_op(self, name, src, dst, rows, cols, tile0, tile1, type_flag, es,
+                   transpose_outer=False):
+        o0, o1 = -(-rows // tile0), -(-cols // tile1)
+        flags = type_flag | (uk.UNPACK_TRANSPOSE_OUTER if transpose_outer else 0)
+        s0, s1 = (o1, o0) if transpose_outer else (o0, o1)
+        lib = self.lib
+        sp, dp = src.data_ptr(), dst.data_ptr()
+
+        def launch():
+            lib.unpack(sp, 0, s1 * tile0 * tile1, tile0 * tile1, dp, 0, cols, 1, s0,
+                       s1, tile0, tile1, rows, cols, flags)
+        # Only the bytes of tiles' valid elements have to move.
+        return Op(name, launch, 0.0, float(2 * rows * cols * es), "hbm")
+
+    def _mmt4d_op(self, lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0, type_flag, dtype,
+                  in_es, accumulate=False, logical=None):
+        flags = type_flag | (uk.MMT4D_ACCUMULATE if accumulate else 0)
+        lib = self.lib
+        lp, rp, op_ = lhs4.data_ptr(), rhs4.data_ptr(), out4.data_ptr()
+
+        def launch():
+            lib.mmt4d(lp, 0, K1 * M0 * K0, rp, 0, K1 * N0 * K0, op_, 0, N1 * M0 * N0,
+                      M1, N1, K1, M0, N0, K0, flags)
+        M, N, K = logical if logical else (M1 * M0, N1 * N0, K1 * K0)
+        out_bytes = M1 * N1 * M0 * N0 * 4 * (2 if accumulate else 1)
+        nbytes = (M1 * K1 * M0 * K0 + N1 * K1 * N0 * K0) * in_es + out_bytes
+        return Op("mmt4d", launch, 2.0 * M * N * K, float(nbytes), "mfma", dtype)
+
+    # --------------------------------------------------------------- workloads
+    def workload(self, name: str) -> Workload:
+        torch = self.torch
+        if name in ("c2_f16_chain_4096", "c2_f16_chain_ragged"):
+            M, N, K = (4096, 4096, 4096) if name.endswith("4096") else (4095, 4097, 4096)
+            M0 = N0 = K0 = 16
+            M1, N1, K1 = -(-M // M0), -(-N // N0), K // K0
+            a = self.normal((M, K), torch.float16, 1)
+            bt = self.normal((N, K), torch.float16, 2)   # RHS given transposed: [N, K]
+            lhs4 = self.empty(M1 * K1 * M0 * K0, torch.float16)
+            rhs4 = self.empty(N1 * K1 * N0 * K0, torch.float16)
+            out4 = self.empty(M1 * N1 * M0 * N0, torch.float32)
+            out = self.empty(M * N, torch.float32)
+            ops = [self._pack_op("pack_lhs", a, M, K, lhs4, M0, K0, uk.PACK_TYPE_F16F16, 2),
+                   self._pack_op("pack_rhs", bt, N, K, rhs4, N0, K0, uk.PACK_TYPE_F16F16, 2),
+                   self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                  uk.MMT4D_TYPE_F16F16F32, "f16", 2, logical=(M, N, K)),
+                   self._unpack_op("unpack", out4, out, M, N, M0, N0, uk.UNPACK_TYPE_F32F32, 4)]
+            return Workload(name, f"pack->mmt4d->unpack f16xf16->f32 M={M} N={N} K={K} tiles 16x16x16",
+                            ops, 2.0 * M * N * K, sum(o.bytes for o in ops), "f16",
+                            dict(a=a, bt=bt, lhs4=lhs4, rhs4=rhs4, out4=out4, out=out,
+                                 M=M, N=N, K=K, M0=M0, N0=N0, K0=K0))
+        if name.startswith("s8_mmt4d_"):
+            # s8_mmt4d_<size>_k<K0>, tiles 16x16xK0, packed operands filled directly.
+            _, _, size, k0 = name.split("_")
+            S, K0 = int(size), int(k0[1:])
+            M0 = N0 = 16
+            M1 = N1 = S // 16
+            K1 = S // K0
+            lhs4 = self.uniform_s8((M1 * K1 * M0 * K0,), 3)
+            rhs4 = self.uniform_s8((N1 * K1 * N0 * K0,), 4)
+            out4 = self.empty(M1 * N1 * M0 * N0, torch.int32)
+            op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                uk.MMT4D_TYPE_S8S8S32, "s8", 1)
+            return Workload(name, f"mmt4d s8xs8->s32 {S}^3 tiles 16x16x{K0}", [op], op.flops,
+                            op.bytes, "s8", dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1,
+                                                 N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
+        if name.startswith("bf16_mmt4d_"):
+            _, _, size, k0 = name.split("_")
+            S, K0 = int(size), int(k0[1:])
+            M0 = N0 = 16
+            M1 = N1 = S // 16
+            K1 = S // K0
+            lhs4 = self.normal((M1 * K1 * M0 * K0,), torch.bfloat16, 5)
+            rhs4 = self.normal((N1 * K1 * N0 * K0,), torch.bfloat16, 6)
+            out4 = self.empty(M1 * N1 * M0 * N0, torch.float32)
+            op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                uk.MMT4D_TYPE_BF16BF16F32, "bf16", 2)
+            return Workload(name, f"mmt4d bf16xbf16->f32 {S}^3 tiles 16x16x{K0}", [op],
+                            op.flops, op.bytes, "bf16",
+                            dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
+                                 M0=M0, N0=N0, K0=K0))
+        if name == "c3_s8_decode":
+            # Decode-shaped quantized linear layer: 16 activations rows padded to
+            # M0=32, weights [14336, 4096] pre-packed once (not timed), ACCUMULATE
+            # into a seeded s32 buffer.
+            Mlog, K, N = 16, 4096, 14336
+            M0, N0, K0 = 32, 16, 8
+            M1, N1, K1 = 1, N // N0, K // K0
+            act = self.clipped_normal_s8((Mlog, K), 7, 40.0)
+            w = self.uniform_s8((N, K), 8)
+            lhs4 = self.empty(M1 * K1 * M0 * K0, torch.int8)
+            rhs4 = self.empty(N1 * K1 * N0 * K0, torch.int8)
+            out4 = torch.randint(-2 ** 15, 2 ** 15, (M1 * N1 * M0 * N0,),
+                                 generator=self._gen(9), device="cuda", dtype=torch.int32)
+            pack_w = self._pack_op("pack_weights", w, N, K, rhs4, N0, K0, uk.PACK_TYPE_I8I8, 1)
+            pack_w.launch()   # once, outside any timing
+            pack_a = self._pack_op("pack_act", act, Mlog, K, lhs4, M0, K0, uk.PACK_TYPE_I8I8, 1)
+            pack_a.launch()
+            op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                uk.MMT4D_TYPE_S8S8S32, "s8", 1, accumulate=True,
+                                logical=(Mlog, N, K))
+            op.bound = "hbm"
+            return Workload(name, "mmt4d s8 decode M=16(32) K=4096 N=14336 tiles 32x16x8 ACCUMULATE",
+                            [op], op.flops, op.bytes, "s8",
+                            dict(act=act, w=w, lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1,
+                                 K1=K1, M0=M0, N0=N0, K0=K0))
+        if name == "c4_f8_prefill":
+            M, K, N = 2048, 8192, 28672
+            M0, N0, K0 = 16, 16, 32
+            M1, N1, K1 = M // M0, N // N0, K // K0
+            a = self.normal_f8((M, K), 10)
+            bt = self.normal_f8((N, K), 11)
+            lhs4 = self.empty(M * K, torch.uint8)
+            rhs4 = self.empty(N * K, torch.uint8)
+            out4 = self.empty(M * N, torch.float32)
+            ops = [self._pack_op("pack_lhs", a, M, K, lhs4, M0, K0, uk.PACK_TYPE_I8I8, 1),
+                   self._pack_op("pack_rhs", bt, N, K, rhs4, N0, K0, uk.PACK_TYPE_I8I8, 1),
+                   self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                  uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, "f8", 1)]
+            return Workload(name, "pack+pack+mmt4d f8E4M3FN->f32 M=2048 K=8192 N=28672 tiles 16x16x32",
+                            ops, 2.0 * M * N * K, sum(o.bytes for o in ops), "f8",
+                            dict(a=a, bt=bt, lhs4=lhs4, rhs4=rhs4, out4=out4, M=M, N=N, K=K,
+                                 M1=M1, N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
+        if name in ("c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288"):
+            rows, cols = (12288, 12289) if name.endswith("12289") else (12289, 12288)
+            x = self.normal((rows, cols), torch.float32, 12)
+            o0, o1 = -(-rows // 16), cols
+            packed = self.empty(o0 * o1 * 16, torch.float32)
+            back = self.empty(rows * cols, torch.float32)
+            pad = 0xBF800000  # -1.0f
+            ops = [self._pack_op("pack", x, rows, cols, packed, 16, 1, uk.PACK_TYPE_F32F32, 4,
+                                 pad=pad, transpose_outer=True),
+                   self._unpack_op("unpack", packed, back, rows, cols, 16, 1,
+                                   uk.UNPACK_TYPE_F32F32, 4, transpose_outer=True)]
+            return Workload(name, f"pack+unpack f32 {rows}x{cols} tiles 16x1 TRANSPOSE_OUTER pad -1.0",
+                            ops, 0.0, sum(o.bytes for o in ops), "f32",
+                            dict(x=x, packed=packed, back=back, rows=rows, cols=cols))
+        raise KeyError(name)
+
+    # ------------------------------------------------------------------ timing
+    def time_op(self, op: Op, iters: int, warmup: int = 2):
+        """Average and minimum duration in microseconds of `iters` launches,
+        each bracketed by HIP events on the launch stream."""
+        torch = self.torch
+        with torch.cuda.stream(self.stream):
+            for _ in range(warmup):
+                op.launch()
+            op.kernel = self.lib.last_kernel_name()
+            starts = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+            ends = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+            for i in range(iters):
+                starts[i].record(self.stream)
+                op.launch()
+                ends[i].record(self.stream)
+        self.stream.synchronize()
+        us = [s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends)]
+        return sum(us) / len(us), min(us), sorted(us)[len(us) // 2]
+
+    @staticmethod
+    def roofline(op: Op, avg_us: float) -> dict:
+        if op.bound == "mfma":
+            achieved = op.flops / (avg_us * 1e-6) / 1e12
+            peak = PEAK_TFLOPS[op.dtype]
+            unit = "TFLOP/s"
+        else:
+            achieved = op.bytes / (avg_us * 1e-6) / 1e9
+            peak = PEAK_HBM_GBPS
+            unit = "GB/s"
+        return {"bound": op.bound, "achieved": round(achieved, 3), "peak": peak,
+                "unit": unit, "frac": round(achieved / peak, 4), "traffic": None}
+
+    def run_steps(self, wl: Workload, steps: int, warmup: int, dominant: str):
+        """Times exactly `steps` passes of the whole workload (wall clock around
+        a synchronize on both sides) and, inside the same timed region, each
+        launch of the dominant kernel with HIP events on the launch stream."""
+        import time
+        torch = self.torch
+        dom_starts, dom_ends = [], []
+        with torch.cuda.stream(self.stream):
+            for _ in range(warmup):
+                for op in wl.ops:
+                    op.launch()
+                    op.kernel = self.lib.last_kernel_name()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                for op in wl.ops:
+                    if op.name == dominant:
+                        s = torch.cuda.Event(enable_timing=True)
+                        e = torch.cuda.Event(enable_timing=True)
+                        s.record(self.stream)
+                        op.launch()
+                        e.record(self.stream)
+                        dom_starts.append(s)
+                        dom_ends.append(e)
+                    else:
+                        op.launch()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+        dom_us = [s.elapsed_time(e) * 1e3 for s, e in zip(dom_starts, dom_ends)]
+        return (t1 - t0) / steps, (sum(dom_us) / len(dom_us) if dom_us else math.nan)
+
+    def measured_copy_gbps(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
+        """Device-to-device copy rate (read + write bytes), for a measured HBM
+        ceiling next to the nominal one."""
+        torch = self.torch
+        a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        with torch.cuda.stream(self.stream):
+            b.copy_(a)
+            s = torch.cuda.Event(enable_timing=True)
+            e = torch.cuda.Event(enable_timing=True)
+            s.record(self.stream)
+            for _ in range(iters):
+                b.copy_(a)
+            e.record(self.stream)
+        self.stream.synchronize()
+        return 2.0 * nbytes * iters / (s.elapsed_time(e) * 1e-3) / 1e9
