@@ -312,10 +312,14 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_pointer_mode(int mode);
 
 /* Kernel selection override for testing and benchmarking, per thread.
  *   AUTO    : fastest kernel that serves the case.
- *   GENERIC : always the scalar any-shape kernels. */
+ *   GENERIC : always the scalar any-shape kernels.
+ *   MFMA_VARIANT + v : mmt4d takes MFMA workgroup shape v where it can serve
+ *             the call (1 = 256x256, 2 = 128x128, 3 = 64x64, 4 = 32x64)
+ *             instead of choosing by problem size; pack/unpack as AUTO. */
 enum {
   IREE_UK_AMD_KERNEL_MODE_AUTO = 0,
   IREE_UK_AMD_KERNEL_MODE_GENERIC = 1,
+  IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT = 16,
 };
 IREE_UK_AMD_EXPORT void iree_uk_amd_set_kernel_mode(int mode);
 

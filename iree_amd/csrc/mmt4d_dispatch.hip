@@ -7,7 +7,8 @@
 extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
     const iree_uk_mmt4d_params_t* p, void* stream);
 extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(
-    const iree_uk_mmt4d_params_t* p, void* stream, const char** kernel_name);
+    const iree_uk_mmt4d_params_t* p, void* stream, int forced_variant,
+    const char** kernel_name);
 extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
                                                     int32_t K0, uint32_t flags);
 
@@ -22,7 +23,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
                                             const char** kernel_name) {
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC &&
       iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) {
-    int st = iree_uk_amd_hip_launch_mmt4d_mfma(p, stream, kernel_name);
+    const int forced = kernel_mode >= IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
+                           ? kernel_mode - IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
+                           : 0;
+    int st = iree_uk_amd_hip_launch_mmt4d_mfma(p, stream, forced, kernel_name);
     // A negative status means "shape not served after all"; fall through.
     if (st >= 0) return st;
   }

@@ -1,0 +1,615 @@
+// mmt4d on the gfx950 matrix cores: the kernel template.
+//
+// Operands keep the ukernel ABI layout: LHS [M1][K1][M0][K0], RHS
+// [N1][K1][N0][K0] (both K-major per tile row), OUT [M1][N1][M0][N0]
+// (runtime/src/iree/builtins/ukernel/mmt4d.c:55-100 is the pointer arithmetic
+// this replaces). A workgroup owns a block of whole LHS panels x whole RHS
+// panels; each of its waves owns TM x TN accumulator blocks of 16x16.
+//
+// The MFMA instructions used take, per lane, 16 (2x16 for f8) consecutive
+// bytes of K for ONE row: lane l feeds row l%16 with K-slice l/16. The sum
+// over K is order-free as far as the instruction is concerned, so any
+// assignment of K bytes to (instruction, slice, byte) works as long as LHS and
+// RHS use the same one. That freedom is what lets every K0 be served:
+//
+//   row bytes RB = K0 * sizeof(elem)
+//   RB >= 16 : a 16-byte piece of a tile row is already an MFMA operand;
+//              global -> LDS is a 16-byte-granular copy in which each lane
+//              fetches exactly the piece its LDS slot wants.
+//   RB = 8/4/2: a 16-byte global piece holds R = 16/RB rows of one K-tile. A
+//              lane loads the same R rows from R different K-tiles and
+//              regroups them in registers into R one-row operands (register
+//              selection for RB = 8 and 4, v_perm_b32 for RB = 2) before
+//              storing them to LDS.
+//
+// LDS holds, per pipeline stage, the operands exactly as the waves consume
+// them: [row block of 16][group of 4 K-slices][slice q][row r][16 bytes], so an
+// operand fetch is one ds_read_b128 per lane over a contiguous KiB.
+//
+// Pipeline: double-buffered LDS; global loads run PF steps ahead of the MFMAs
+// through PF register sets; one barrier per K step.
+#ifndef IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
+#define IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+namespace uk_mfma {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+enum class Elem { kS8, kF16, kBF16, kF8 };
+
+template <Elem E> struct ElemTraits;
+
+template <> struct ElemTraits<Elem::kS8> {
+  using Acc = v4i;
+  using Scalar = int32_t;
+  static constexpr int kHalves = 1;  // 16-byte pieces per lane operand
+  static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b[0], c, 0, 0, 0);
+  }
+};
+template <> struct ElemTraits<Elem::kF16> {
+  using Acc = v4f;
+  using Scalar = float;
+  static constexpr int kHalves = 1;
+  static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+        __builtin_bit_cast(v8h, a[0]), __builtin_bit_cast(v8h, b[0]), c, 0, 0, 0);
+  }
+};
+template <> struct ElemTraits<Elem::kBF16> {
+  using Acc = v4f;
+  using Scalar = float;
+  static constexpr int kHalves = 1;
+  static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+        __builtin_bit_cast(v8bf, a[0]), __builtin_bit_cast(v8bf, b[0]), c, 0, 0, 0);
+  }
+};
+template <> struct ElemTraits<Elem::kF8> {
+  using Acc = v4f;
+  using Scalar = float;
+  static constexpr int kHalves = 2;
+  static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
+    v8i av = {a[0][0], a[0][1], a[0][2], a[0][3], a[1][0], a[1][1], a[1][2], a[1][3]};
+    v8i bv = {b[0][0], b[0][1], b[0][2], b[0][3], b[1][0], b[1][1], b[1][2], b[1][3]};
+    // Formats 0/0 = E4M3 x E4M3; block scales of 2^0 (E8M0 code 127).
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+        av, bv, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  }
+};
+
+struct Args {
+  const char* lhs;
+  const char* rhs;
+  char* out;
+  int64_t lhs_stride;  // bytes between LHS panels
+  int64_t rhs_stride;  // bytes between RHS panels
+  int64_t out_stride;  // bytes between rows of output tiles
+  int32_t M1, N1, K1;
+  int32_t M0, N0;
+  int32_t rb;          // bytes per tile row (K0 * element size), power of two
+  int32_t lrb;         // log2(rb)
+  int32_t bpm, bpn;    // whole panels per workgroup along M and N
+  int32_t grid_m, grid_n;
+  int32_t steps;       // K steps
+  uint32_t accumulate;
+  uint32_t tail;       // 1 when the last K step is partial
+  uint32_t band;       // workgroup rows per rasterization band
+};
+
+// Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that
+// store together write rows of the same residue mod 8 for different K slices;
+// XOR-ing the slot with (2*slice + top row bit) spreads them over the eight
+// 16-byte bank groups. Readers apply the same mask.
+__device__ __forceinline__ uint32_t swizzle_mask(uint32_t ch, uint32_t hi) {
+  return (2 * (ch & 3) + hi) & 7;
+}
+
+// Regroups R pieces (each: R rows x RB bytes of one K-tile) into R pieces
+// (each: one row x 16 bytes over R K-tiles). in[t] is K-tile t; out[j] row j.
+template <int RBC>
+__device__ __forceinline__ void regroup(const v4i* in, v4i* out) {
+  if constexpr (RBC == 8) {
+    out[0] = v4i{in[0][0], in[0][1], in[1][0], in[1][1]};
+    out[1] = v4i{in[0][2], in[0][3], in[1][2], in[1][3]};
+  } else if constexpr (RBC == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = v4i{in[0][j], in[1][j], in[2][j], in[3][j]};
+  } else if constexpr (RBC == 2) {
+    // Dword d of K-tile t holds rows 2d (low half) and 2d+1 (high half).
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        out[j][w] = (int)__builtin_amdgcn_perm((uint32_t)in[2 * w + 1][j >> 1],
+                                               (uint32_t)in[2 * w][j >> 1], sel);
+      }
+    }
+  } else {
+    out[0] = in[0];
+  }
+}
+
+// Workgroup -> output block. Consecutive workgroup ids go round-robin to the
+// 8 XCDs, each with its own L2; give every XCD a contiguous share of the
+// blocks and walk that share in bands of `band` block rows so that the
+// workgroups resident on one XCD at a time reuse each other's panels.
+__device__ __forceinline__ void block_of_workgroup(uint32_t wg, const Args& a,
+                                                   int* bm, int* bn) {
+  const uint32_t total = (uint32_t)a.grid_m * (uint32_t)a.grid_n;
+  const uint32_t per_xcd = (total + 7) / 8;
+  uint32_t id = (wg & 7) * per_xcd + (wg >> 3);
+  if (id >= total || (total & 7)) id = wg;  // uneven split: plain order
+  const uint32_t band_blocks = a.band * (uint32_t)a.grid_n;
+  const uint32_t b = id / band_blocks;
+  const uint32_t in_band = id - b * band_blocks;
+  const uint32_t rows = min(a.band, (uint32_t)a.grid_m - b * a.band);
+  const uint32_t col = in_band / rows;
+  *bm = (int)(b * a.band + (in_band - col * rows));
+  *bn = (int)col;
+}
+
+// TM x TN accumulator blocks per wave, WGM x WGN waves per workgroup, NKK MFMA
+// K-groups per pipeline step. PIPE 0: two LDS stages, loads one step ahead.
+// PIPE 1: three LDS stages, loads three steps ahead, fragments one step ahead.
+// RBC: 16 = row bytes >= 16 (direct), 8/4/2 = regrouping loaders.
+template <Elem E, int RBC, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>
+__global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
+  using TT = ElemTraits<E>;
+  using Acc = typename TT::Acc;
+  using Scalar = typename TT::Scalar;
+  constexpr int NW = WGM * WGN;
+  constexpr int HALVES = TT::kHalves;
+  constexpr int NCHB = NKK * HALVES;       // groups of 4 chunks per step
+  constexpr int NCH = NCHB * 4;            // 16-byte chunks per row per step
+  constexpr int KS = NCH * 16;             // bytes of K per row per step
+  constexpr int BM = WGM * TM * 16;
+  constexpr int BN = WGN * TN * 16;
+  constexpr int R = RBC >= 16 ? 1 : 16 / RBC;
+  // A loader block is 64 units (one per lane); a unit is R loads + R stores.
+  constexpr int BLOCKS_A = BM * NCH / R / 64;
+  // PIPE 2 keeps only the LHS in LDS; RHS fragments come straight from global.
+  constexpr int BLOCKS = (PIPE == 2 ? BM : BM + BN) * NCH / R / 64;
+  constexpr int NU = (BLOCKS + NW - 1) / NW;
+  constexpr int IMAGE_A = BM * KS;
+  constexpr int STAGE = (PIPE == 2 ? BM : BM + BN) * KS;
+  static_assert((BM * NCH / R) % 64 == 0 && (BN * NCH / R) % 64 == 0, "block split");
+  // When the blocks do not divide evenly over the waves, the surplus (wave, i)
+  // slots are idle: they load from a valid address and skip the store.
+  constexpr bool EVEN = BLOCKS % NW == 0;
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN;
+  const int wn = wave - wm * WGN;
+  int wg_m, wg_n;
+  block_of_workgroup(blockIdx.x, a, &wg_m, &wg_n);
+  const int pm0 = wg_m * a.bpm;  // first LHS panel of this workgroup
+  const int pn0 = wg_n * a.bpn;
+  const int lrb = a.lrb;
+  const int kts_per_step = KS >> lrb;
+  const uint32_t q = lane >> 4, r = lane & 15;
+
+  // ---- loader set-up: per-unit constants --------------------------------
+  // Operand choice, base pointer and strides depend on (wave, i) only and live
+  // in scalar registers; per lane there is one 32-bit offset per unit.
+  const char* sbase[NU];
+  uint32_t voff[NU];     // byte offset of the unit's first piece at step 0
+  uint32_t sstep[NU];    // bytes to advance per K step
+  uint32_t skt[NU];      // bytes between consecutive loads of a unit
+  int32_t kt0[NU];       // K-tile index of the first load at step 0
+  uint32_t loff[NU];     // LDS offset (within a stage) of the unit's first store
+#pragma unroll
+  for (int i = 0; i < NU; ++i) {
+    const int blk = wave + i * NW;
+    const bool is_b = blk >= BLOCKS_A;
+    const int xblk = is_b ? blk - BLOCKS_A : blk;
+    const int X0 = is_b ? a.N0 : a.M0;
+    const int X1 = is_b ? a.N1 : a.M1;
+    const int px0 = is_b ? pn0 : pm0;
+    const int bpx = is_b ? a.bpn : a.bpm;
+    const int64_t xstride = is_b ? a.rhs_stride : a.lhs_stride;
+    const uint32_t image = is_b ? IMAGE_A : 0;
+    const uint32_t kt_bytes = (uint32_t)X0 << lrb;  // one K-tile of the panel
+    sbase[i] = (is_b ? a.rhs : a.lhs) + (int64_t)px0 * xstride;
+    sstep[i] = (uint32_t)kts_per_step * kt_bytes;
+    int pl;
+    if constexpr (RBC >= 16) {
+      // Block = (row block, chunk group); lane (q, r) owns LDS slot `lane` and
+      // fetches the piece that belongs there: row r of the block, chunk 4*cb+q.
+      const int rbk = xblk / NCHB, cb = xblk - rbk * NCHB;
+      const uint32_t row = (uint32_t)rbk * 16 + r;
+      pl = (int)(row / (uint32_t)X0);
+      const uint32_t m0 = row - (uint32_t)pl * X0;
+      const uint32_t kb = (uint32_t)(cb * 4 + q) * 16;  // K byte of the chunk
+      const uint32_t ktl = kb >> lrb;
+      kt0[i] = (int32_t)ktl;
+      voff[i] = (uint32_t)pl * (uint32_t)xstride + ktl * kt_bytes + (m0 << lrb) +
+                (kb & ((1u << lrb) - 1));
+      skt[i] = 0;
+      loff[i] = image + (uint32_t)xblk * 1024 + lane * 16;
+    } else {
+      // Units in order [panel][chunk g][row group]; the unit's R loads read
+      // K-tiles g, g + NCH, g + 2*NCH, ... so that one load instruction covers
+      // NCH consecutive K-tiles of a panel.
+      const uint32_t u = (uint32_t)xblk * 64 + lane;
+      const uint32_t groups = (uint32_t)X0 / R;
+      const uint32_t t1 = u / groups;
+      const uint32_t mg = u - t1 * groups;
+      pl = (int)(t1 / NCH);
+      const uint32_t g = t1 - (uint32_t)pl * NCH;
+      kt0[i] = (int32_t)g;
+      voff[i] = (uint32_t)pl * (uint32_t)xstride + g * kt_bytes + mg * 16;
+      skt[i] = NCH * kt_bytes;
+      const uint32_t row = (uint32_t)pl * X0 + mg * R;  // first of R rows
+      const uint32_t rr = row & 15;  // R divides 16: the R rows share a block
+      // Slot of row rr + j is (rr + j) ^ mask; R <= 8 and rr % R == 0, so j
+      // only touches the low bits and the store applies j ^ ... itself.
+      loff[i] = image + (((row >> 4) * NCHB + (g >> 2)) * 64 + (g & 3) * 16) * 16 +
+                ((rr & 8) | ((rr & 7) ^ swizzle_mask(g, rr >> 3))) * 16;
+    }
+    // Units outside the problem read from the start of the first panel.
+    if (!(pl < bpx && px0 + pl < X1)) voff[i] = 0;
+    if (!EVEN && blk >= BLOCKS) {
+      sbase[i] = a.lhs + (int64_t)pm0 * a.lhs_stride;
+      voff[i] = 0;
+      sstep[i] = 0;
+      skt[i] = 0;
+    }
+
+  }
+
+  // ---- reader set-up ------------------------------------------------------
+  uint32_t rd_slot[NCHB];
+#pragma unroll
+  for (int cb = 0; cb < NCHB; ++cb) {
+    const uint32_t mask = RBC >= 16 ? 0u : swizzle_mask(cb * 4 + q, r >> 3);
+    rd_slot[cb] = (q * 16 + (r ^ mask)) * 16;
+  }
+  const uint32_t rd_a = (uint32_t)(wm * TM) * NCHB * 1024;
+  const uint32_t rd_b = IMAGE_A + (uint32_t)(wn * TN) * NCHB * 1024;
+
+  // ---- accumulators -------------------------------------------------------
+  // Lane (q, c = r) of block (tm, tn) holds rows 4q..4q+3, column c.
+  Acc acc[TM][TN];
+  auto for_each_output = [&](auto f) {
+    // The lane coordinates pass through an empty asm so that the address
+    // arithmetic of the prologue (ACCUMULATE loads) and of the epilogue
+    // (stores) is not shared: shared, it would stay live in ~80 registers
+    // across the whole K loop.
+    uint32_t oq = q, orr = r;
+    asm volatile("" : "+v"(oq), "+v"(orr));
+    const char* out_base = a.out + (int64_t)pm0 * a.out_stride +
+                           (int64_t)pn0 * a.M0 * a.N0 * 4;
+    uint32_t col_off[TN];
+    bool col_ok[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int col = (wn * TN + tn) * 16 + (int)orr;
+      const int pl = col / a.N0, n0 = col - pl * a.N0;
+      col_ok[tn] = pl < a.bpn && pn0 + pl < a.N1;
+      col_off[tn] = (uint32_t)pl * (uint32_t)(a.M0 * a.N0 * 4) + (uint32_t)n0 * 4;
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int row = (wm * TM + tm) * 16 + 4 * (int)oq + e;
+        const int pl = row / a.M0, m0 = row - pl * a.M0;
+        const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * 4);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+          if (row_ok && col_ok[tn]) {
+            f(tm, tn, e, reinterpret_cast<Scalar*>(const_cast<char*>(out_base) + (row_off + col_off[tn])));
+          }
+        }
+        // Keep the unrolled rows from being hoisted together: that would
+        // hold one address pair per output element live at once.
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
+  if (a.accumulate) {
+    for_each_output([&](int tm, int tn, int e, Scalar* p) { acc[tm][tn][e] = *p; });
+  }
+
+  // ---- pipeline -----------------------------------------------------------
+  // Loads are unconditional in the steady state: units outside the problem
+  // read (valid) bytes of the workgroup's first panel, and what they bring
+  // only ever reaches accumulator rows or columns that are never stored.
+  // `tail` marks the one step in which K-tiles past K1 must read as zero.
+  auto load_piece = [&](int i, uint32_t off) {
+    return *reinterpret_cast<const v4i*>(sbase[i] + off);
+  };
+  auto load_global = [&](v4i (&dst)[NU][R], int step, bool tail) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const uint32_t off = voff[i] + (uint32_t)step * sstep[i];
+      const int kt = step * kts_per_step + kt0[i];
+#pragma unroll
+      for (int t = 0; t < R; ++t) {
+        if (!tail) {
+          dst[i][t] = load_piece(i, off + t * skt[i]);
+        } else {
+          const bool ok = (kt + t * NCH) < a.K1;
+          const v4i v = load_piece(i, ok ? off + t * skt[i] : 0u);
+          dst[i][t] = ok ? v : v4i{0, 0, 0, 0};
+        }
+      }
+    }
+  };
+  auto store_lds = [&](const v4i (&src)[NU][R], uint32_t stage_off) {
+    char* base = lds + stage_off;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      if (!EVEN && wave + i * NW >= BLOCKS) continue;
+      if constexpr (RBC >= 16) {
+        *reinterpret_cast<v4i*>(base + loff[i]) = src[i][0];
+      } else {
+        v4i outp[R];
+        regroup<RBC>(src[i], outp);
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          // Row rr + j sits at slot low bits (rr ^ mask) ^ j.
+          *reinterpret_cast<v4i*>(base + (loff[i] ^ (uint32_t)(j * 16))) = outp[j];
+        }
+      }
+    }
+  };
+  auto read_frags = [&](v4i (&fa)[TM][HALVES], v4i (&fb)[TN][HALVES], uint32_t stage_off,
+                        int kk) {
+    const char* base = lds + stage_off;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        fa[tm][h] = *reinterpret_cast<const v4i*>(
+            base + rd_a + (tm * NCHB + kk * HALVES + h) * 1024 + rd_slot[kk * HALVES + h]);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        fb[tn][h] = *reinterpret_cast<const v4i*>(
+            base + rd_b + (tn * NCHB + kk * HALVES + h) * 1024 + rd_slot[kk * HALVES + h]);
+  };
+  auto mfmas = [&](const v4i (&fa)[TM][HALVES], const v4i (&fb)[TN][HALVES]) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fa[tm], fb[tn], acc[tm][tn]);
+  };
+  const int last = a.steps - 1;
+  const bool has_tail = a.tail != 0;
+
+  if constexpr (PIPE == 0) {
+    // Two LDS stages; each step: issue next global loads, compute, store, barrier.
+    v4i regs[NU][R];
+    load_global(regs, 0, has_tail && last == 0);
+    store_lds(regs, 0);
+    __syncthreads();
+    for (int s = 0; s < a.steps; ++s) {
+      const uint32_t cur = (s & 1) * STAGE;
+      if (s < last) {
+        if (has_tail && s + 1 == last) load_global(regs, s + 1, true);
+        else load_global(regs, s + 1, false);
+      }
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        v4i fa[TM][HALVES], fb[TN][HALVES];
+        read_frags(fa, fb, cur, kk);
+        mfmas(fa, fb);
+      }
+      if (s < last) store_lds(regs, cur ^ STAGE);
+      __syncthreads();
+    }
+  } else if constexpr (PIPE == 1) {
+    // Three LDS stages, two register sets. In iteration s a wave runs the
+    // MFMAs of step s row by row (tm) and, between rows, issues everything
+    // that does not depend on them: the global loads of step s+3, the LDS
+    // stores of step s+2 (loaded during iteration s-1) into stage (s+2)%3,
+    // the LHS fragments of the next row, and one RHS fragment of step s+1
+    // from stage (s+1)%3. K must be a whole number of steps here (no tail).
+    static_assert(NKK == 1, "pipelined variant steps one MFMA K-group at a time");
+    static_assert(TM % 2 == 0, "LHS fragment slots alternate by row parity");
+    constexpr int NP = NU * R;  // 16-byte pieces per thread per step
+    v4i regs[2][NU][R];
+    v4i fa[2][HALVES], fb[2][TN][HALVES];
+    auto read_a = [&](v4i (&dst)[HALVES], uint32_t stage_off, int tm) {
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        dst[h] = *reinterpret_cast<const v4i*>(lds + stage_off + rd_a +
+                                               (tm * NCHB + h) * 1024 + rd_slot[h]);
+    };
+    auto read_b = [&](v4i (&dst)[HALVES], uint32_t stage_off, int tn) {
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        dst[h] = *reinterpret_cast<const v4i*>(lds + stage_off + rd_b +
+                                               (tn * NCHB + h) * 1024 + rd_slot[h]);
+    };
+    load_global(regs[0], 0, false);
+    store_lds(regs[0], 0);
+    load_global(regs[0], min(1, last), false);
+    store_lds(regs[0], STAGE);
+    load_global(regs[1], min(2, last), false);
+    __syncthreads();
+    read_a(fa[0], 0, 0);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) read_b(fb[0][tn], 0, tn);
+    uint32_t st_cur = 0, st_next = STAGE, st_write = 2 * STAGE;
+    auto iteration = [&](int s, auto parity) {
+      constexpr int P = decltype(parity)::value;
+      const int ld_step = min(s + 3, last);
+      v4i outp[NU][R];
+      if constexpr (RBC < 16) {
+#pragma unroll
+        for (int i = 0; i < NU; ++i) regroup<RBC>(regs[P ^ 1][i], outp[i]);
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        // Stores of step s+2 and loads of step s+3, an even share per row.
+#pragma unroll
+        for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k) {
+          const int i = k / R, j = k % R;
+          if (!EVEN && wave + i * NW >= BLOCKS) continue;
+          char* dst = lds + st_write + (RBC >= 16 ? loff[i] : (loff[i] ^ (uint32_t)(j * 16)));
+          *reinterpret_cast<v4i*>(dst) = RBC >= 16 ? regs[P ^ 1][i][0] : outp[i][j];
+        }
+#pragma unroll
+        for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k) {
+          const int i = k / R, t = k % R;
+          regs[P][i][t] = load_piece(i, voff[i] + (uint32_t)ld_step * sstep[i] + t * skt[i]);
+        }
+        // Fragments: LHS of the next row (or of row 0 of step s+1), and this
+        // row's share of the RHS fragments of step s+1.
+        if (tm + 1 < TM) read_a(fa[(tm + 1) & 1], st_cur, tm + 1);
+        else read_a(fa[0], st_next, 0);
+#pragma unroll
+        for (int tn = tm * TN / TM; tn < (tm + 1) * TN / TM; ++tn)
+          read_b(fb[P ^ 1][tn], st_next, tn);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = TT::mfma(fa[tm & 1], fb[P][tn], acc[tm][tn]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();
+      const uint32_t t = st_cur;
+      st_cur = st_next;
+      st_next = st_write;
+      st_write = t;
+    };
+    int s = 0;
+    for (; s + 1 < a.steps; s += 2) {
+      iteration(s, std::integral_constant<int, 0>{});
+      iteration(s + 1, std::integral_constant<int, 1>{});
+    }
+    if (s < a.steps) iteration(s, std::integral_constant<int, 0>{});
+  }
+  else if constexpr (PIPE == 2) {
+    // LHS through three LDS stages as in PIPE 1; RHS fragments are loaded by
+    // each wave straight from global memory into registers, one step ahead:
+    // a 16-byte piece of a tile row IS the lane's MFMA operand when RB >= 16.
+    // This halves the LDS traffic per MFMA, which is what bounds PIPE 1. The
+    // waves that share a column block re-read the same lines from L1/L2.
+    static_assert(RBC >= 16, "register-direct RHS needs row bytes >= 16");
+    static_assert(NKK == 1 && TM % 2 == 0, "see PIPE 1");
+    constexpr int NP = NU;  // 16-byte LHS pieces per thread per step
+    v4i regs[2][NU][R];
+    v4i fa[2][HALVES], fb[2][TN][HALVES];
+    const char* sbase_b = a.rhs + (int64_t)pn0 * a.rhs_stride;
+    const uint32_t kt_bytes_b = (uint32_t)a.N0 << lrb;
+    const uint32_t sstep_b = (uint32_t)kts_per_step * kt_bytes_b;
+    uint32_t voff_b[TN][HALVES];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const uint32_t row = (uint32_t)(wn * TN + tn) * 16 + r;
+      const uint32_t pl = row / (uint32_t)a.N0;
+      const uint32_t n0 = row - pl * a.N0;
+      const bool ok = (int)pl < a.bpn && pn0 + (int)pl < a.N1;
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h) {
+        const uint32_t kb = (uint32_t)(h * 4 + q) * 16;
+        voff_b[tn][h] = ok ? pl * (uint32_t)a.rhs_stride + (kb >> lrb) * kt_bytes_b +
+                                 (n0 << lrb) + (kb & ((1u << lrb) - 1))
+                           : 0u;
+      }
+    }
+    auto load_b = [&](v4i (&dst)[HALVES], int tn, int step) {
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        dst[h] = *reinterpret_cast<const v4i*>(sbase_b + (voff_b[tn][h] + (uint32_t)step * sstep_b));
+    };
+    auto read_a = [&](v4i (&dst)[HALVES], uint32_t stage_off, int tm) {
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        dst[h] = *reinterpret_cast<const v4i*>(lds + stage_off + rd_a +
+                                               (tm * NCHB + h) * 1024 + rd_slot[h]);
+    };
+    load_global(regs[0], 0, false);
+    store_lds(regs[0], 0);
+    load_global(regs[0], min(1, last), false);
+    store_lds(regs[0], STAGE);
+    load_global(regs[1], min(2, last), false);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) load_b(fb[0][tn], tn, 0);
+    __syncthreads();
+    read_a(fa[0], 0, 0);
+    uint32_t st_cur = 0, st_next = STAGE, st_write = 2 * STAGE;
+    auto iteration = [&](int s, auto parity) {
+      constexpr int P = decltype(parity)::value;
+      const int ld_step = min(s + 3, last);
+      const int b_step = min(s + 1, last);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int tn = tm * TN / TM; tn < (tm + 1) * TN / TM; ++tn) {
+#ifndef UK_DBG_NO_B
+          load_b(fb[P ^ 1][tn], tn, b_step);
+#endif
+        }
+#pragma unroll
+        for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k) {
+#ifndef UK_DBG_NO_A_STORE
+          *reinterpret_cast<v4i*>(lds + st_write + loff[k]) = regs[P ^ 1][k][0];
+#endif
+#ifndef UK_DBG_NO_A_LOAD
+          regs[P][k][0] = load_piece(k, voff[k] + (uint32_t)ld_step * sstep[k]);
+#endif
+        }
+#ifndef UK_DBG_NO_A_READ
+        if (tm + 1 < TM) read_a(fa[(tm + 1) & 1], st_cur, tm + 1);
+        else read_a(fa[0], st_next, 0);
+#endif
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = TT::mfma(fa[tm & 1], fb[P][tn], acc[tm][tn]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();
+      const uint32_t t = st_cur;
+      st_cur = st_next;
+      st_next = st_write;
+      st_write = t;
+    };
+    int s = 0;
+    for (; s + 1 < a.steps; s += 2) {
+      iteration(s, std::integral_constant<int, 0>{});
+      iteration(s + 1, std::integral_constant<int, 1>{});
+    }
+    if (s < a.steps) iteration(s, std::integral_constant<int, 0>{});
+  }
+
+  // ---- epilogue -----------------------------------------------------------
+  for_each_output([&](int tm, int tn, int e, Scalar* p) { *p = acc[tm][tn][e]; });
+}
+
+template <Elem E, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>
+struct Shape {
+  static constexpr int NCH = NKK * ElemTraits<E>::kHalves * 4;
+  static constexpr int KS = NCH * 16;
+  static constexpr int BM = WGM * TM * 16;
+  static constexpr int BN = WGN * TN * 16;
+  static constexpr size_t kLdsBytes =
+      (PIPE ? 3 : 2) * (size_t)(PIPE == 2 ? BM : BM + BN) * KS;
+};
+
+}  // namespace uk_mfma
+
+#endif  // IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_

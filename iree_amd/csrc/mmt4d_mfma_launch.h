@@ -1,0 +1,164 @@
+// Host-side selection and launch of the MFMA mmt4d kernels for one element
+// type. Included by one translation unit per element type so that the kernel
+// instantiations compile in parallel.
+#ifndef IREE_UK_AMD_MMT4D_MFMA_LAUNCH_H_
+#define IREE_UK_AMD_MMT4D_MFMA_LAUNCH_H_
+
+#include <hip/hip_runtime.h>
+
+#include "mmt4d_mfma_kernel.h"
+#include "uk_device_common.h"
+#include "uk_hip_abi.h"
+
+namespace uk_mfma {
+
+// What the dispatcher hands to the per-type launcher: the problem in bytes.
+struct Problem {
+  const char* lhs;
+  const char* rhs;
+  char* out;
+  int64_t lhs_stride, rhs_stride, out_stride;  // bytes
+  int32_t M1, N1, K1, M0, N0;
+  int32_t rb, lrb;  // bytes per tile row and its log2
+  bool accumulate;
+};
+
+// Launches one kernel variant over K-tiles [kt_begin, kt_begin + kt_count).
+// Returns a HIP status, or -1 if the variant cannot serve the shape.
+template <Elem E, int RBC, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>
+int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate,
+                   hipStream_t stream) {
+  using SH = Shape<E, TM, TN, WGM, WGN, NKK, PIPE>;
+  constexpr int R = RBC >= 16 ? 1 : 16 / RBC;
+  if (p.rb > SH::KS) return -1;                       // a tile row must fit one step
+  if (p.M0 > SH::BM || p.N0 > SH::BN) return -1;      // at least one whole panel
+  if (p.M0 % R || p.N0 % R) return -1;                // pieces hold whole rows
+  Args a;
+  const int64_t kt_bytes_m = (int64_t)p.M0 << p.lrb, kt_bytes_n = (int64_t)p.N0 << p.lrb;
+  a.lhs = p.lhs + kt_begin * kt_bytes_m;
+  a.rhs = p.rhs + kt_begin * kt_bytes_n;
+  a.out = p.out;
+  a.lhs_stride = p.lhs_stride;
+  a.rhs_stride = p.rhs_stride;
+  a.out_stride = p.out_stride;
+  a.M1 = p.M1; a.N1 = p.N1; a.K1 = kt_count;
+  a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
+  a.bpm = SH::BM / p.M0;
+  a.bpn = SH::BN / p.N0;
+  const int64_t grid_m = uk::ceil_div(p.M1, a.bpm), grid_n = uk::ceil_div(p.N1, a.bpn);
+  if (grid_m * grid_n >= (1ll << 31)) return -1;
+  a.grid_m = (int32_t)grid_m;
+  a.grid_n = (int32_t)grid_n;
+  const int64_t k_bytes = (int64_t)kt_count << p.lrb;
+  a.steps = (int32_t)uk::ceil_div(k_bytes, SH::KS);
+  if (a.steps < 1) a.steps = 1;
+  a.tail = (k_bytes % SH::KS) != 0;
+  if (PIPE != 0 && (a.tail || kt_count == 0)) return -1;
+  a.accumulate = accumulate;
+  a.band = 4;
+  // 32-bit offsets inside a workgroup's share of each operand.
+  const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
+  const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
+  const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.N1 * p.M0 * p.N0 * 4;
+  if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31)) return -1;
+  auto kernel = mmt4d_mfma_kernel<E, RBC, TM, TN, WGM, WGN, NKK, PIPE>;
+  if (SH::kLdsBytes > 64 * 1024) {
+    // Raising the dynamic LDS limit is a per-function setting; do it once.
+    static hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+        (int)SH::kLdsBytes);
+    if (attr != hipSuccess) return (int)attr;
+  }
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)(grid_m * grid_n)), dim3(WGM * WGN * 64),
+                     SH::kLdsBytes, stream, a);
+  return (int)hipGetLastError();
+}
+
+// Number of workgroups a BM x BN blocking gives for the problem.
+inline int64_t workgroups(const Problem& p, int BM, int BN) {
+  const int bpm = BM / p.M0, bpn = BN / p.N0;
+  if (bpm < 1 || bpn < 1) return 0;
+  return uk::ceil_div(p.M1, bpm) * uk::ceil_div(p.N1, bpn);
+}
+
+// Variant choice for row-bytes class RBC:
+//   big   256x256 workgroup tile, 8 waves of 128x64, software-pipelined
+//         (register-direct RHS when RB >= 16): needs K in whole steps, the
+//         remainder of K (if any) is a second, accumulating launch;
+//   mid   128x128, 4 waves, any K;
+//   small 64x64, 4 waves, any K: for problems with too few 128x128 blocks to
+//         occupy the 256 CUs;
+// `forced` (1 big, 2 mid, 3 small, 4 skinny; 0 = choose) overrides the size
+// heuristic for tests and tuning.
+//   skinny 32 rows x 64 columns: M-thin (decode-shaped) problems, which are
+//         bound by streaming the RHS and want every CU pulling on it.
+template <Elem E, int RBC>
+int launch_class(const Problem& p, int forced, hipStream_t stream, const char** name) {
+  constexpr int H = ElemTraits<E>::kHalves;
+  constexpr int NKK2 = 2 / H;             // 128 bytes of K per step
+  constexpr int BIG_PIPE = RBC >= 16 ? 2 : 1;
+  constexpr int BIG_KS = 64 * H;
+  const int64_t rows_m = (int64_t)p.M1 * p.M0;
+  int choice;
+  if (forced >= 1 && forced <= 4) {
+    choice = forced;
+  } else if (rows_m <= 32 && workgroups(p, 32, 64) >= 1) {
+    choice = 4;
+  } else if (workgroups(p, 256, 256) >= 192) {
+    choice = 1;
+  } else if (workgroups(p, 128, 128) >= 192) {
+    choice = 2;
+  } else {
+    choice = 3;
+  }
+  if (choice == 1) {
+    const int kts_per_step = BIG_KS >> p.lrb;
+    const int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
+    if (kt_main > 0) {
+      int st = launch_variant<E, RBC, 8, 4, 2, 4, 1, BIG_PIPE>(p, 0, kt_main, p.accumulate, stream);
+      if (st == 0) {
+        *name = RBC >= 16 ? "mmt4d_mfma_256x256_rhs_direct" : "mmt4d_mfma_256x256_regroup";
+        if (kt_main == p.K1) return 0;
+        return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+      }
+      if (st > 0) return st;
+    }
+    choice = 2;
+  }
+  if (choice == 4) {
+    // With 2-byte rows a 16-byte piece spans 8 rows and 32 rows do not fill a
+    // loader block; that combination takes the 64x64 variant.
+    if constexpr (RBC != 2) {
+      int st = launch_variant<E, RBC, 2, 1, 1, 4, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
+      if (st >= 0) { *name = "mmt4d_mfma_32x64"; return st; }
+    }
+    choice = 3;
+  }
+  if (choice == 2) {
+    int st = launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
+    if (st >= 0) { *name = "mmt4d_mfma_128x128"; return st; }
+  }
+  int st = launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
+  if (st >= 0) { *name = "mmt4d_mfma_64x64"; return st; }
+  st = launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
+  if (st >= 0) *name = "mmt4d_mfma_128x128";
+  return st;
+}
+
+template <Elem E>
+int launch_elem(const Problem& p, int forced, hipStream_t stream, const char** name) {
+  if constexpr (E == Elem::kF8) {
+    return p.rb >= 16 ? launch_class<E, 16>(p, forced, stream, name) : -1;
+  } else {
+    switch (p.rb) {
+      case 2: return launch_class<E, 2>(p, forced, stream, name);
+      case 4: return launch_class<E, 4>(p, forced, stream, name);
+      case 8: return launch_class<E, 8>(p, forced, stream, name);
+      default: return launch_class<E, 16>(p, forced, stream, name);
+    }
+  }
+}
+
+}  // namespace uk_mfma
+
+#endif  // IREE_UK_AMD_MMT4D_MFMA_LAUNCH_H_

@@ -64,20 +64,26 @@ MFMA_TILES = [
 def _mfma_shapes(M0, N0, K0, bits):
     kb = K0 * bits // 8  # bytes of K per tile row
     k_small = max(1, 32 // kb)
-    k_big = max(3, 700 // kb)
+    k_big = max(3, 700 // kb)          # several pipeline steps plus a remainder
+    k_whole = max(1, 5 * 128 // kb)    # a whole number of steps, odd count
     m_wg = max(1, 256 // M0)
     n_wg = max(1, 256 // N0)
     return ((1, 1, 1), (1, 1, k_small), (2, 3, k_big), (m_wg + 1, 1, k_small + 1),
             (1, n_wg + 3, 5), (m_wg + 2, n_wg + 1, k_big // 2 + 1), (0, 2, 2),
-            (2, 2, 0))
+            (2, 2, 0), (m_wg + 1, 2 * n_wg + 1, k_whole), (3, 2, 2 * k_whole))
 
 
+# 0 = let the library choose by problem size; 1..4 = force the 256x256,
+# 128x128, 64x64 and 32x64 workgroup shapes (a forced shape that cannot serve a
+# case falls through to the next one that can).
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("n", range(len(MFMA_TILES)))
-def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n):
+def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu
     tf, M0, N0, K0 = MFMA_TILES[n]
     if not lib.mmt4d_info(M0, N0, K0, tf):
         pytest.skip("no MFMA kernel for this tile shape; covered by the generic kernel")
+    lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
     bits = uk.MMT4D_TYPE_BITS[tf][0]
     # Loose strides and offsets in steps of 16 elements: the MFMA kernels need
     # 16-byte aligned panels (anything else goes to the generic kernel, which
@@ -91,7 +97,7 @@ def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n):
         # No generic-fallback flag: only an MFMA kernel may serve these calls.
         got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
         assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
-        if c.M and c.N and not (c.K == 0 and c.flags & uk.MMT4D_ACCUMULATE):
+        if c.M and c.N and c.K:  # K == 0 is a zero fill, left to the generic kernel
             assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
 
 
@@ -113,8 +119,10 @@ def _normal_operand(rng, kind, n, scale=1.0):
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
     (uk.MMT4D_TYPE_F32F32F32, 8, 8, 4)])
 @pytest.mark.parametrize("accumulate", [0, 1])
-def test_mmt4d_float_tolerance_on_normal_inputs(gpu, oracle, tf, M0, N0, K0, accumulate):
+@pytest.mark.parametrize("variant", [0, 1])
+def test_mmt4d_float_tolerance_on_normal_inputs(gpu, oracle, tf, M0, N0, K0, accumulate, variant):
     lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
     lk = T.MMT4D_KINDS[tf][0]
     rng = np.random.default_rng(21)
     M, N, K = 9, 11, max(1, 2048 // K0)
