@@ -18,6 +18,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <utility>
 
 #include "uk_device_common.h"
@@ -153,6 +154,11 @@ struct TiledArgs {
   FastDiv div_tile_grans;           // granules per tile
   FastDiv div_tile_row_grans;
   FastDiv div_tile0;
+  FastDiv div_tile_bytes;
+  uint32_t nblk0;                   // blocks along dim 0
+  uint32_t lds_buf_bytes;           // one LDS buffer of the streaming kernels
+  uint32_t mat_stride0_bytes32;     // == mat_stride0_bytes when it fits
+  uint32_t sl0_bytes32, sl1_bytes32;
 };
 
 template <int N> struct Bytes;
@@ -413,6 +419,264 @@ __global__ __launch_bounds__(kThreads) void unpack_tiled_kernel(TiledArgs a) {
   }
 }
 
+
+//===----------------------------------------------------------------------===//
+// Streaming (persistent) tiled kernels.
+//
+// Same two-phase LDS scheme as the kernels above, restructured so that the
+// per-byte instruction count is small enough for HBM to be the bound:
+//   * a workgroup walks many blocks; everything that depends only on the
+//     thread and the block shape (global offsets inside a block, LDS offsets
+//     of every granule) is computed once, before the walk;
+//   * all loads of a phase are issued before any of their data is used;
+//   * LDS is double-buffered, one barrier per block, so the stores of block b
+//     and the loads of block b+1 are in flight together;
+//   * global accesses are non-temporal (every byte is touched once).
+// Blocks on the ragged edge of the matrix take a slower, bounds-checked path.
+//===----------------------------------------------------------------------===//
+
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+template <int N> struct GBytes;
+template <> struct GBytes<4> { using type = uint32_t; };
+template <> struct GBytes<8> { using type = v2u; };
+template <> struct GBytes<16> { using type = v4u; };
+
+template <int N>
+__device__ __forceinline__ typename GBytes<N>::type gload(const char* gptr) {
+  using T = typename GBytes<N>::type;
+  return __builtin_nontemporal_load(reinterpret_cast<const T*>(gptr));
+}
+template <int N>
+__device__ __forceinline__ void gstore(char* gptr, typename GBytes<N>::type v) {
+  using T = typename GBytes<N>::type;
+  __builtin_nontemporal_store(v, reinterpret_cast<T*>(gptr));
+}
+
+constexpr uint32_t kStreamBlockBytes = 16384;  // LDS bytes per buffer, at most
+
+struct StreamTables1 {  // 2-D side items of one thread
+  uint32_t goff;        // byte offset inside the block's 2-D window
+  uint32_t loff;        // LDS byte offset
+};
+
+// Items of the 2-D side: vector idx of the block -> row r, vector v.
+template <int MV>
+__device__ __forceinline__ void mat_item(const TiledArgs& a, uint32_t idx,
+                                         uint32_t* r, uint32_t* cb) {
+  uint32_t v;
+  a.div_row_vecs.divmod(idx, *r, v);
+  *cb = v * MV;
+}
+
+// Items of the tiled side: vector idx of the block -> run, tile, byte in tile.
+template <int VEC>
+__device__ __forceinline__ void tiled_item(const TiledArgs& a, uint32_t idx,
+                                           uint32_t* run, uint32_t* t,
+                                           uint32_t* in_tile, uint32_t* tl0,
+                                           uint32_t* tl1) {
+  uint32_t v;
+  a.div_run_vecs.divmod(idx, *run, v);
+  const uint32_t pos = v * VEC;
+  *t = a.div_tile_bytes.div(pos);
+  *in_tile = pos - *t * a.tile_bytes;
+  *tl0 = a.transpose_outer ? *t : *run;
+  *tl1 = a.transpose_outer ? *run : *t;
+}
+
+template <int N>
+__device__ __forceinline__ void lds_store_pieces(char* dst, typename GBytes<N>::type v,
+                                                 uint32_t piece) {
+  if (piece >= N) {
+    *reinterpret_cast<typename GBytes<N>::type*>(dst) = v;
+  } else {
+    __attribute__((aligned(16))) char tmp[N];
+    *reinterpret_cast<typename GBytes<N>::type*>(tmp) = v;
+    store_pieces<N>(dst, tmp, piece);
+  }
+}
+template <int N>
+__device__ __forceinline__ typename GBytes<N>::type lds_load_pieces(const char* src,
+                                                                     uint32_t piece) {
+  if (piece >= N) return *reinterpret_cast<const typename GBytes<N>::type*>(src);
+  __attribute__((aligned(16))) char tmp[N];
+  load_pieces<N>(tmp, src, piece);
+  return *reinterpret_cast<const typename GBytes<N>::type*>(tmp);
+}
+
+template <int G, int VEC, int MV, bool UNPACK>
+__global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  constexpr int N1 = kStreamBlockBytes / MV / kThreads;   // 2-D side items per thread
+  constexpr int N2 = kStreamBlockBytes / VEC / kThreads;  // tiled side items per thread
+  constexpr int NG = VEC / G;                             // granules per tiled vector
+  using MatVec = typename GBytes<MV>::type;
+  using TileVec = typename GBytes<VEC>::type;
+  using Gran = typename GBytes<G < 4 ? 4 : G>::type;  // G >= 4 here (see planner)
+  static_assert(G >= 4, "streaming kernels move granules of at least 4 bytes");
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t total1 = a.block_rows * a.div_row_vecs.d;
+  const uint32_t total2 = a.num_runs * a.run_vecs;
+  const uint32_t piece = a.lds_piece < MV ? a.lds_piece : MV;
+  const uint32_t size1_bytes = a.mat_size1 * a.elem_bytes;
+
+  // ---- per-thread tables (block independent) ----------------------------
+  uint32_t g1off[N1], l1off[N1];
+#pragma unroll
+  for (int i = 0; i < N1; ++i) {
+    uint32_t r, cb;
+    mat_item<MV>(a, tid + i * kThreads, &r, &cb);
+    g1off[i] = r * a.mat_stride0_bytes32 + cb;
+    l1off[i] = r * a.lds_pitch + cb;
+  }
+  uint32_t g2off[N2], l2off[N2][NG];
+#pragma unroll
+  for (int i = 0; i < N2; ++i) {
+    uint32_t run, t, in_tile, tl0, tl1;
+    tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+    g2off[i] = tl0 * a.sl0_bytes32 + tl1 * a.sl1_bytes32 + in_tile;
+    for_each_granule<G, VEC>(a, run, t, in_tile, [&](int k, uint32_t off) { l2off[i][k] = off; });
+  }
+
+  const uint32_t nblocks = a.nblk0 * a.nblk1;
+  uint32_t buf = 0;
+  for (uint32_t blk = blockIdx.x; blk < nblocks; blk += gridDim.x) {
+    const uint32_t blk0 = blk / a.nblk1;
+    const uint32_t blk1 = blk - blk0 * a.nblk1;
+    const uint32_t row_base = blk0 * a.block_rows;
+    const uint32_t col_base_bytes = blk1 * a.block_row_bytes;
+    const char* mat_c = (UNPACK ? a.dst : a.src) + (int64_t)row_base * a.mat_stride0_bytes +
+                        col_base_bytes;
+    const char* tiled_c = (UNPACK ? a.src : a.dst) + (int64_t)(blk0 * a.G0) * a.sl0_bytes +
+                          (int64_t)(blk1 * a.G1) * a.sl1_bytes;
+    char* lbuf = lds + buf * a.lds_buf_bytes;
+    buf ^= 1;
+    // Interior: the whole block lies inside the matrix and the tile grid.
+    const bool interior = row_base + a.block_rows <= a.mat_size0 &&
+                          col_base_bytes + a.block_row_bytes <= size1_bytes &&
+                          (blk0 + 1) * a.G0 <= a.outer0 && (blk1 + 1) * a.G1 <= a.outer1;
+
+    if constexpr (!UNPACK) {
+      // ---- pack phase 1: 2-D rows -> LDS ----
+      if (interior) {
+        MatVec reg[N1];
+#pragma unroll
+        for (int i = 0; i < N1; ++i)
+          if (tid + i * kThreads < total1) reg[i] = gload<MV>(mat_c + g1off[i]);
+#pragma unroll
+        for (int i = 0; i < N1; ++i)
+          if (tid + i * kThreads < total1) lds_store_pieces<MV>(lbuf + l1off[i], reg[i], piece);
+      } else {
+        for (uint32_t idx = tid; idx < total1; idx += kThreads) {
+          uint32_t r, cb;
+          mat_item<MV>(a, idx, &r, &cb);
+          __attribute__((aligned(16))) char reg[MV];
+          const bool row_ok = row_base + r < a.mat_size0;
+          const char* gp = mat_c + (r * a.mat_stride0_bytes32 + cb);
+          const uint32_t es = a.elem_bytes;
+          for (uint32_t b = 0; b < MV; b += es) {
+            const bool ok = row_ok && (col_base_bytes + cb + b) < size1_bytes;
+            if (es == 4) {
+              *reinterpret_cast<uint32_t*>(reg + b) =
+                  ok ? *reinterpret_cast<const uint32_t*>(gp + b) : a.pad32;
+            } else if (es == 2) {
+              *reinterpret_cast<uint16_t*>(reg + b) =
+                  ok ? *reinterpret_cast<const uint16_t*>(gp + b) : (uint16_t)a.pad32;
+            } else {
+              reg[b] = ok ? gp[b] : (char)a.pad32;
+            }
+          }
+          store_pieces<MV>(lbuf + r * a.lds_pitch + cb, reg, piece);
+        }
+      }
+      __syncthreads();
+      // ---- pack phase 2: LDS -> tiled runs ----
+      {
+        TileVec reg[N2];
+#pragma unroll
+        for (int i = 0; i < N2; ++i) {
+          if (tid + i * kThreads < total2) {
+            __attribute__((aligned(16))) char tmp[VEC];
+#pragma unroll
+            for (int k = 0; k < NG; ++k)
+              *reinterpret_cast<Gran*>(tmp + k * G) =
+                  *reinterpret_cast<const Gran*>(lbuf + l2off[i][k]);
+            reg[i] = *reinterpret_cast<const TileVec*>(tmp);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < N2; ++i) {
+          if (tid + i * kThreads < total2) {
+            bool ok = true;
+            if (!interior) {
+              uint32_t run, t, in_tile, tl0, tl1;
+              tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+              ok = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
+            }
+            if (ok) gstore<VEC>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
+          }
+        }
+      }
+    } else {
+      // ---- unpack phase 1: tiled runs -> LDS (scatter by granules) ----
+      {
+        TileVec reg[N2];
+        bool ok[N2];
+#pragma unroll
+        for (int i = 0; i < N2; ++i) {
+          ok[i] = tid + i * kThreads < total2;
+          if (ok[i] && !interior) {
+            uint32_t run, t, in_tile, tl0, tl1;
+            tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+            ok[i] = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
+          }
+          if (ok[i]) reg[i] = gload<VEC>(tiled_c + g2off[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < N2; ++i) {
+          if (ok[i]) {
+            __attribute__((aligned(16))) char tmp[VEC];
+            *reinterpret_cast<TileVec*>(tmp) = reg[i];
+#pragma unroll
+            for (int k = 0; k < NG; ++k)
+              *reinterpret_cast<Gran*>(lbuf + l2off[i][k]) =
+                  *reinterpret_cast<const Gran*>(tmp + k * G);
+          }
+        }
+      }
+      __syncthreads();
+      // ---- unpack phase 2: LDS rows -> 2-D rows ----
+      if (interior) {
+        MatVec reg[N1];
+#pragma unroll
+        for (int i = 0; i < N1; ++i)
+          if (tid + i * kThreads < total1) reg[i] = lds_load_pieces<MV>(lbuf + l1off[i], piece);
+#pragma unroll
+        for (int i = 0; i < N1; ++i)
+          if (tid + i * kThreads < total1) gstore<MV>(const_cast<char*>(mat_c) + g1off[i], reg[i]);
+      } else {
+        const uint32_t es = a.elem_bytes;
+        for (uint32_t idx = tid; idx < total1; idx += kThreads) {
+          uint32_t r, cb;
+          mat_item<MV>(a, idx, &r, &cb);
+          if (row_base + r >= a.mat_size0) continue;
+          __attribute__((aligned(16))) char reg[MV];
+          load_pieces<MV>(reg, lbuf + r * a.lds_pitch + cb, piece);
+          char* gp = const_cast<char*>(mat_c) + (r * a.mat_stride0_bytes32 + cb);
+          for (uint32_t b = 0; b < MV && col_base_bytes + cb + b < size1_bytes; b += es) {
+            if (es == 4) copy_bytes<4>(gp + b, reg + b);
+            else if (es == 2) copy_bytes<2>(gp + b, reg + b);
+            else gp[b] = reg[b];
+          }
+        }
+      }
+    }
+    // No second barrier: the next block uses the other LDS buffer, and its
+    // barrier orders this block's LDS reads before the buffer is reused.
+  }
+}
+
 //===----------------------------------------------------------------------===//
 // Host-side planning.
 //===----------------------------------------------------------------------===//
@@ -420,7 +684,8 @@ __global__ __launch_bounds__(kThreads) void unpack_tiled_kernel(TiledArgs a) {
 struct TiledPlan {
   bool ok = false;
   TiledArgs args;
-  int G = 0, VEC = 0;
+  int G = 0, VEC = 0, MV = 0;
+  bool stream = false;
   uint32_t grid = 0;
   uint32_t lds_bytes = 0;
 };
@@ -521,6 +786,24 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   a.div_tile_grans = FastDiv((uint32_t)(tile_bytes / G));
   a.div_tile_row_grans = FastDiv(a.tile_row_grans);
   a.div_tile0 = FastDiv((uint32_t)v.tile0);
+  a.div_tile_bytes = FastDiv((uint32_t)tile_bytes);
+  a.nblk0 = (uint32_t)nblk0;
+  a.lds_buf_bytes = (uint32_t)((lds_bytes + 255) / 256 * 256);
+  // Streaming kernels: 32-bit offsets inside one block on both sides, granules
+  // of at least 4 bytes, at most 4 granules per vector, block within budget.
+  plan.stream = mat_vec >= 4 && G >= 4 && VEC / G <= 4 &&
+                block_rows * block_row_bytes <= kStreamBlockBytes &&
+                lds_bytes <= 2 * kStreamBlockBytes &&
+                block_rows * std::abs(mat_stride0) * es < (1ll << 31) &&
+                (G0 * std::abs(v.sl0) + G1 * std::abs(v.sl1)) * es < (1ll << 31);
+  plan.MV = mat_vec >= 16 ? 16 : 4;
+  if (plan.stream) {
+    a.mat_vec = (uint32_t)plan.MV;
+    a.div_row_vecs = FastDiv((uint32_t)(block_row_bytes / plan.MV));
+    a.mat_stride0_bytes32 = (uint32_t)(mat_stride0 * es);
+    a.sl0_bytes32 = (uint32_t)(v.sl0 * es);
+    a.sl1_bytes32 = (uint32_t)(v.sl1 * es);
+  }
   plan.G = G;
   plan.VEC = VEC;
   plan.grid = (uint32_t)(nblk0 * nblk1);
@@ -557,6 +840,24 @@ struct UnpackLauncher {
                        dim3(kThreads), plan.lds_bytes, stream, plan.args);
   }
 };
+
+template <bool UNPACK>
+bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
+  // Persistent grid: up to 4 workgroups per CU, two LDS buffers each.
+  const uint32_t nblocks = plan.grid;
+  const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
+  const uint32_t lds = 2 * plan.args.lds_buf_bytes;
+#define UK_CASE(g, vv, mv)                                                          \
+  if (plan.G == g && plan.VEC == vv && plan.MV == mv) {                              \
+    hipLaunchKernelGGL((stream_tiled_kernel<g, vv, mv, UNPACK>), dim3(grid),         \
+                       dim3(kThreads), lds, stream, plan.args);                      \
+    return true;                                                                     \
+  }
+  UK_CASE(16, 16, 16) UK_CASE(8, 16, 16) UK_CASE(4, 16, 16) UK_CASE(4, 4, 16)
+  UK_CASE(16, 16, 4) UK_CASE(8, 16, 4) UK_CASE(4, 16, 4) UK_CASE(4, 4, 4)
+#undef UK_CASE
+  return false;
+}
 
 uint32_t replicate_pad(uint64_t pad, int es) {
   if (es == 1) return (uint32_t)(pad & 0xFF) * 0x01010101u;
@@ -597,6 +898,10 @@ extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
       plan.args.src = src;
       plan.args.dst = dst;
       plan.args.pad32 = replicate_pad(p->padding_value, es);
+      if (plan.stream && launch_stream<false>(plan, stream)) {
+        *kernel_name = "pack_stream";
+        return (int)hipGetLastError();
+      }
       if (dispatch_gv<PackLauncher>(plan.G, plan.VEC, plan, stream)) {
         *kernel_name = "pack_tiled";
         return (int)hipGetLastError();
@@ -649,6 +954,10 @@ extern "C" int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* p,
       plan.args.src = src;
       plan.args.dst = dst;
       plan.args.pad32 = 0;
+      if (plan.stream && launch_stream<true>(plan, stream)) {
+        *kernel_name = "unpack_stream";
+        return (int)hipGetLastError();
+      }
       if (dispatch_gv<UnpackLauncher>(plan.G, plan.VEC, plan, stream)) {
         *kernel_name = "unpack_tiled";
         return (int)hipGetLastError();
