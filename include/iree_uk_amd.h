@@ -327,6 +327,17 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_kernel_mode(int mode);
  * ("" if it returned early). Static storage; never NULL. */
 IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_kernel_name(void);
 
+/* Per-kernel device timing for the calling thread. Between begin and end,
+ * every kernel an entry point launches carries its own start/stop event pair
+ * (the events timestamp the kernel itself, as a profiler would). end waits for
+ * the kernels, writes up to `capacity` durations in microseconds to
+ * elapsed_us[] in launch order with the launching op in kinds[] (0 pack,
+ * 1 unpack, 2 mmt4d; either array may be NULL), and returns the number of
+ * kernels launched since begin. */
+IREE_UK_AMD_EXPORT void iree_uk_amd_timing_begin(void);
+IREE_UK_AMD_EXPORT int iree_uk_amd_timing_end(double* elapsed_us, int* kinds,
+                                              int capacity);
+
 /* Number of devices visible to HIP (0 when there is none or no driver). */
 IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);
 

@@ -9,6 +9,7 @@
 
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
+#include "uk_launch.h"
 
 namespace {
 
@@ -244,7 +245,7 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
   const int64_t cap = 256 * 64;
   const int grid = (int)(blocks < cap ? blocks : cap);
 #define UK_LAUNCH(K) \
-  case K: hipLaunchKernelGGL(mmt4d_generic_kernel<K>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+  case K: uk::launch(2, mmt4d_generic_kernel<K>, dim3(grid), dim3(kThreads), 0, stream, a); break;
   switch (kind) {
     UK_LAUNCH(Kind::kF32) UK_LAUNCH(Kind::kS8S8) UK_LAUNCH(Kind::kS16S16)
     UK_LAUNCH(Kind::kS16S8) UK_LAUNCH(Kind::kS8S4) UK_LAUNCH(Kind::kS16U4)

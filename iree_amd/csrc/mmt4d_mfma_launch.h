@@ -9,6 +9,7 @@
 #include "mmt4d_mfma_kernel.h"
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
+#include "uk_launch.h"
 
 namespace uk_mfma {
 
@@ -69,8 +70,8 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
         (int)SH::kLdsBytes);
     if (attr != hipSuccess) return (int)attr;
   }
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)(grid_m * grid_n)), dim3(WGM * WGN * 64),
-                     SH::kLdsBytes, stream, a);
+  uk::launch(2, kernel, dim3((uint32_t)(grid_m * grid_n)), dim3(WGM * WGN * 64),
+             SH::kLdsBytes, stream, a);
   return (int)hipGetLastError();
 }
 

@@ -23,6 +23,7 @@
 
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
+#include "uk_launch.h"
 
 namespace {
 
@@ -828,16 +829,16 @@ bool dispatch_gv(int G, int VEC, const TiledPlan& plan, hipStream_t stream) {
 template <int G, int VEC>
 struct PackLauncher {
   static void launch(const TiledPlan& plan, hipStream_t stream) {
-    hipLaunchKernelGGL((pack_tiled_kernel<G, VEC>), dim3(plan.grid),
-                       dim3(kThreads), plan.lds_bytes, stream, plan.args);
+    uk::launch(0, pack_tiled_kernel<G, VEC>, dim3(plan.grid), dim3(kThreads),
+               plan.lds_bytes, stream, plan.args);
   }
 };
 
 template <int G, int VEC>
 struct UnpackLauncher {
   static void launch(const TiledPlan& plan, hipStream_t stream) {
-    hipLaunchKernelGGL((unpack_tiled_kernel<G, VEC>), dim3(plan.grid),
-                       dim3(kThreads), plan.lds_bytes, stream, plan.args);
+    uk::launch(1, unpack_tiled_kernel<G, VEC>, dim3(plan.grid), dim3(kThreads),
+               plan.lds_bytes, stream, plan.args);
   }
 };
 
@@ -849,8 +850,8 @@ bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
   const uint32_t lds = 2 * plan.args.lds_buf_bytes;
 #define UK_CASE(g, vv, mv)                                                          \
   if (plan.G == g && plan.VEC == vv && plan.MV == mv) {                              \
-    hipLaunchKernelGGL((stream_tiled_kernel<g, vv, mv, UNPACK>), dim3(grid),         \
-                       dim3(kThreads), lds, stream, plan.args);                      \
+    uk::launch(UNPACK ? 1 : 0, stream_tiled_kernel<g, vv, mv, UNPACK>, dim3(grid),   \
+               dim3(kThreads), lds, stream, plan.args);                              \
     return true;                                                                     \
   }
   UK_CASE(16, 16, 16) UK_CASE(8, 16, 16) UK_CASE(4, 16, 16) UK_CASE(4, 4, 16)
@@ -926,9 +927,9 @@ extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
   a.transpose_outer = to;
   const int grid = grid_for(a.total);
   switch (es) {
-    case 1: hipLaunchKernelGGL(pack_generic_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
-    case 2: hipLaunchKernelGGL(pack_generic_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
-    default: hipLaunchKernelGGL(pack_generic_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    case 1: uk::launch(0, pack_generic_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    case 2: uk::launch(0, pack_generic_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    default: uk::launch(0, pack_generic_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
   }
   *kernel_name = "pack_generic";
   return (int)hipGetLastError();
@@ -982,9 +983,9 @@ extern "C" int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* p,
   a.transpose_outer = to;
   const int grid = grid_for(a.total);
   switch (es) {
-    case 2: hipLaunchKernelGGL(unpack_generic_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
-    case 1: hipLaunchKernelGGL(unpack_generic_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
-    default: hipLaunchKernelGGL(unpack_generic_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    case 2: uk::launch(1, unpack_generic_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    case 1: uk::launch(1, unpack_generic_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
+    default: uk::launch(1, unpack_generic_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, a); break;
   }
   *kernel_name = "unpack_generic";
   return (int)hipGetLastError();

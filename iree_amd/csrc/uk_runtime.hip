@@ -1,7 +1,44 @@
 // Thin C-ABI wrappers over the HIP runtime for the plain-C host layer.
 #include <hip/hip_runtime.h>
 
+#include <vector>
+
 #include "uk_hip_abi.h"
+#include "uk_launch.h"
+
+namespace {
+
+// Per-thread ring of event pairs for kernel timing.
+struct TimingState {
+  bool on = false;
+  std::vector<hipEvent_t> start, stop;
+  std::vector<int> kind;
+  size_t used = 0;
+};
+thread_local TimingState g_timing;
+
+}  // namespace
+
+namespace uk {
+
+bool timing_next_events(int kind, hipEvent_t* start, hipEvent_t* stop) {
+  TimingState& t = g_timing;
+  if (!t.on) return false;
+  if (t.used == t.start.size()) {
+    hipEvent_t a, b;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return false;
+    t.start.push_back(a);
+    t.stop.push_back(b);
+    t.kind.push_back(0);
+  }
+  t.kind[t.used] = kind;
+  *start = t.start[t.used];
+  *stop = t.stop[t.used];
+  ++t.used;
+  return true;
+}
+
+}  // namespace uk
 
 extern "C" {
 
@@ -75,6 +112,29 @@ int iree_uk_amd_hip_copy2d_to_host(void* dst, int64_t dst_pitch,
 
 int iree_uk_amd_hip_stream_synchronize(void* stream) {
   return (int)hipStreamSynchronize((hipStream_t)stream);
+}
+
+void iree_uk_amd_timing_begin(void) {
+  g_timing.on = true;
+  g_timing.used = 0;
+}
+
+int iree_uk_amd_timing_end(double* elapsed_us, int* kinds, int capacity) {
+  TimingState& t = g_timing;
+  t.on = false;
+  int n = 0;
+  for (size_t i = 0; i < t.used; ++i) {
+    if (hipEventSynchronize(t.stop[i]) != hipSuccess) break;
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, t.start[i], t.stop[i]) != hipSuccess) break;
+    if (n < capacity) {
+      if (elapsed_us) elapsed_us[n] = (double)ms * 1e3;
+      if (kinds) kinds[n] = t.kind[i];
+    }
+    ++n;
+  }
+  t.used = 0;
+  return n;
 }
 
 const char* iree_uk_amd_hip_error_string(int status) {

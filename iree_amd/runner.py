@@ -256,22 +256,26 @@ class Runner:
         raise KeyError(name)
 
     # ------------------------------------------------------------------ timing
+    KIND = {"pack": 0, "unpack": 1, "mmt4d": 2}
+
     def time_op(self, op: Op, iters: int, warmup: int = 2):
-        """Average and minimum duration in microseconds of `iters` launches,
-        each bracketed by HIP events on the launch stream."""
+        """(average, minimum, median) device duration in microseconds of
+        `iters` launches. Each launch carries its own HIP start/stop event pair
+        on the launch stream (iree_uk_amd_timing_begin/end), which timestamps
+        the kernel itself."""
         torch = self.torch
         with torch.cuda.stream(self.stream):
             for _ in range(warmup):
                 op.launch()
             op.kernel = self.lib.last_kernel_name()
-            starts = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
-            ends = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
-            for i in range(iters):
-                starts[i].record(self.stream)
+            self.stream.synchronize()
+            self.lib.timing_begin()
+            for _ in range(iters):
                 op.launch()
-                ends[i].record(self.stream)
-        self.stream.synchronize()
-        us = [s.elapsed_time(e) * 1e3 for s, e in zip(starts, ends)]
+            recs = self.lib.timing_end()
+        # A call may launch two kernels (whole K steps + remainder): sum per call.
+        per_call = len(recs) // iters
+        us = [sum(t for _, t in recs[i * per_call:(i + 1) * per_call]) for i in range(iters)]
         return sum(us) / len(us), min(us), sorted(us)[len(us) // 2]
 
     @staticmethod
@@ -289,34 +293,35 @@ class Runner:
 
     def run_steps(self, wl: Workload, steps: int, warmup: int, dominant: str):
         """Times exactly `steps` passes of the whole workload (wall clock around
-        a synchronize on both sides) and, inside the same timed region, each
-        launch of the dominant kernel with HIP events on the launch stream."""
+        a synchronize on both sides). Inside the same timed region every kernel
+        launch carries a HIP event pair; returns (seconds per step, average
+        device microseconds per launch of the dominant op)."""
         import time
         torch = self.torch
-        dom_starts, dom_ends = [], []
+        dom_kind = self.KIND["mmt4d" if dominant == "mmt4d" else
+                             ("unpack" if dominant.startswith("unpack") else "pack")]
+        n_dom = sum(1 for op in wl.ops if op.name == dominant)
         with torch.cuda.stream(self.stream):
             for _ in range(warmup):
                 for op in wl.ops:
                     op.launch()
                     op.kernel = self.lib.last_kernel_name()
             torch.cuda.synchronize()
+            self.lib.timing_begin()
             t0 = time.perf_counter()
             for _ in range(steps):
                 for op in wl.ops:
-                    if op.name == dominant:
-                        s = torch.cuda.Event(enable_timing=True)
-                        e = torch.cuda.Event(enable_timing=True)
-                        s.record(self.stream)
-                        op.launch()
-                        e.record(self.stream)
-                        dom_starts.append(s)
-                        dom_ends.append(e)
-                    else:
-                        op.launch()
+                    op.launch()
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-        dom_us = [s.elapsed_time(e) * 1e3 for s, e in zip(dom_starts, dom_ends)]
-        return (t1 - t0) / steps, (sum(dom_us) / len(dom_us) if dom_us else math.nan)
+            recs = self.lib.timing_end(capacity=max(4096, 8 * steps * len(wl.ops)))
+        dom_total = sum(t for k, t in recs if k == dom_kind)
+        # Ops of the same kind as the dominant one but with another name (e.g.
+        # pack_lhs vs pack_rhs) only occur for pure data-movement workloads,
+        # where the figure is then the average over that kind.
+        n_kind = sum(1 for op in wl.ops if self.KIND.get(op.name.split("_")[0], -1) == dom_kind)
+        dom_us = dom_total / (steps * max(1, n_kind if n_dom == 0 else n_kind)) if recs else math.nan
+        return (t1 - t0) / steps, dom_us
 
     def measured_copy_gbps(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """Device-to-device copy rate (read + write bytes), for a measured HBM

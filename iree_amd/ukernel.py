@@ -149,6 +149,9 @@ class UKernelLibrary:
         L.iree_uk_amd_device_count.restype = ctypes.c_int
         L.iree_uk_amd_version.restype = ctypes.c_char_p
         L.iree_uk_amd_set_assert_handler.argtypes = [_vp]
+        L.iree_uk_amd_timing_begin.restype = None
+        L.iree_uk_amd_timing_end.argtypes = [_vp, _vp, ctypes.c_int]
+        L.iree_uk_amd_timing_end.restype = ctypes.c_int
         self._handler_ref = None
         self._violations: list[str] = []
 
@@ -226,6 +229,19 @@ class UKernelLibrary:
 
     def last_kernel_name(self) -> str:
         return self.lib.iree_uk_amd_last_kernel_name().decode()
+
+    def timing_begin(self):
+        """Starts per-kernel device timing of this thread's calls."""
+        self.lib.iree_uk_amd_timing_begin()
+
+    def timing_end(self, capacity: int = 4096):
+        """Returns [(kind, microseconds)] for every kernel launched since
+        timing_begin, in launch order; kind is 0 pack, 1 unpack, 2 mmt4d."""
+        us = (ctypes.c_double * capacity)()
+        kinds = (ctypes.c_int * capacity)()
+        n = self.lib.iree_uk_amd_timing_end(us, kinds, capacity)
+        n = min(n, capacity)
+        return [(kinds[i], us[i]) for i in range(n)]
 
     def device_count(self) -> int:
         return int(self.lib.iree_uk_amd_device_count())
