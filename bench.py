@@ -31,6 +31,23 @@ EXTRA_WORKLOADS = [
 ]
 
 
+def recorded_traffic(workload: str, op: str):
+    """HBM bytes per launch of the dominant kernel, from the committed
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of this workload (counters
+    cannot be read from inside the process); None when there is none."""
+    if workload != "c2_f16_chain_4096" or op != "mmt4d":
+        return None
+    path = os.path.join(ROOT, "profiles", "c2_f16_chain_4096_hbm_traffic.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("mmt4d_traffic_bytes_per_launch:"):
+                    return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_threads() -> int:
     try:
         n = len(os.sched_getaffinity(0))
@@ -140,6 +157,7 @@ def main() -> int:
     roof = R.roofline(dom, dom_us)
     roof["kernel"] = dom.kernel
     roof["avg_us"] = round(dom_us, 2)
+    roof["traffic"] = recorded_traffic(args.workload, dominant)
 
     per_kernel = {}
     for op in wl.ops:
