@@ -104,6 +104,7 @@ struct Args {
   uint32_t accumulate;
   uint32_t tail;       // 1 when the last K step is partial
   uint32_t band;       // workgroup rows per rasterization band
+  uint32_t vec_out;    // 1: N0 % 4 == 0 and `out`, out_stride are 16-byte aligned
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that
@@ -164,7 +165,8 @@ __device__ __forceinline__ void block_of_workgroup(uint32_t wg, const Args& a,
 // PIPE 1: three LDS stages, loads three steps ahead, fragments one step ahead.
 // RBC: 16 = row bytes >= 16 (direct), 8/4/2 = regrouping loaders.
 template <Elem E, int RBC, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>
-__global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
+__global__ __launch_bounds__(WGM* WGN * 64)
+void mmt4d_mfma_kernel(Args a) {
   using TT = ElemTraits<E>;
   using Acc = typename TT::Acc;
   using Scalar = typename TT::Scalar;
@@ -179,10 +181,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
   // A loader block is 64 units (one per lane); a unit is R loads + R stores.
   constexpr int BLOCKS_A = BM * NCH / R / 64;
   // PIPE 2 keeps only the LHS in LDS; RHS fragments come straight from global.
-  constexpr int BLOCKS = (PIPE == 2 ? BM : BM + BN) * NCH / R / 64;
+  constexpr int BLOCKS = (PIPE >= 2 ? BM : BM + BN) * NCH / R / 64;
   constexpr int NU = (BLOCKS + NW - 1) / NW;
   constexpr int IMAGE_A = BM * KS;
-  constexpr int STAGE = (PIPE == 2 ? BM : BM + BN) * KS;
+  constexpr int STAGE = (PIPE >= 2 ? BM : BM + BN) * KS;
   static_assert((BM * NCH / R) % 64 == 0 && (BN * NCH / R) % 64 == 0, "block split");
   // When the blocks do not divide evenly over the waves, the surplus (wave, i)
   // slots are idle: they load from a valid address and skip the store.
@@ -283,43 +285,62 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
   const uint32_t rd_b = IMAGE_A + (uint32_t)(wn * TN) * NCHB * 1024;
 
   // ---- accumulators -------------------------------------------------------
-  // Lane (q, c = r) of block (tm, tn) holds rows 4q..4q+3, column c.
+  // The MFMA takes the RHS fragment as its first operand, so lane (q, r) of
+  // block (tm, tn) holds output row r, columns 4q..4q+3: four consecutive
+  // elements of one row of the [M0][N0] output tile when N0 is a multiple of
+  // four, which one 16-byte access moves (a wave then covers whole tiles
+  // contiguously). `vec_out` is 0 when that does not hold or the output is not
+  // 16-byte aligned; elements then move one by one.
   Acc acc[TM][TN];
-  auto for_each_output = [&](auto f) {
+  auto for_each_output = [&](auto f4, auto f1) {
     // The lane coordinates pass through an empty asm so that the address
     // arithmetic of the prologue (ACCUMULATE loads) and of the epilogue
-    // (stores) is not shared: shared, it would stay live in ~80 registers
-    // across the whole K loop.
+    // (stores) is not shared: shared, it would stay live across the K loop.
     uint32_t oq = q, orr = r;
     asm volatile("" : "+v"(oq), "+v"(orr));
-    const char* out_base = a.out + (int64_t)pm0 * a.out_stride +
-                           (int64_t)pn0 * a.M0 * a.N0 * 4;
-    uint32_t col_off[TN];
-    bool col_ok[TN];
+    char* out_base = a.out + (int64_t)pm0 * a.out_stride + (int64_t)pn0 * a.M0 * a.N0 * 4;
+    const uint32_t tile_bytes = (uint32_t)(a.M0 * a.N0 * 4);
+    if (a.vec_out) {
+      uint32_t col_off[TN];
+      bool col_ok[TN];
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-      const int col = (wn * TN + tn) * 16 + (int)orr;
-      const int pl = col / a.N0, n0 = col - pl * a.N0;
-      col_ok[tn] = pl < a.bpn && pn0 + pl < a.N1;
-      col_off[tn] = (uint32_t)pl * (uint32_t)(a.M0 * a.N0 * 4) + (uint32_t)n0 * 4;
-    }
+      for (int tn = 0; tn < TN; ++tn) {
+        const int col = (wn * TN + tn) * 16 + 4 * (int)oq;
+        const int pl = col / a.N0, n0 = col - pl * a.N0;
+        col_ok[tn] = pl < a.bpn && pn0 + pl < a.N1;
+        col_off[tn] = (uint32_t)pl * tile_bytes + (uint32_t)n0 * 4;
+      }
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int row = (wm * TM + tm) * 16 + 4 * (int)oq + e;
+      for (int tm = 0; tm < TM; ++tm) {
+        const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
         const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
         const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * 4);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
-          if (row_ok && col_ok[tn]) {
-            f(tm, tn, e, reinterpret_cast<Scalar*>(const_cast<char*>(out_base) + (row_off + col_off[tn])));
-          }
+          if (row_ok && col_ok[tn]) f4(tm, tn, reinterpret_cast<Acc*>(out_base + (row_off + col_off[tn])));
         }
-        // Keep the unrolled rows from being hoisted together: that would
-        // hold one address pair per output element live at once.
+        // Keep the unrolled rows from being hoisted together.
         __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        const int row = (wm * TM + tm) * 16 + (int)orr;
+        const int pl = row / a.M0, m0 = row - pl * a.M0;
+        const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * 4);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int col = (wn * TN + tn) * 16 + 4 * (int)oq + e;
+            const int pc = col / a.N0, n0 = col - pc * a.N0;
+            if (row_ok && pc < a.bpn && pn0 + pc < a.N1)
+              f1(tm, tn, e, reinterpret_cast<Scalar*>(out_base + (row_off + (uint32_t)pc * tile_bytes + (uint32_t)n0 * 4)));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
   };
@@ -328,7 +349,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
   if (a.accumulate) {
-    for_each_output([&](int tm, int tn, int e, Scalar* p) { acc[tm][tn][e] = *p; });
+    for_each_output([&](int tm, int tn, Acc* p) { acc[tm][tn] = *p; },
+                    [&](int tm, int tn, int e, Scalar* p) { acc[tm][tn][e] = *p; });
   }
 
   // ---- pipeline -----------------------------------------------------------
@@ -394,7 +416,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fa[tm], fb[tn], acc[tm][tn]);
+      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fb[tn], fa[tm], acc[tm][tn]);
   };
   const int last = a.steps - 1;
   const bool has_tail = a.tail != 0;
@@ -486,7 +508,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
           read_b(fb[P ^ 1][tn], st_next, tn);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
-          acc[tm][tn] = TT::mfma(fa[tm & 1], fb[P][tn], acc[tm][tn]);
+          acc[tm][tn] = TT::mfma(fb[P][tn], fa[tm & 1], acc[tm][tn]);
         __builtin_amdgcn_sched_barrier(0);
       }
       __syncthreads();
@@ -560,26 +582,18 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
       for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
         for (int tn = tm * TN / TM; tn < (tm + 1) * TN / TM; ++tn) {
-#ifndef UK_DBG_NO_B
           load_b(fb[P ^ 1][tn], tn, b_step);
-#endif
         }
 #pragma unroll
         for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k) {
-#ifndef UK_DBG_NO_A_STORE
           *reinterpret_cast<v4i*>(lds + st_write + loff[k]) = regs[P ^ 1][k][0];
-#endif
-#ifndef UK_DBG_NO_A_LOAD
           regs[P][k][0] = load_piece(k, voff[k] + (uint32_t)ld_step * sstep[k]);
-#endif
         }
-#ifndef UK_DBG_NO_A_READ
         if (tm + 1 < TM) read_a(fa[(tm + 1) & 1], st_cur, tm + 1);
         else read_a(fa[0], st_next, 0);
-#endif
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
-          acc[tm][tn] = TT::mfma(fa[tm & 1], fb[P][tn], acc[tm][tn]);
+          acc[tm][tn] = TT::mfma(fb[P][tn], fa[tm & 1], acc[tm][tn]);
         __builtin_amdgcn_sched_barrier(0);
       }
       __syncthreads();
@@ -596,8 +610,99 @@ __global__ __launch_bounds__(WGM* WGN * 64) void mmt4d_mfma_kernel(Args a) {
     if (s < a.steps) iteration(s, std::integral_constant<int, 0>{});
   }
 
+  else if constexpr (PIPE == 3) {
+    // As PIPE 2 with every prefetch one step deeper, unrolled by three so that
+    // LDS stage, register set and fragment buffer indices are all the
+    // compile-time phase P = s % 3:
+    //   iteration s computes step s from LDS stage P and RHS buffer P,
+    //   issues the LHS global loads of step s+4 into register set (P+1)%3,
+    //   stores register set (P+2)%3 (step s+2, loaded in iteration s-2) to
+    //   LDS stage (P+2)%3, and loads the RHS fragments of step s+2 into
+    //   buffer (P+2)%3. LHS fragments are fetched one row ahead.
+    static_assert(RBC >= 16, "register-direct RHS needs row bytes >= 16");
+    static_assert(NKK == 1 && TM % 2 == 0, "see PIPE 1");
+    constexpr int NP = NU;
+    v4i regs[3][NU][R];
+    v4i fa[2][HALVES], fb[3][TN][HALVES];
+    const char* sbase_b = a.rhs + (int64_t)pn0 * a.rhs_stride;
+    const uint32_t kt_bytes_b = (uint32_t)a.N0 << lrb;
+    const uint32_t sstep_b = (uint32_t)kts_per_step * kt_bytes_b;
+    uint32_t voff_b[TN][HALVES];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const uint32_t row = (uint32_t)(wn * TN + tn) * 16 + r;
+      const uint32_t pl = row / (uint32_t)a.N0;
+      const uint32_t n0 = row - pl * a.N0;
+      const bool ok = (int)pl < a.bpn && pn0 + (int)pl < a.N1;
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h) {
+        const uint32_t kb = (uint32_t)(h * 4 + q) * 16;
+        voff_b[tn][h] = ok ? pl * (uint32_t)a.rhs_stride + (kb >> lrb) * kt_bytes_b +
+                                 (n0 << lrb) + (kb & ((1u << lrb) - 1))
+                           : 0u;
+      }
+    }
+    auto load_b = [&](v4i (&dst)[HALVES], int tn, int step) {
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        dst[h] = *reinterpret_cast<const v4i*>(sbase_b + (voff_b[tn][h] + (uint32_t)step * sstep_b));
+    };
+    auto read_a = [&](v4i (&dst)[HALVES], uint32_t stage_off, int tm) {
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h)
+        dst[h] = *reinterpret_cast<const v4i*>(lds + stage_off + rd_a +
+                                               (tm * NCHB + h) * 1024 + rd_slot[h]);
+    };
+    load_global(regs[0], 0, false);
+    store_lds(regs[0], 0);
+    load_global(regs[1], min(1, last), false);
+    store_lds(regs[1], STAGE);
+    load_global(regs[2], min(2, last), false);
+    load_global(regs[0], min(3, last), false);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      load_b(fb[0][tn], tn, 0);
+      load_b(fb[1][tn], tn, min(1, last));
+    }
+    __syncthreads();
+    read_a(fa[0], 0, 0);
+    auto iteration = [&](int s, auto phase) {
+      constexpr int P = decltype(phase)::value;
+      constexpr uint32_t st_cur = P * STAGE, st_next = ((P + 1) % 3) * STAGE,
+                         st_write = ((P + 2) % 3) * STAGE;
+      const int ld_step = min(s + 4, last);
+      const int b_step = min(s + 2, last);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int tn = tm * TN / TM; tn < (tm + 1) * TN / TM; ++tn)
+          load_b(fb[(P + 2) % 3][tn], tn, b_step);
+#pragma unroll
+        for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k) {
+          *reinterpret_cast<v4i*>(lds + st_write + loff[k]) = regs[(P + 2) % 3][k][0];
+          regs[(P + 1) % 3][k][0] = load_piece(k, voff[k] + (uint32_t)ld_step * sstep[k]);
+        }
+        if (tm + 1 < TM) read_a(fa[(tm + 1) & 1], st_cur, tm + 1);
+        else read_a(fa[0], st_next, 0);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = TT::mfma(fb[P][tn], fa[tm & 1], acc[tm][tn]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();
+    };
+    int s = 0;
+    for (; s + 2 < a.steps; s += 3) {
+      iteration(s, std::integral_constant<int, 0>{});
+      iteration(s + 1, std::integral_constant<int, 1>{});
+      iteration(s + 2, std::integral_constant<int, 2>{});
+    }
+    if (s < a.steps) iteration(s, std::integral_constant<int, 0>{});
+    if (s + 1 < a.steps) iteration(s + 1, std::integral_constant<int, 1>{});
+  }
   // ---- epilogue -----------------------------------------------------------
-  for_each_output([&](int tm, int tn, int e, Scalar* p) { *p = acc[tm][tn][e]; });
+  for_each_output([&](int tm, int tn, Acc* p) { __builtin_nontemporal_store(acc[tm][tn], p); },
+                  [&](int tm, int tn, int e, Scalar* p) { *p = acc[tm][tn][e]; });
 }
 
 template <Elem E, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>
@@ -607,7 +712,7 @@ struct Shape {
   static constexpr int BM = WGM * TM * 16;
   static constexpr int BN = WGN * TN * 16;
   static constexpr size_t kLdsBytes =
-      (PIPE ? 3 : 2) * (size_t)(PIPE == 2 ? BM : BM + BN) * KS;
+      (PIPE ? 3 : 2) * (size_t)(PIPE >= 2 ? BM : BM + BN) * KS;
 };
 
 }  // namespace uk_mfma

@@ -57,6 +57,7 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   if (PIPE != 0 && (a.tail || kt_count == 0)) return -1;
   a.accumulate = accumulate;
   a.band = 4;
+  a.vec_out = p.N0 % 4 == 0 && ((uintptr_t)p.out % 16) == 0 && p.out_stride % 16 == 0;
   // 32-bit offsets inside a workgroup's share of each operand.
   const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
   const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
@@ -97,7 +98,9 @@ template <Elem E, int RBC>
 int launch_class(const Problem& p, int forced, hipStream_t stream, const char** name) {
   constexpr int H = ElemTraits<E>::kHalves;
   constexpr int NKK2 = 2 / H;             // 128 bytes of K per step
-  constexpr int BIG_PIPE = RBC >= 16 ? 2 : 1;
+  // Three RHS fragment buffers fit the register file only with one fragment
+  // register quad per block (all types but f8).
+  constexpr int BIG_PIPE = RBC >= 16 ? (ElemTraits<E>::kHalves == 1 ? 3 : 2) : 1;
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
