@@ -701,7 +701,7 @@ void mmt4d_mfma_kernel(Args a) {
     if (s + 1 < a.steps) iteration(s + 1, std::integral_constant<int, 1>{});
   }
   // ---- epilogue -----------------------------------------------------------
-  for_each_output([&](int tm, int tn, Acc* p) { __builtin_nontemporal_store(acc[tm][tn], p); },
+  for_each_output([&](int tm, int tn, Acc* p) { *p = acc[tm][tn]; },
                   [&](int tm, int tn, int e, Scalar* p) { *p = acc[tm][tn][e]; });
 }
 

@@ -443,15 +443,21 @@ template <> struct GBytes<4> { using type = uint32_t; };
 template <> struct GBytes<8> { using type = v2u; };
 template <> struct GBytes<16> { using type = v4u; };
 
+// Global accesses of the streaming kernels. Addresses are 4-byte aligned at
+// least; wider vectors at such addresses are legal on gfx950 under HSA
+// (unaligned access mode), and the types say so.
+// Plain (cache-allocating) accesses on purpose: what pack writes is read by
+// mmt4d next, and what unpack reads was just written by mmt4d, so for operands
+// up to the size of the memory-side cache the hand-over never reaches HBM.
 template <int N>
 __device__ __forceinline__ typename GBytes<N>::type gload(const char* gptr) {
-  using T = typename GBytes<N>::type;
-  return __builtin_nontemporal_load(reinterpret_cast<const T*>(gptr));
+  typedef typename GBytes<N>::type T4 __attribute__((aligned(4)));
+  return *reinterpret_cast<const T4*>(gptr);
 }
 template <int N>
 __device__ __forceinline__ void gstore(char* gptr, typename GBytes<N>::type v) {
-  using T = typename GBytes<N>::type;
-  __builtin_nontemporal_store(v, reinterpret_cast<T*>(gptr));
+  typedef typename GBytes<N>::type T4 __attribute__((aligned(4)));
+  *reinterpret_cast<T4*>(gptr) = v;
 }
 
 constexpr uint32_t kStreamBlockBytes = 16384;  // LDS bytes per buffer, at most
@@ -541,33 +547,73 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
   }
 
   const uint32_t nblocks = a.nblk0 * a.nblk1;
+
+  // Block coordinates, base pointers and whether the whole block lies inside
+  // the matrix and the tile grid ("interior").
+  struct Block {
+    uint32_t blk0, blk1, row_base, col_base_bytes;
+    const char* mat_c;
+    const char* tiled_c;
+    bool interior;
+  };
+  auto block_at = [&](uint32_t blk) {
+    Block b;
+    b.blk0 = blk / a.nblk1;
+    b.blk1 = blk - b.blk0 * a.nblk1;
+    b.row_base = b.blk0 * a.block_rows;
+    b.col_base_bytes = b.blk1 * a.block_row_bytes;
+    b.mat_c = (UNPACK ? a.dst : a.src) + (int64_t)b.row_base * a.mat_stride0_bytes + b.col_base_bytes;
+    b.tiled_c = (UNPACK ? a.src : a.dst) + (int64_t)(b.blk0 * a.G0) * a.sl0_bytes +
+                (int64_t)(b.blk1 * a.G1) * a.sl1_bytes;
+    b.interior = b.row_base + a.block_rows <= a.mat_size0 &&
+                 b.col_base_bytes + a.block_row_bytes <= size1_bytes &&
+                 (b.blk0 + 1) * a.G0 <= a.outer0 && (b.blk1 + 1) * a.G1 <= a.outer1;
+    return b;
+  };
+
+  // The global loads of an interior block are issued one block ahead, before
+  // the barrier and the store phase of the current block, so that a workgroup
+  // keeps loads and stores in flight together. Edge blocks load in place.
+  MatVec pre1[UNPACK ? 1 : N1];
+  TileVec pre2[UNPACK ? N2 : 1];
+  auto prefetch = [&](const Block& b) {
+    if constexpr (!UNPACK) {
+#pragma unroll
+      for (int i = 0; i < N1; ++i)
+        if (tid + i * kThreads < total1) pre1[i] = gload<MV>(b.mat_c + g1off[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < N2; ++i)
+        if (tid + i * kThreads < total2) pre2[i] = gload<VEC>(b.tiled_c + g2off[i]);
+    }
+  };
+
+  // Workgroups are handed to the eight XCDs round-robin. Within one sweep of
+  // the grid, the workgroups of one XCD take consecutive blocks (column blocks
+  // of one block row first): neighbouring blocks share the cache lines that
+  // their unaligned row segments straddle, and the L2 of the XCD then sees
+  // both halves of such a line at about the same time.
+  const uint32_t first_blk = (gridDim.x & 7) ? blockIdx.x
+                                             : (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   uint32_t buf = 0;
-  for (uint32_t blk = blockIdx.x; blk < nblocks; blk += gridDim.x) {
-    const uint32_t blk0 = blk / a.nblk1;
-    const uint32_t blk1 = blk - blk0 * a.nblk1;
-    const uint32_t row_base = blk0 * a.block_rows;
-    const uint32_t col_base_bytes = blk1 * a.block_row_bytes;
-    const char* mat_c = (UNPACK ? a.dst : a.src) + (int64_t)row_base * a.mat_stride0_bytes +
-                        col_base_bytes;
-    const char* tiled_c = (UNPACK ? a.src : a.dst) + (int64_t)(blk0 * a.G0) * a.sl0_bytes +
-                          (int64_t)(blk1 * a.G1) * a.sl1_bytes;
+  bool have_pre = false;
+  for (uint32_t blk = first_blk; blk < nblocks; blk += gridDim.x) {
+    const Block b = block_at(blk);
+    const uint32_t blk0 = b.blk0, blk1 = b.blk1, row_base = b.row_base,
+                   col_base_bytes = b.col_base_bytes;
+    const char* mat_c = b.mat_c;
+    const char* tiled_c = b.tiled_c;
+    const bool interior = b.interior;
     char* lbuf = lds + buf * a.lds_buf_bytes;
     buf ^= 1;
-    // Interior: the whole block lies inside the matrix and the tile grid.
-    const bool interior = row_base + a.block_rows <= a.mat_size0 &&
-                          col_base_bytes + a.block_row_bytes <= size1_bytes &&
-                          (blk0 + 1) * a.G0 <= a.outer0 && (blk1 + 1) * a.G1 <= a.outer1;
+    if (interior && !have_pre) prefetch(b);
 
     if constexpr (!UNPACK) {
       // ---- pack phase 1: 2-D rows -> LDS ----
       if (interior) {
-        MatVec reg[N1];
 #pragma unroll
         for (int i = 0; i < N1; ++i)
-          if (tid + i * kThreads < total1) reg[i] = gload<MV>(mat_c + g1off[i]);
-#pragma unroll
-        for (int i = 0; i < N1; ++i)
-          if (tid + i * kThreads < total1) lds_store_pieces<MV>(lbuf + l1off[i], reg[i], piece);
+          if (tid + i * kThreads < total1) lds_store_pieces<MV>(lbuf + l1off[i], pre1[i], piece);
       } else {
         for (uint32_t idx = tid; idx < total1; idx += kThreads) {
           uint32_t r, cb;
@@ -576,77 +622,87 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
           const bool row_ok = row_base + r < a.mat_size0;
           const char* gp = mat_c + (r * a.mat_stride0_bytes32 + cb);
           const uint32_t es = a.elem_bytes;
-          for (uint32_t b = 0; b < MV; b += es) {
-            const bool ok = row_ok && (col_base_bytes + cb + b) < size1_bytes;
+          for (uint32_t bb = 0; bb < MV; bb += es) {
+            const bool ok = row_ok && (col_base_bytes + cb + bb) < size1_bytes;
             if (es == 4) {
-              *reinterpret_cast<uint32_t*>(reg + b) =
-                  ok ? *reinterpret_cast<const uint32_t*>(gp + b) : a.pad32;
+              *reinterpret_cast<uint32_t*>(reg + bb) =
+                  ok ? *reinterpret_cast<const uint32_t*>(gp + bb) : a.pad32;
             } else if (es == 2) {
-              *reinterpret_cast<uint16_t*>(reg + b) =
-                  ok ? *reinterpret_cast<const uint16_t*>(gp + b) : (uint16_t)a.pad32;
+              *reinterpret_cast<uint16_t*>(reg + bb) =
+                  ok ? *reinterpret_cast<const uint16_t*>(gp + bb) : (uint16_t)a.pad32;
             } else {
-              reg[b] = ok ? gp[b] : (char)a.pad32;
+              reg[bb] = ok ? gp[bb] : (char)a.pad32;
             }
           }
           store_pieces<MV>(lbuf + r * a.lds_pitch + cb, reg, piece);
         }
       }
-      __syncthreads();
-      // ---- pack phase 2: LDS -> tiled runs ----
-      {
-        TileVec reg[N2];
-#pragma unroll
-        for (int i = 0; i < N2; ++i) {
-          if (tid + i * kThreads < total2) {
-            __attribute__((aligned(16))) char tmp[VEC];
-#pragma unroll
-            for (int k = 0; k < NG; ++k)
-              *reinterpret_cast<Gran*>(tmp + k * G) =
-                  *reinterpret_cast<const Gran*>(lbuf + l2off[i][k]);
-            reg[i] = *reinterpret_cast<const TileVec*>(tmp);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < N2; ++i) {
-          if (tid + i * kThreads < total2) {
-            bool ok = true;
-            if (!interior) {
-              uint32_t run, t, in_tile, tl0, tl1;
-              tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
-              ok = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
-            }
-            if (ok) gstore<VEC>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
-          }
-        }
-      }
     } else {
       // ---- unpack phase 1: tiled runs -> LDS (scatter by granules) ----
-      {
-        TileVec reg[N2];
-        bool ok[N2];
+      bool ok[N2];
 #pragma unroll
-        for (int i = 0; i < N2; ++i) {
-          ok[i] = tid + i * kThreads < total2;
-          if (ok[i] && !interior) {
+      for (int i = 0; i < N2; ++i) {
+        ok[i] = tid + i * kThreads < total2;
+        if (!interior) {
+          if (ok[i]) {
             uint32_t run, t, in_tile, tl0, tl1;
             tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
             ok[i] = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
           }
-          if (ok[i]) reg[i] = gload<VEC>(tiled_c + g2off[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < N2; ++i) {
-          if (ok[i]) {
-            __attribute__((aligned(16))) char tmp[VEC];
-            *reinterpret_cast<TileVec*>(tmp) = reg[i];
-#pragma unroll
-            for (int k = 0; k < NG; ++k)
-              *reinterpret_cast<Gran*>(lbuf + l2off[i][k]) =
-                  *reinterpret_cast<const Gran*>(tmp + k * G);
-          }
+          if (ok[i]) pre2[i] = gload<VEC>(tiled_c + g2off[i]);
         }
       }
-      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        if (ok[i]) {
+          __attribute__((aligned(16))) char tmp[VEC];
+          *reinterpret_cast<TileVec*>(tmp) = pre2[i];
+#pragma unroll
+          for (int k = 0; k < NG; ++k)
+            *reinterpret_cast<Gran*>(lbuf + l2off[i][k]) =
+                *reinterpret_cast<const Gran*>(tmp + k * G);
+        }
+      }
+    }
+
+    // Next block's loads (interior blocks only).
+    have_pre = false;
+    if (blk + gridDim.x < nblocks) {
+      const Block nb = block_at(blk + gridDim.x);
+      if (nb.interior) {
+        prefetch(nb);
+        have_pre = true;
+      }
+    }
+    __syncthreads();
+
+    if constexpr (!UNPACK) {
+      // ---- pack phase 2: LDS -> tiled runs ----
+      TileVec reg[N2];
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        if (tid + i * kThreads < total2) {
+          __attribute__((aligned(16))) char tmp[VEC];
+#pragma unroll
+          for (int k = 0; k < NG; ++k)
+            *reinterpret_cast<Gran*>(tmp + k * G) =
+                *reinterpret_cast<const Gran*>(lbuf + l2off[i][k]);
+          reg[i] = *reinterpret_cast<const TileVec*>(tmp);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        if (tid + i * kThreads < total2) {
+          bool ok = true;
+          if (!interior) {
+            uint32_t run, t, in_tile, tl0, tl1;
+            tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+            ok = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
+          }
+          if (ok) gstore<VEC>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
+        }
+      }
+    } else {
       // ---- unpack phase 2: LDS rows -> 2-D rows ----
       if (interior) {
         MatVec reg[N1];
@@ -665,10 +721,10 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
           __attribute__((aligned(16))) char reg[MV];
           load_pieces<MV>(reg, lbuf + r * a.lds_pitch + cb, piece);
           char* gp = const_cast<char*>(mat_c) + (r * a.mat_stride0_bytes32 + cb);
-          for (uint32_t b = 0; b < MV && col_base_bytes + cb + b < size1_bytes; b += es) {
-            if (es == 4) copy_bytes<4>(gp + b, reg + b);
-            else if (es == 2) copy_bytes<2>(gp + b, reg + b);
-            else gp[b] = reg[b];
+          for (uint32_t bb = 0; bb < MV && col_base_bytes + cb + bb < size1_bytes; bb += es) {
+            if (es == 4) copy_bytes<4>(gp + bb, reg + bb);
+            else if (es == 2) copy_bytes<2>(gp + bb, reg + bb);
+            else gp[bb] = reg[bb];
           }
         }
       }
@@ -798,6 +854,10 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
                 block_rows * std::abs(mat_stride0) * es < (1ll << 31) &&
                 (G0 * std::abs(v.sl0) + G1 * std::abs(v.sl1)) * es < (1ll << 31);
   plan.MV = mat_vec >= 16 ? 16 : 4;
+  // The streaming kernels move 16 bytes per lane on the 2-D side from any
+  // 4-byte aligned row start (LDS offsets stay 16-byte aligned: they are
+  // relative to the block's window).
+  if (plan.stream && block_row_bytes % 16 == 0) plan.MV = 16;
   if (plan.stream) {
     a.mat_vec = (uint32_t)plan.MV;
     a.div_row_vecs = FastDiv((uint32_t)(block_row_bytes / plan.MV));

@@ -292,10 +292,15 @@ class Runner:
                 "unit": unit, "frac": round(achieved / peak, 4), "traffic": None}
 
     def run_steps(self, wl: Workload, steps: int, warmup: int, dominant: str):
-        """Times exactly `steps` passes of the whole workload (wall clock around
-        a synchronize on both sides). Inside the same timed region every kernel
-        launch carries a HIP event pair; returns (seconds per step, average
-        device microseconds per launch of the dominant op)."""
+        """Runs the whole workload `warmup` untimed times, then twice `steps`
+        times, each pass bracketed by a synchronize on both sides and timed on
+        the wall clock:
+          pass 1, launches only: seconds per step of the whole job;
+          pass 2, every launch carrying a HIP start/stop event pair on the
+          launch stream: average device microseconds per launch of the
+          dominant op (the event pairs serialize the queue a little, so this
+          pass is slower as a whole and is reported separately).
+        Returns (seconds per step, seconds per step with events, dominant us)."""
         import time
         torch = self.torch
         dom_kind = self.KIND["mmt4d" if dominant == "mmt4d" else
@@ -307,13 +312,19 @@ class Runner:
                     op.launch()
                     op.kernel = self.lib.last_kernel_name()
             torch.cuda.synchronize()
-            self.lib.timing_begin()
             t0 = time.perf_counter()
             for _ in range(steps):
                 for op in wl.ops:
                     op.launch()
             torch.cuda.synchronize()
             t1 = time.perf_counter()
+            self.lib.timing_begin()
+            t2 = time.perf_counter()
+            for _ in range(steps):
+                for op in wl.ops:
+                    op.launch()
+            torch.cuda.synchronize()
+            t3 = time.perf_counter()
             recs = self.lib.timing_end(capacity=max(4096, 8 * steps * len(wl.ops)))
         dom_total = sum(t for k, t in recs if k == dom_kind)
         # Ops of the same kind as the dominant one but with another name (e.g.
@@ -321,7 +332,7 @@ class Runner:
         # where the figure is then the average over that kind.
         n_kind = sum(1 for op in wl.ops if self.KIND.get(op.name.split("_")[0], -1) == dom_kind)
         dom_us = dom_total / (steps * max(1, n_kind if n_dom == 0 else n_kind)) if recs else math.nan
-        return (t1 - t0) / steps, dom_us
+        return (t1 - t0) / steps, (t3 - t2) / steps, dom_us
 
     def measured_copy_gbps(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """Device-to-device copy rate (read + write bytes), for a measured HBM
