@@ -6,6 +6,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "mmt4d_mfma_kernel.h"
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
@@ -114,6 +116,67 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 2;
   } else {
     choice = 3;
+  }
+  if (choice == 1 && forced == 0) {
+    // Tile quantization: a last row or column of 256x256 workgroups that is
+    // mostly padding can cost a whole extra round on the 256 CUs. Compare, in
+    // units of one round of big tiles, keeping it in the big launch against
+    // splitting it off as a strip that the smaller variants compute (at
+    // roughly 0.45 of the big variant's rate, and never faster than about a
+    // quarter round: their K loop is as long).
+    const int bpm = 256 / p.M0, bpn = 256 / p.N0;
+    const int64_t gm_c = uk::ceil_div(p.M1, bpm), gn_c = uk::ceil_div(p.N1, bpn);
+    const int64_t gm_f = p.M1 / bpm, gn_f = p.N1 / bpn;
+    auto rounds = [](int64_t wgs) { return (double)uk::ceil_div(wgs, 256); };
+    auto strip_cost = [&](int64_t panels_m, int64_t panels_n) {
+      const double tiles = (double)(panels_m * p.M0) * (double)(panels_n * p.N0) / 65536.0;
+      return std::max(0.25, tiles / 256.0 / 0.45);
+    };
+    double best = rounds(gm_c * gn_c);
+    int split_m = 0, split_n = 0;
+    for (int fm = 0; fm < 2; ++fm) {
+      for (int fn = 0; fn < 2; ++fn) {
+        if (!fm && !fn) continue;
+        if (fm && (gm_f == 0 || gm_f == gm_c)) continue;
+        if (fn && (gn_f == 0 || gn_f == gn_c)) continue;
+        const int64_t gm = fm ? gm_f : gm_c, gn = fn ? gn_f : gn_c;
+        double cost = rounds(gm * gn);
+        const int64_t main_n = fn ? gn_f * bpn : p.N1;
+        if (fn) cost += strip_cost(p.M1, p.N1 - main_n);
+        if (fm) cost += strip_cost(p.M1 - gm_f * bpm, main_n);
+        if (cost < best - 0.1) { best = cost; split_m = fm; split_n = fn; }
+      }
+    }
+    if (split_m || split_n) {
+      const int32_t main_m = split_m ? (int32_t)(gm_f * bpm) : p.M1;
+      const int32_t main_n = split_n ? (int32_t)(gn_f * bpn) : p.N1;
+      Problem q = p;
+      q.M1 = main_m;
+      q.N1 = main_n;
+      int st = launch_class<E, RBC>(q, 0, stream, name);
+      if (st != 0) return st;
+      const char* strip_name = nullptr;
+      if (split_n) {  // columns [main_n, N1), all rows
+        q = p;
+        q.rhs = p.rhs + (int64_t)main_n * p.rhs_stride;
+        q.out = p.out + (int64_t)main_n * p.M0 * p.N0 * 4;
+        q.N1 = p.N1 - main_n;
+        st = launch_class<E, RBC>(q, 0, stream, &strip_name);
+        // The main part has run: "not served" must not reach the caller, who
+        // would recompute (and with ACCUMULATE, re-add) the whole problem.
+        if (st != 0) return st < 0 ? (int)hipErrorUnknown : st;
+      }
+      if (split_m) {  // rows [main_m, M1), columns [0, main_n)
+        q = p;
+        q.lhs = p.lhs + (int64_t)main_m * p.lhs_stride;
+        q.out = p.out + (int64_t)main_m * p.out_stride;
+        q.M1 = p.M1 - main_m;
+        q.N1 = main_n;
+        st = launch_class<E, RBC>(q, 0, stream, &strip_name);
+        if (st != 0) return st < 0 ? (int)hipErrorUnknown : st;
+      }
+      return 0;
+    }
   }
   if (choice == 1) {
     const int kts_per_step = BIG_KS >> p.lrb;

@@ -101,6 +101,24 @@ def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
             assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
 
 
+# Shapes big enough for the 256x256 variant whose last row and/or column of
+# workgroups is mostly padding: the library computes those as separate strips
+# with the smaller variants. (tile counts M1, N1, K1 for 16x16x16 s8 tiles)
+@pytest.mark.parametrize("shape", [(256, 257, 4), (241, 273, 5), (257, 256, 8)])
+def test_mmt4d_split_off_remainder_strips(gpu, oracle, shape):
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    tf, M0, N0, K0 = uk.MMT4D_TYPE_S8S8S32, 16, 16, 16
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=777, slack=16, shapes=(shape,))):
+        rng = np.random.default_rng(100 + ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256"), lib.last_kernel_name()
+
+
 def _normal_operand(rng, kind, n, scale=1.0):
     x = (rng.standard_normal(n) * scale).astype(np.float32)
     if kind == "f16":
