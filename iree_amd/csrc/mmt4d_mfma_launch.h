@@ -196,7 +196,9 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     // With 2-byte rows a 16-byte piece spans 8 rows and 32 rows do not fill a
     // loader block; that combination takes the 64x64 variant.
     if constexpr (RBC != 2) {
-      int st = launch_variant<E, RBC, 2, 1, 1, 4, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
+      // 256 bytes of K per step: these problems are bound by memory latency,
+      // and a longer step keeps more bytes in flight per workgroup.
+      int st = launch_variant<E, RBC, 2, 1, 1, 4, 4 / H, 0>(p, 0, p.K1, p.accumulate, stream);
       if (st >= 0) { *name = "mmt4d_mfma_32x64"; return st; }
     }
     choice = 3;
