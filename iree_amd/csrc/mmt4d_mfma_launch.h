@@ -178,9 +178,12 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
       return 0;
     }
   }
+  // Whole pipeline steps of K go to a software-pipelined variant; what is left
+  // of K (less than one step) to the two-stage variant of the same or a
+  // smaller workgroup shape, as a second, accumulating launch.
+  const int kts_per_step = BIG_KS >> p.lrb;
+  const int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
   if (choice == 1) {
-    const int kts_per_step = BIG_KS >> p.lrb;
-    const int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
     if (kt_main > 0) {
       int st = launch_variant<E, RBC, 8, 4, 2, 4, 1, BIG_PIPE>(p, 0, kt_main, p.accumulate, stream);
       if (st == 0) {
@@ -204,8 +207,30 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 3;
   }
   if (choice == 2) {
+    if constexpr (RBC >= 16) {
+      if (kt_main > 0) {
+        int st = launch_variant<E, RBC, 4, 2, 2, 4, 1, 3>(p, 0, kt_main, p.accumulate, stream);
+        if (st == 0) {
+          *name = "mmt4d_mfma_128x128_rhs_direct";
+          if (kt_main == p.K1) return 0;
+          return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+        }
+        if (st > 0) return st;
+      }
+    }
     int st = launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
     if (st >= 0) { *name = "mmt4d_mfma_128x128"; return st; }
+  }
+  if constexpr (RBC >= 16) {
+    if (kt_main > 0) {
+      int st = launch_variant<E, RBC, 2, 2, 2, 2, 1, 3>(p, 0, kt_main, p.accumulate, stream);
+      if (st == 0) {
+        *name = "mmt4d_mfma_64x64_rhs_direct";
+        if (kt_main == p.K1) return 0;
+        return launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+      }
+      if (st > 0) return st;
+    }
   }
   int st = launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
   if (st >= 0) { *name = "mmt4d_mfma_64x64"; return st; }
