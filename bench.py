@@ -32,12 +32,12 @@ EXTRA_WORKLOADS = [
 
 
 def recorded_traffic(workload: str, op: str):
-    """HBM bytes per launch of the dominant kernel, from the committed
+    """HBM-side bytes per launch of the dominant kernel, from the committed
     rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of this workload (counters
     cannot be read from inside the process); None when there is none."""
-    if workload != "c2_f16_chain_4096" or op != "mmt4d":
+    if op != "mmt4d":
         return None
-    path = os.path.join(ROOT, "profiles", "c2_f16_chain_4096_hbm_traffic.txt")
+    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt")
     try:
         with open(path) as f:
             for line in f:
@@ -133,7 +133,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f16_chain_4096")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
