@@ -81,9 +81,11 @@ template <> struct ElemTraits<Elem::kF8> {
   static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
     v8i av = {a[0][0], a[0][1], a[0][2], a[0][3], a[1][0], a[1][1], a[1][2], a[1][3]};
     v8i bv = {b[0][0], b[0][1], b[0][2], b[0][3], b[1][0], b[1][1], b[1][2], b[1][3]};
-    // Formats 0/0 = E4M3 x E4M3; block scales of 2^0 (E8M0 code 127).
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-        av, bv, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    // Formats 0/0 = E4M3 x E4M3. Zero scale operands select the unscaled
+    // instruction (v_mfma_f32_16x16x128_f8f6f4, plain products); the scaled
+    // form with 2^0 block scales computes the same but is a two-part
+    // instruction (scale load + MFMA) and issues more slowly.
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, 0, 0, 0, 0, 0, 0);
   }
 };
 
