@@ -344,6 +344,25 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);
 /* Library version, "major.minor". */
 IREE_UK_AMD_EXPORT const char* iree_uk_amd_version(void);
 
+/*===----------------------------------------------------------------------===*/
+/* HAL executable plugin face                                                  */
+/*===----------------------------------------------------------------------===*/
+
+/* The library is also a HAL executable plugin: an IREE runtime started with
+ * `--executable_plugin=<path to this library>`
+ * (runtime/src/iree/tooling/context_util.c:589-614) looks this symbol up
+ * (runtime/src/iree/hal/local/executable_plugin.h:185-191, export name :188-189)
+ * and resolves the imports `iree_uk_mmt4d`, `iree_uk_pack` and `iree_uk_unpack`
+ * of compiled LLVMCPU programs through it. The result is the reference's
+ * `const iree_hal_executable_plugin_header_t**` (interface version 0.1,
+ * executable_plugin.h:404-461), or NULL when `max_version` is below 0.1. Each
+ * resolved import is an `int fn(void* params_ptr, void* context, void*
+ * reserved)` thunk (runtime/src/iree/hal/local/executable_library.h:150-158)
+ * that forwards to the `_p` entry points above and returns non-zero when the
+ * call failed. */
+IREE_UK_AMD_EXPORT const void* iree_hal_executable_plugin_query(
+    uint32_t max_version, void* reserved);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif
