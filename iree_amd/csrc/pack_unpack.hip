@@ -622,6 +622,19 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
           const bool row_ok = row_base + r < a.mat_size0;
           const char* gp = mat_c + (r * a.mat_stride0_bytes32 + cb);
           const uint32_t es = a.elem_bytes;
+          // Whole vector inside the matrix, or whole vector padding: one access.
+          if (row_ok && col_base_bytes + cb + MV <= size1_bytes) {
+            lds_store_pieces<MV>(lbuf + r * a.lds_pitch + cb, gload<MV>(gp), piece);
+            continue;
+          }
+          if (!row_ok || col_base_bytes + cb >= size1_bytes) {
+            MatVec padv;
+            uint32_t* pw = reinterpret_cast<uint32_t*>(&padv);
+#pragma unroll
+            for (int w = 0; w < MV / 4; ++w) pw[w] = a.pad32;
+            lds_store_pieces<MV>(lbuf + r * a.lds_pitch + cb, padv, piece);
+            continue;
+          }
           for (uint32_t bb = 0; bb < MV; bb += es) {
             const bool ok = row_ok && (col_base_bytes + cb + bb) < size1_bytes;
             if (es == 4) {
@@ -718,9 +731,13 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
           uint32_t r, cb;
           mat_item<MV>(a, idx, &r, &cb);
           if (row_base + r >= a.mat_size0) continue;
+          char* gp = const_cast<char*>(mat_c) + (r * a.mat_stride0_bytes32 + cb);
+          if (col_base_bytes + cb + MV <= size1_bytes) {  // whole vector inside
+            gstore<MV>(gp, lds_load_pieces<MV>(lbuf + r * a.lds_pitch + cb, piece));
+            continue;
+          }
           __attribute__((aligned(16))) char reg[MV];
           load_pieces<MV>(reg, lbuf + r * a.lds_pitch + cb, piece);
-          char* gp = const_cast<char*>(mat_c) + (r * a.mat_stride0_bytes32 + cb);
           for (uint32_t bb = 0; bb < MV && col_base_bytes + cb + bb < size1_bytes; bb += es) {
             if (es == 4) copy_bytes<4>(gp + bb, reg + bb);
             else if (es == 2) copy_bytes<2>(gp + bb, reg + bb);
