@@ -460,7 +460,8 @@ __device__ __forceinline__ void gstore(char* gptr, typename GBytes<N>::type v) {
   *reinterpret_cast<T4*>(gptr) = v;
 }
 
-constexpr uint32_t kStreamBlockBytes = 16384;  // LDS bytes per buffer, at most
+constexpr uint32_t kStreamBlockBytes = 16384;     // matrix bytes per block, streaming kernels
+constexpr uint32_t kStreamBigBlockBytes = 65536;  // same, large transposing problems
 
 struct StreamTables1 {  // 2-D side items of one thread
   uint32_t goff;        // byte offset inside the block's 2-D window
@@ -511,11 +512,11 @@ __device__ __forceinline__ typename GBytes<N>::type lds_load_pieces(const char* 
   return *reinterpret_cast<const typename GBytes<N>::type*>(tmp);
 }
 
-template <int G, int VEC, int MV, bool UNPACK>
+template <int G, int VEC, int MV, bool UNPACK, int BLK>
 __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  constexpr int N1 = kStreamBlockBytes / MV / kThreads;   // 2-D side items per thread
-  constexpr int N2 = kStreamBlockBytes / VEC / kThreads;  // tiled side items per thread
+  constexpr int N1 = BLK / MV / kThreads;   // 2-D side items per thread
+  constexpr int N2 = BLK / VEC / kThreads;  // tiled side items per thread
   constexpr int NG = VEC / G;                             // granules per tiled vector
   using MatVec = typename GBytes<MV>::type;
   using TileVec = typename GBytes<VEC>::type;
@@ -760,6 +761,7 @@ struct TiledPlan {
   TiledArgs args;
   int G = 0, VEC = 0, MV = 0;
   bool stream = false;
+  bool big = false;  // 64 KB blocks (see plan_tiled)
   uint32_t grid = 0;
   uint32_t lds_bytes = 0;
 };
@@ -768,7 +770,8 @@ struct TiledPlan {
 // (source of pack, destination of unpack), `tiled` the 4-D side.
 TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
                      int64_t mat_stride0, int64_t mat_stride1, int64_t mat_size0,
-                     int64_t mat_size1, const char* tiled_ptr, bool ti, bool to) {
+                     int64_t mat_size1, const char* tiled_ptr, bool ti, bool to,
+                     bool allow_big = true) {
   TiledPlan plan;
   if (mat_stride1 != 1) return plan;
   const int64_t tile_elems = v.tile0 * v.tile1;
@@ -787,8 +790,17 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   if (G > VEC) G = VEC;
 
   // Block shape. A run is the contiguous tiled-side span of one block.
-  const int64_t kMinSpan = 256;    // bytes, both sides
-  const int64_t kTarget = 16384;   // LDS bytes per block, about
+  // Large element-granular transposes (4-byte granules: every 16-byte vector
+  // of one side is four scattered words of the other) take 64 KB blocks with
+  // 512-byte segments on both sides instead of 16 KB and 256: fewer, longer
+  // segments mean fewer cache lines that a segment only partly covers, which
+  // is what bounds them (f32 12288x12289 unpack: 3.3 -> 4.1 TB/s). Smaller
+  // problems keep the small blocks: they need the parallelism.
+  const int64_t total_bytes = v.outer0 * v.outer1 * tile_bytes;
+  const bool big = allow_big && G == 4 && VEC == 16 && total_bytes >= (192ll << 20);
+  const int64_t kMinSpan = big ? 512 : 256;                      // bytes, both sides
+  const int64_t kTarget = big ? kStreamBigBlockBytes : kStreamBlockBytes;  // bytes per block, about
+  const int64_t stream_block = kTarget;
   int64_t G0 = 1, G1 = uk::ceil_div(kMinSpan, v.tile1 * es);
   if (to) {
     G0 = uk::ceil_div(kMinSpan, tile_bytes);
@@ -816,7 +828,11 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   }
   pitch = uk::ceil_div(pitch, G) * G;
   const int64_t lds_bytes = block_rows * pitch;
-  if (lds_bytes > 64 * 1024) return plan;
+  if (lds_bytes > (big ? 80 : 64) * 1024) {
+    if (big) return plan_tiled(v, es, mat_ptr, mat_stride0, mat_stride1, mat_size0, mat_size1,
+                               tiled_ptr, ti, to, false);
+    return plan;
+  }
 
   // 2-D side vector width.
   const int64_t mat_vec = std::min(
@@ -866,8 +882,8 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   // Streaming kernels: 32-bit offsets inside one block on both sides, granules
   // of at least 4 bytes, at most 4 granules per vector, block within budget.
   plan.stream = mat_vec >= 4 && G >= 4 && VEC / G <= 4 &&
-                block_rows * block_row_bytes <= kStreamBlockBytes &&
-                lds_bytes <= 2 * kStreamBlockBytes &&
+                block_rows * block_row_bytes <= stream_block &&
+                lds_bytes <= (big ? 80 * 1024 : 2 * stream_block) &&
                 block_rows * std::abs(mat_stride0) * es < (1ll << 31) &&
                 (G0 * std::abs(v.sl0) + G1 * std::abs(v.sl1)) * es < (1ll << 31);
   plan.MV = mat_vec >= 16 ? 16 : 4;
@@ -875,6 +891,11 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   // 4-byte aligned row start (LDS offsets stay 16-byte aligned: they are
   // relative to the block's window).
   if (plan.stream && block_row_bytes % 16 == 0) plan.MV = 16;
+  if (big && !(plan.stream && plan.MV == 16)) {
+    return plan_tiled(v, es, mat_ptr, mat_stride0, mat_stride1, mat_size0, mat_size1, tiled_ptr,
+                      ti, to, false);
+  }
+  plan.big = big;
   if (plan.stream) {
     a.mat_vec = (uint32_t)plan.MV;
     a.div_row_vecs = FastDiv((uint32_t)(block_row_bytes / plan.MV));
@@ -923,12 +944,24 @@ template <bool UNPACK>
 bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
   // Persistent grid: up to 4 workgroups per CU, two LDS buffers each.
   const uint32_t nblocks = plan.grid;
-  const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
   const uint32_t lds = 2 * plan.args.lds_buf_bytes;
+  if (plan.big) {
+    // One workgroup per CU: two 66 KB buffers fill its LDS.
+    if (!(plan.G == 4 && plan.VEC == 16 && plan.MV == 16)) return false;
+    auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes>;
+    static hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+        160 * 1024);
+    if (attr != hipSuccess || lds > 160 * 1024) return false;
+    uk::launch(UNPACK ? 1 : 0, kernel, dim3(nblocks < 256 ? nblocks : 256), dim3(kThreads), lds,
+               stream, plan.args);
+    return true;
+  }
+  const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
 #define UK_CASE(g, vv, mv)                                                          \
   if (plan.G == g && plan.VEC == vv && plan.MV == mv) {                              \
-    uk::launch(UNPACK ? 1 : 0, stream_tiled_kernel<g, vv, mv, UNPACK>, dim3(grid),   \
-               dim3(kThreads), lds, stream, plan.args);                              \
+    uk::launch(UNPACK ? 1 : 0, stream_tiled_kernel<g, vv, mv, UNPACK, kStreamBlockBytes>, \
+               dim3(grid), dim3(kThreads), lds, stream, plan.args);                  \
     return true;                                                                     \
   }
   UK_CASE(16, 16, 16) UK_CASE(8, 16, 16) UK_CASE(4, 16, 16) UK_CASE(4, 4, 16)

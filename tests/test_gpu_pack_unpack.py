@@ -139,7 +139,10 @@ def test_pack_unpack_round_trip_and_numpy_identity(gpu):
     for (dtype, tf, t0, t1, ti, to, shape) in (
             (np.float32, uk.PACK_TYPE_F32F32, 16, 1, False, True, (1537, 1030)),
             (np.float16, uk.PACK_TYPE_F16F16, 16, 16, False, False, (2047, 2049)),
-            (np.int32, uk.PACK_TYPE_I32I32, 16, 16, True, True, (1000, 999))):
+            (np.int32, uk.PACK_TYPE_I32I32, 16, 16, True, True, (1000, 999)),
+            # above 192 MB: the 64 KB-block kernels for large element-granular
+            # transposes, with rows that are only 4-byte aligned and ragged edges
+            (np.float32, uk.PACK_TYPE_F32F32, 16, 1, False, True, (7169, 7171))):
         x = rng.integers(-30000, 30000, shape).astype(dtype)
         pad_val = dtype(-1)
         pad_bits = int(np.array([pad_val]).view({2: np.uint16, 4: np.uint32}[x.itemsize])[0])
