@@ -106,7 +106,7 @@ struct Args {
   uint32_t accumulate;
   uint32_t tail;       // 1 when the last K step is partial
   uint32_t band;       // workgroup rows per rasterization band
-  uint32_t vec_out;    // 1: N0 % 4 == 0 and `out`, out_stride are 16-byte aligned
+  uint32_t vec_out;    // 1: 4 consecutive columns of a row are contiguous, 16-byte aligned
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that

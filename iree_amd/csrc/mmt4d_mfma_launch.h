@@ -59,7 +59,11 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   if (PIPE != 0 && (a.tail || kt_count == 0)) return -1;
   a.accumulate = accumulate;
   a.band = 4;
-  a.vec_out = p.N0 % 4 == 0 && ((uintptr_t)p.out % 16) == 0 && p.out_stride % 16 == 0;
+  // Four consecutive output columns of one row are contiguous when they lie in
+  // one tile row (N0 % 4 == 0), or when tiles are single rows (M0 == 1: the
+  // tiles of a row then follow each other) and the row ends on a multiple of 4.
+  a.vec_out = (p.N0 % 4 == 0 || (p.M0 == 1 && ((int64_t)p.N1 * p.N0) % 4 == 0)) &&
+              ((uintptr_t)p.out % 16) == 0 && p.out_stride % 16 == 0;
   // 32-bit offsets inside a workgroup's share of each operand.
   const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
   const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;

@@ -119,6 +119,27 @@ def test_mmt4d_split_off_remainder_strips(gpu, oracle, shape):
         assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256"), lib.last_kernel_name()
 
 
+def test_mmt4d_single_row_tiles_equal_row_major_matmul(gpu):
+    """With M0 = N0 = 1 the mmt4d layouts are plain row-major [M][K], [N][K]
+    and [M][N]: the call must equal the integer matrix product A . B^T
+    (independent of the oracle: a closed form)."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    rng = np.random.default_rng(3)
+    for (M, N, K, K0) in ((300, 260, 512, 16), (257, 131, 192, 64), (64, 64, 64, 16)):
+        a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+        bt = rng.integers(-128, 128, (N, K), dtype=np.int8)
+        out0 = rng.integers(-1000, 1000, (M, N)).astype(np.int32)
+        d = [T.DeviceBytes(torch, x) for x in (a, bt, out0)]
+        flags = uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE
+        lib.mmt4d(d[0].ptr, 0, K, d[1].ptr, 0, K, d[2].ptr, 0, N, M, N, K // K0, 1, 1, K0, flags)
+        lib.synchronize()
+        assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
+        want = out0.astype(np.int64) + a.astype(np.int64) @ bt.astype(np.int64).T
+        got = d[2].numpy().view(np.int32).reshape(M, N)
+        assert np.array_equal(got, want.astype(np.int32)), (M, N, K, K0)
+
+
 def _normal_operand(rng, kind, n, scale=1.0):
     x = (rng.standard_normal(n) * scale).astype(np.float32)
     if kind == "f16":
