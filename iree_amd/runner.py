@@ -63,6 +63,7 @@ class Runner:
         self.seed = seed
         self.lib.set_stream(self.stream.cuda_stream)
         self.lib.set_pointer_mode(uk.POINTER_MODE_DEVICE)
+        self.settle_seconds = 0.05
 
     def close(self):
         self.lib.set_stream(None)
@@ -258,7 +259,7 @@ class Runner:
     # ------------------------------------------------------------------ timing
     KIND = {"pack": 0, "unpack": 1, "mmt4d": 2}
 
-    def time_op(self, op: Op, iters: int, warmup: int = 2):
+    def time_op(self, op: Op, iters: int, warmup: int = 5):
         """(average, minimum, median) device duration in microseconds of
         `iters` launches. Each launch carries its own HIP start/stop event pair
         on the launch stream (iree_uk_amd_timing_begin/end), which timestamps
@@ -307,10 +308,22 @@ class Runner:
                              ("unpack" if dominant.startswith("unpack") else "pack")]
         n_dom = sum(1 for op in wl.ops if op.name == dominant)
         with torch.cuda.stream(self.stream):
+            # The device needs tens of milliseconds of load before its clocks
+            # settle (the first ~60 steps of the f16 chain run ~12 % slower than
+            # the following ones): run untimed steps for `settle_seconds` first.
+            t_settle = time.perf_counter()
+            while time.perf_counter() - t_settle < self.settle_seconds:
+                for _ in range(8):
+                    for op in wl.ops:
+                        op.launch()
+                torch.cuda.synchronize()
             for _ in range(warmup):
                 for op in wl.ops:
                     op.launch()
                     op.kernel = self.lib.last_kernel_name()
+            for op in wl.ops:
+                op.launch()
+                op.kernel = self.lib.last_kernel_name()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
