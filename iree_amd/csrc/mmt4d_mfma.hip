@@ -10,6 +10,7 @@ int launch_s8(const Problem& p, int forced, hipStream_t stream, const char** nam
 int launch_f16(const Problem& p, int forced, hipStream_t stream, const char** name);
 int launch_bf16(const Problem& p, int forced, hipStream_t stream, const char** name);
 int launch_f8(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_f32(const Problem& p, int forced, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 
 namespace {
@@ -22,6 +23,7 @@ bool elem_of(uint32_t flags, Elem* e, int* elem_bytes) {
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *e = Elem::kF16; *elem_bytes = 2; return true;
     case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *e = Elem::kBF16; *elem_bytes = 2; return true;
     case IREE_UK_AMD_FLAG_MMT4D_TYPE_F8E4M3FNF8E4M3FNF32: *e = Elem::kF8; *elem_bytes = 1; return true;
+    case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: *e = Elem::kF32; *elem_bytes = 4; return true;
     default: return false;
   }
 }
@@ -88,6 +90,7 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     case Elem::kF16: return uk_mfma::launch_f16(pr, forced_variant, stream, kernel_name);
     case Elem::kBF16: return uk_mfma::launch_bf16(pr, forced_variant, stream, kernel_name);
     case Elem::kF8: return uk_mfma::launch_f8(pr, forced_variant, stream, kernel_name);
+    case Elem::kF32: return uk_mfma::launch_f32(pr, forced_variant, stream, kernel_name);
   }
   return -1;
 }

@@ -44,7 +44,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-enum class Elem { kS8, kF16, kBF16, kF8 };
+enum class Elem { kS8, kF16, kBF16, kF8, kF32 };
 
 template <Elem E> struct ElemTraits;
 
@@ -86,6 +86,24 @@ template <> struct ElemTraits<Elem::kF8> {
     // form with 2^0 block scales computes the same but is a two-part
     // instruction (scale load + MFMA) and issues more slowly.
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+
+template <> struct ElemTraits<Elem::kF32> {
+  using Acc = v4f;
+  using Scalar = float;
+  static constexpr int kHalves = 1;
+  // v_mfma_f32_16x16x4_f32 takes one f32 of K per lane (row l%16, k = l/16):
+  // the lane's 16-byte piece feeds four of them, one per word. Which four K
+  // values meet in one instruction is the same for both operands, which is
+  // all the sum needs.
+  static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
+    const v4f af = __builtin_bit_cast(v4f, a[0]), bf = __builtin_bit_cast(v4f, b[0]);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[0], bf[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[1], bf[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[2], bf[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[3], bf[3], c, 0, 0, 0);
+    return c;
   }
 };
 

@@ -247,6 +247,13 @@ template <Elem E>
 int launch_elem(const Problem& p, int forced, hipStream_t stream, const char** name) {
   if constexpr (E == Elem::kF8) {
     return p.rb >= 16 ? launch_class<E, 16>(p, forced, stream, name) : -1;
+  } else if constexpr (E == Elem::kF32) {
+    switch (p.rb) {
+      case 2: return -1;
+      case 4: return launch_class<E, 4>(p, forced, stream, name);
+      case 8: return launch_class<E, 8>(p, forced, stream, name);
+      default: return launch_class<E, 16>(p, forced, stream, name);
+    }
   } else {
     switch (p.rb) {
       case 2: return launch_class<E, 2>(p, forced, stream, name);

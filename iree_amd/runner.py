@@ -22,7 +22,7 @@ from . import ukernel as uk
 
 # Published MI355X peaks (dense).
 PEAK_HBM_GBPS = 8000.0
-PEAK_TFLOPS = {"s8": 5000.0, "f8": 5000.0, "f16": 2500.0, "bf16": 2500.0}
+PEAK_TFLOPS = {"s8": 5000.0, "f8": 5000.0, "f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 
 
 @dataclasses.dataclass
@@ -196,6 +196,21 @@ class Runner:
                                 uk.MMT4D_TYPE_BF16BF16F32, "bf16", 2)
             return Workload(name, f"mmt4d bf16xbf16->f32 {S}^3 tiles 16x16x{K0}", [op],
                             op.flops, op.bytes, "bf16",
+                            dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
+                                 M0=M0, N0=N0, K0=K0))
+        if name.startswith("f32_mmt4d_"):
+            _, _, size, k0 = name.split("_")
+            S, K0 = int(size), int(k0[1:])
+            M0 = N0 = 16
+            M1 = N1 = S // 16
+            K1 = S // K0
+            lhs4 = self.normal((M1 * K1 * M0 * K0,), torch.float32, 13)
+            rhs4 = self.normal((N1 * K1 * N0 * K0,), torch.float32, 14)
+            out4 = self.empty(M1 * N1 * M0 * N0, torch.float32)
+            op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                uk.MMT4D_TYPE_F32F32F32, "f32", 4)
+            return Workload(name, f"mmt4d f32xf32->f32 {S}^3 tiles 16x16x{K0}", [op],
+                            op.flops, op.bytes, "f32",
                             dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
                                  M0=M0, N0=N0, K0=K0))
         if name == "c3_s8_decode":

@@ -58,6 +58,8 @@ MFMA_TILES = [
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 16),
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 128),
+    (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 4),
+    (uk.MMT4D_TYPE_F32F32F32, 8, 8, 2), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 32),
 ]
 
 
@@ -156,7 +158,7 @@ def _normal_operand(rng, kind, n, scale=1.0):
     (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16), (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 2),
     (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
-    (uk.MMT4D_TYPE_F32F32F32, 8, 8, 4)])
+    (uk.MMT4D_TYPE_F32F32F32, 8, 8, 4), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1)])
 @pytest.mark.parametrize("accumulate", [0, 1])
 @pytest.mark.parametrize("variant", [0, 1])
 def test_mmt4d_float_tolerance_on_normal_inputs(gpu, oracle, tf, M0, N0, K0, accumulate, variant):
