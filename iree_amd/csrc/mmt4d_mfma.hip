@@ -11,19 +11,32 @@ int launch_f16(const Problem& p, int forced, hipStream_t stream, const char** na
 int launch_bf16(const Problem& p, int forced, hipStream_t stream, const char** name);
 int launch_f8(const Problem& p, int forced, hipStream_t stream, const char** name);
 int launch_f32(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_f16f16(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_bf16bf16(const Problem& p, int forced, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 
 namespace {
 
 using uk_mfma::Elem;
 
-bool elem_of(uint32_t flags, Elem* e, int* elem_bytes) {
+// Element type of the MFMA kernel that serves the type triple in `flags`, the
+// operand element size and the output element size; false when there is none.
+// The 16-bit float outputs are served only with
+// IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS (one rounding at the end is
+// what an f32 accumulator gives; rounding after every K element is not).
+bool elem_of(uint32_t flags, Elem* e, int* elem_bytes, int* out_bytes) {
+  const bool skip = (flags & IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) != 0;
+  *out_bytes = 4;
   switch (flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32: *e = Elem::kS8; *elem_bytes = 1; return true;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *e = Elem::kF16; *elem_bytes = 2; return true;
     case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *e = Elem::kBF16; *elem_bytes = 2; return true;
     case IREE_UK_AMD_FLAG_MMT4D_TYPE_F8E4M3FNF8E4M3FNF32: *e = Elem::kF8; *elem_bytes = 1; return true;
     case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: *e = Elem::kF32; *elem_bytes = 4; return true;
+    case IREE_UK_FLAG_MMT4D_TYPE_F16F16F16:
+      *e = Elem::kF16F16; *elem_bytes = 2; *out_bytes = 2; return skip;
+    case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16BF16:
+      *e = Elem::kBF16BF16; *elem_bytes = 2; *out_bytes = 2; return skip;
     default: return false;
   }
 }
@@ -39,8 +52,8 @@ bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
                                                     int32_t K0, uint32_t flags) {
   Elem e;
-  int eb;
-  if (!elem_of(flags, &e, &eb)) return 0;
+  int eb, ob;
+  if (!elem_of(flags, &e, &eb, &ob)) return 0;
   const int64_t rb = (int64_t)K0 * eb;
   if (!is_pow2(rb) || rb < 2 || rb > 128) return 0;
   if (e == Elem::kF8 && rb < 16) return 0;
@@ -58,24 +71,24 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
                                                  void* stream_v, int forced_variant,
                                                  const char** kernel_name) {
   Elem e;
-  int eb;
-  if (!elem_of(p->flags, &e, &eb)) return -1;
+  int eb, ob;
+  if (!elem_of(p->flags, &e, &eb, &ob)) return -1;
   if (!iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) return -1;
   if (p->K == 0) return -1;  // zero fill only: the generic kernel does it
   hipStream_t stream = (hipStream_t)stream_v;
   uk_mfma::Problem pr;
   pr.lhs = (const char*)p->lhs_buffer + p->lhs_offset * eb;
   pr.rhs = (const char*)p->rhs_buffer + p->rhs_offset * eb;
-  pr.out = (char*)p->out_buffer + p->out_offset * 4;
+  pr.out = (char*)p->out_buffer + p->out_offset * ob;
   pr.lhs_stride = p->lhs_stride0 * eb;
   pr.rhs_stride = p->rhs_stride0 * eb;
-  pr.out_stride = p->out_stride0 * 4;
+  pr.out_stride = p->out_stride0 * ob;
   // 16-byte vector loads need 16-byte aligned panels.
   if (((uintptr_t)pr.lhs | (uintptr_t)pr.rhs | (uint64_t)pr.lhs_stride |
        (uint64_t)pr.rhs_stride) & 15) {
     return -1;
   }
-  if ((uintptr_t)pr.out & 3) return -1;
+  if ((uintptr_t)pr.out & (uintptr_t)(ob - 1)) return -1;
   pr.M1 = (int32_t)p->M;
   pr.N1 = (int32_t)p->N;
   pr.K1 = (int32_t)p->K;
@@ -91,6 +104,8 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     case Elem::kBF16: return uk_mfma::launch_bf16(pr, forced_variant, stream, kernel_name);
     case Elem::kF8: return uk_mfma::launch_f8(pr, forced_variant, stream, kernel_name);
     case Elem::kF32: return uk_mfma::launch_f32(pr, forced_variant, stream, kernel_name);
+    case Elem::kF16F16: return uk_mfma::launch_f16f16(pr, forced_variant, stream, kernel_name);
+    case Elem::kBF16BF16: return uk_mfma::launch_bf16bf16(pr, forced_variant, stream, kernel_name);
   }
   return -1;
 }

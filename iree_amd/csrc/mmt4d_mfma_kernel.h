@@ -36,6 +36,8 @@
 
 #include <type_traits>
 
+#include "uk_float_convert.h"
+
 namespace uk_mfma {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -44,13 +46,48 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-enum class Elem { kS8, kF16, kBF16, kF8, kF32 };
+// kF16F16 / kBF16BF16: 16-bit float output, accumulated in f32 over all of K
+// and rounded once at the end (IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS,
+// runtime/src/iree/builtins/ukernel/mmt4d_tile_generic.c:258-286,348-376).
+enum class Elem { kS8, kF16, kBF16, kF8, kF32, kF16F16, kBF16BF16 };
+
+typedef uint16_t v4u16 __attribute__((ext_vector_type(4)));
+
+// Output access for 4-byte outputs: the accumulator quad as it is.
+template <typename Acc, typename T>
+struct Out32 {
+  static constexpr int kOutBytes = 4;
+  static __device__ __forceinline__ Acc load4(const char* p) { return *reinterpret_cast<const Acc*>(p); }
+  static __device__ __forceinline__ void store4(char* p, Acc v) { *reinterpret_cast<Acc*>(p) = v; }
+  static __device__ __forceinline__ T load1(const char* p) { return *reinterpret_cast<const T*>(p); }
+  static __device__ __forceinline__ void store1(char* p, T v) { *reinterpret_cast<T*>(p) = v; }
+};
+// 16-bit float outputs with EB exponent bits, converted like the CPU ukernel.
+template <int EB>
+struct Out16 {
+  static constexpr int kOutBytes = 2;
+  static __device__ __forceinline__ v4f load4(const char* p) {
+    const v4u16 h = *reinterpret_cast<const v4u16*>(p);
+    return v4f{uk::small16_to_f32<EB>(h[0]), uk::small16_to_f32<EB>(h[1]),
+               uk::small16_to_f32<EB>(h[2]), uk::small16_to_f32<EB>(h[3])};
+  }
+  static __device__ __forceinline__ void store4(char* p, v4f v) {
+    *reinterpret_cast<v4u16*>(p) = v4u16{uk::f32_to_small16<EB>(v[0]), uk::f32_to_small16<EB>(v[1]),
+                                         uk::f32_to_small16<EB>(v[2]), uk::f32_to_small16<EB>(v[3])};
+  }
+  static __device__ __forceinline__ float load1(const char* p) {
+    return uk::small16_to_f32<EB>(*reinterpret_cast<const uint16_t*>(p));
+  }
+  static __device__ __forceinline__ void store1(char* p, float v) {
+    *reinterpret_cast<uint16_t*>(p) = uk::f32_to_small16<EB>(v);
+  }
+};
 
 template <Elem E> struct ElemTraits;
 
 template <> struct ElemTraits<Elem::kS8> {
   using Acc = v4i;
-  using Scalar = int32_t;
+  using Out = Out32<v4i, int32_t>;
   static constexpr int kHalves = 1;  // 16-byte pieces per lane operand
   static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b[0], c, 0, 0, 0);
@@ -58,7 +95,7 @@ template <> struct ElemTraits<Elem::kS8> {
 };
 template <> struct ElemTraits<Elem::kF16> {
   using Acc = v4f;
-  using Scalar = float;
+  using Out = Out32<v4f, float>;
   static constexpr int kHalves = 1;
   static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(
@@ -67,7 +104,7 @@ template <> struct ElemTraits<Elem::kF16> {
 };
 template <> struct ElemTraits<Elem::kBF16> {
   using Acc = v4f;
-  using Scalar = float;
+  using Out = Out32<v4f, float>;
   static constexpr int kHalves = 1;
   static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
@@ -76,7 +113,7 @@ template <> struct ElemTraits<Elem::kBF16> {
 };
 template <> struct ElemTraits<Elem::kF8> {
   using Acc = v4f;
-  using Scalar = float;
+  using Out = Out32<v4f, float>;
   static constexpr int kHalves = 2;
   static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
     v8i av = {a[0][0], a[0][1], a[0][2], a[0][3], a[1][0], a[1][1], a[1][2], a[1][3]};
@@ -91,7 +128,7 @@ template <> struct ElemTraits<Elem::kF8> {
 
 template <> struct ElemTraits<Elem::kF32> {
   using Acc = v4f;
-  using Scalar = float;
+  using Out = Out32<v4f, float>;
   static constexpr int kHalves = 1;
   // v_mfma_f32_16x16x4_f32 takes one f32 of K per lane (row l%16, k = l/16):
   // the lane's 16-byte piece feeds four of them, one per word. Which four K
@@ -105,6 +142,13 @@ template <> struct ElemTraits<Elem::kF32> {
     c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[3], bf[3], c, 0, 0, 0);
     return c;
   }
+};
+
+template <> struct ElemTraits<Elem::kF16F16> : ElemTraits<Elem::kF16> {
+  using Out = Out16<5>;
+};
+template <> struct ElemTraits<Elem::kBF16BF16> : ElemTraits<Elem::kBF16> {
+  using Out = Out16<8>;
 };
 
 struct Args {
@@ -189,7 +233,8 @@ __global__ __launch_bounds__(WGM* WGN * 64)
 void mmt4d_mfma_kernel(Args a) {
   using TT = ElemTraits<E>;
   using Acc = typename TT::Acc;
-  using Scalar = typename TT::Scalar;
+  using Out = typename TT::Out;
+  constexpr int OB = Out::kOutBytes;  // bytes per output element
   constexpr int NW = WGM * WGN;
   constexpr int HALVES = TT::kHalves;
   constexpr int NCHB = NKK * HALVES;       // groups of 4 chunks per step
@@ -318,8 +363,8 @@ void mmt4d_mfma_kernel(Args a) {
     // (stores) is not shared: shared, it would stay live across the K loop.
     uint32_t oq = q, orr = r;
     asm volatile("" : "+v"(oq), "+v"(orr));
-    char* out_base = a.out + (int64_t)pm0 * a.out_stride + (int64_t)pn0 * a.M0 * a.N0 * 4;
-    const uint32_t tile_bytes = (uint32_t)(a.M0 * a.N0 * 4);
+    char* out_base = a.out + (int64_t)pm0 * a.out_stride + (int64_t)pn0 * a.M0 * a.N0 * OB;
+    const uint32_t tile_bytes = (uint32_t)(a.M0 * a.N0 * OB);
     if (a.vec_out) {
       uint32_t col_off[TN];
       bool col_ok[TN];
@@ -328,17 +373,17 @@ void mmt4d_mfma_kernel(Args a) {
         const int col = (wn * TN + tn) * 16 + 4 * (int)oq;
         const int pl = col / a.N0, n0 = col - pl * a.N0;
         col_ok[tn] = pl < a.bpn && pn0 + pl < a.N1;
-        col_off[tn] = (uint32_t)pl * tile_bytes + (uint32_t)n0 * 4;
+        col_off[tn] = (uint32_t)pl * tile_bytes + (uint32_t)n0 * OB;
       }
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
         const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
         const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
-        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * 4);
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * OB);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
-          if (row_ok && col_ok[tn]) f4(tm, tn, reinterpret_cast<Acc*>(out_base + (row_off + col_off[tn])));
+          if (row_ok && col_ok[tn]) f4(tm, tn, out_base + (row_off + col_off[tn]));
         }
         // Keep the unrolled rows from being hoisted together.
         __builtin_amdgcn_sched_barrier(0);
@@ -349,7 +394,7 @@ void mmt4d_mfma_kernel(Args a) {
         const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
         const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
-        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * 4);
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * OB);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
 #pragma unroll
@@ -357,7 +402,7 @@ void mmt4d_mfma_kernel(Args a) {
             const int col = (wn * TN + tn) * 16 + 4 * (int)oq + e;
             const int pc = col / a.N0, n0 = col - pc * a.N0;
             if (row_ok && pc < a.bpn && pn0 + pc < a.N1)
-              f1(tm, tn, e, reinterpret_cast<Scalar*>(out_base + (row_off + (uint32_t)pc * tile_bytes + (uint32_t)n0 * 4)));
+              f1(tm, tn, e, out_base + (row_off + (uint32_t)pc * tile_bytes + (uint32_t)n0 * OB));
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -369,8 +414,8 @@ void mmt4d_mfma_kernel(Args a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
   if (a.accumulate) {
-    for_each_output([&](int tm, int tn, Acc* p) { acc[tm][tn] = *p; },
-                    [&](int tm, int tn, int e, Scalar* p) { acc[tm][tn][e] = *p; });
+    for_each_output([&](int tm, int tn, char* p) { acc[tm][tn] = Out::load4(p); },
+                    [&](int tm, int tn, int e, char* p) { acc[tm][tn][e] = Out::load1(p); });
   }
 
   // ---- pipeline -----------------------------------------------------------
@@ -721,8 +766,8 @@ void mmt4d_mfma_kernel(Args a) {
     if (s + 1 < a.steps) iteration(s + 1, std::integral_constant<int, 1>{});
   }
   // ---- epilogue -----------------------------------------------------------
-  for_each_output([&](int tm, int tn, Acc* p) { *p = acc[tm][tn]; },
-                  [&](int tm, int tn, int e, Scalar* p) { *p = acc[tm][tn][e]; });
+  for_each_output([&](int tm, int tn, char* p) { Out::store4(p, acc[tm][tn]); },
+                  [&](int tm, int tn, int e, char* p) { Out::store1(p, acc[tm][tn][e]); });
 }
 
 template <Elem E, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>

@@ -63,11 +63,13 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   // one tile row (N0 % 4 == 0), or when tiles are single rows (M0 == 1: the
   // tiles of a row then follow each other) and the row ends on a multiple of 4.
   a.vec_out = (p.N0 % 4 == 0 || (p.M0 == 1 && ((int64_t)p.N1 * p.N0) % 4 == 0)) &&
-              ((uintptr_t)p.out % 16) == 0 && p.out_stride % 16 == 0;
+              ((uintptr_t)p.out % (4 * ElemTraits<E>::Out::kOutBytes)) == 0 &&
+              p.out_stride % (4 * ElemTraits<E>::Out::kOutBytes) == 0;
   // 32-bit offsets inside a workgroup's share of each operand.
   const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
   const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
-  const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.N1 * p.M0 * p.N0 * 4;
+  constexpr int OB = ElemTraits<E>::Out::kOutBytes;
+  const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.N1 * p.M0 * p.N0 * OB;
   if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31)) return -1;
   auto kernel = mmt4d_mfma_kernel<E, RBC, TM, TN, WGM, WGN, NKK, PIPE>;
   if (SH::kLdsBytes > 64 * 1024) {
@@ -163,7 +165,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
       if (split_n) {  // columns [main_n, N1), all rows
         q = p;
         q.rhs = p.rhs + (int64_t)main_n * p.rhs_stride;
-        q.out = p.out + (int64_t)main_n * p.M0 * p.N0 * 4;
+        q.out = p.out + (int64_t)main_n * p.M0 * p.N0 * ElemTraits<E>::Out::kOutBytes;
         q.N1 = p.N1 - main_n;
         st = launch_class<E, RBC>(q, 0, stream, &strip_name);
         // The main part has run: "not served" must not reach the caller, who

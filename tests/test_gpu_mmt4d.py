@@ -121,6 +121,32 @@ def test_mmt4d_split_off_remainder_strips(gpu, oracle, shape):
         assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256"), lib.last_kernel_name()
 
 
+# 16-bit float outputs: an MFMA kernel serves them when the caller allows a
+# single rounding at the end (SKIP_INTERMEDIATE_ROUNDINGS); on the reference
+# tests' small-integer inputs every f32 partial sum is exact, so the result must
+# equal the oracle's bit for bit, final rounding included.
+@pytest.mark.parametrize("variant", [0, 1, 3])
+@pytest.mark.parametrize("tf,M0,N0,K0", [
+    (uk.MMT4D_TYPE_F16F16F16, 16, 16, 8), (uk.MMT4D_TYPE_F16F16F16, 16, 16, 1),
+    (uk.MMT4D_TYPE_BF16BF16BF16, 16, 16, 8), (uk.MMT4D_TYPE_BF16BF16BF16, 8, 32, 2)])
+def test_mmt4d_16bit_outputs_single_rounding(gpu, oracle, tf, M0, N0, K0, variant):
+    lib, torch = gpu
+    assert lib.mmt4d_info(M0, N0, K0, tf | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS)
+    assert not lib.mmt4d_info(M0, N0, K0, tf)   # rounding after every element: generic only
+    lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=15000, slack=16,
+                                         extra_flags=uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS,
+                                         shapes=_mfma_shapes(M0, N0, K0, 16))):
+        rng = np.random.default_rng(ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        if c.M and c.N and c.K:
+            assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
+
+
 def test_mmt4d_single_row_tiles_equal_row_major_matmul(gpu):
     """With M0 = N0 = 1 the mmt4d layouts are plain row-major [M][K], [N][K]
     and [M][N]: the call must equal the integer matrix product A . B^T
