@@ -223,3 +223,56 @@ def test_mmt4d_host_pointers_are_staged(gpu, oracle):
                   got.ctypes.data - c.out_offset * 4, c.out_offset, c.out_stride0,
                   c.M, c.N, c.K, c.M0, c.N0, c.K0, c.flags | 0x200)
         assert np.array_equal(got, want), c.label()
+
+
+def test_entry_points_from_concurrent_threads(gpu, oracle):
+    """The entry points are re-entrant (runtime/src/iree/builtins/ukernel/
+    README.md:26): four host threads, each on its own slab of one problem
+    selected through offsets (as the CPU task system slices work), one using
+    host buffers (staged), the others device buffers on their own streams."""
+    import threading
+    lib, torch = gpu
+    rng = np.random.default_rng(11)
+    M1, N1, K1, M0, N0, K0 = 8, 6, 24, 16, 16, 16
+    lhs = rng.integers(-128, 128, M1 * K1 * M0 * K0, dtype=np.int8)
+    rhs = rng.integers(-128, 128, N1 * K1 * N0 * K0, dtype=np.int8)
+    out0 = rng.integers(-99, 99, M1 * N1 * M0 * N0).astype(np.int32)
+    flags = uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE | 0x200
+    want = out0.copy()
+    oracle.mmt4d(lhs, 0, K1 * M0 * K0, rhs, 0, K1 * N0 * K0, want, 0, N1 * M0 * N0,
+                 M1, N1, K1, M0, N0, K0, flags)
+    got_host = out0.copy()
+    d_lhs, d_rhs, d_out = (T.DeviceBytes(torch, x) for x in (lhs, rhs, out0))
+    errors = []
+
+    def slab(t, rows):
+        try:
+            lo = t * rows
+            if t == 0:   # host pointers, default stream
+                lib.mmt4d(lhs.ctypes.data, lo * K1 * M0 * K0, K1 * M0 * K0, rhs.ctypes.data, 0,
+                          K1 * N0 * K0, got_host.ctypes.data, lo * N1 * M0 * N0, N1 * M0 * N0,
+                          rows, N1, K1, M0, N0, K0, flags)
+            else:
+                s = torch.cuda.Stream()
+                lib.set_stream(s.cuda_stream)
+                lib.mmt4d(d_lhs.ptr, lo * K1 * M0 * K0, K1 * M0 * K0, d_rhs.ptr, 0, K1 * N0 * K0,
+                          d_out.ptr, lo * N1 * M0 * N0, N1 * M0 * N0, rows, N1, K1, M0, N0, K0,
+                          flags)
+                lib.synchronize()
+                lib.set_stream(None)
+        except Exception as e:  # noqa: BLE001
+            errors.append(repr(e))
+
+    rows = M1 // 4
+    threads = [threading.Thread(target=slab, args=(t, rows)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    tile_row = N1 * M0 * N0
+    got_dev = d_out.numpy().view(np.int32)
+    assert np.array_equal(got_host[:rows * tile_row], want[:rows * tile_row])
+    assert np.array_equal(got_host[rows * tile_row:], out0[rows * tile_row:])   # other slabs untouched
+    assert np.array_equal(got_dev[rows * tile_row:], want[rows * tile_row:])
+    assert np.array_equal(got_dev[:rows * tile_row], out0[:rows * tile_row])
