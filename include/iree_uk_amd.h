@@ -345,6 +345,52 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);
 IREE_UK_AMD_EXPORT const char* iree_uk_amd_version(void);
 
 /*===----------------------------------------------------------------------===*/
+/* Fused mmt4d + unpack                                                        */
+/*===----------------------------------------------------------------------===*/
+
+/* No counterpart in the reference (its ukernels are separate calls): mmt4d
+ * whose result goes straight into a row-major out_size0 x out_size1 matrix,
+ * `out_stride0` elements between rows. Equal, bit for bit, to iree_uk_mmt4d
+ * into a tiled [M][N][M0][N0] temporary followed by iree_uk_unpack of it
+ * without transposes (tools/unpack_test.c:13-58 is the index map), minus the
+ * temporary's HBM round trip. With IREE_UK_FLAG_MMT4D_ACCUMULATE the matrix is
+ * also the accumulator input. Operand arguments, tile sizes and flags are
+ * those of iree_uk_mmt4d; out_size0 <= M*M0 and out_size1 <= N*N0 (the rest of
+ * the last tiles is dropped). */
+typedef struct iree_uk_amd_mmt4d_unpack_params_t {
+  const void* lhs_buffer;
+  iree_uk_index_t lhs_offset;
+  iree_uk_index_t lhs_stride0;
+  const void* rhs_buffer;
+  iree_uk_index_t rhs_offset;
+  iree_uk_index_t rhs_stride0;
+  void* out_buffer;
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t out_size0;
+  iree_uk_index_t out_size1;
+  iree_uk_index_t M;
+  iree_uk_index_t N;
+  iree_uk_index_t K;
+  int32_t M0;
+  int32_t N0;
+  int32_t K0;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_amd_mmt4d_unpack_params_t;
+
+IREE_UK_AMD_EXPORT void iree_uk_amd_mmt4d_unpack(
+    const void* lhs_buffer, iree_uk_index_t lhs_offset,
+    iree_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0, void* out_buffer,
+    iree_uk_index_t out_offset, iree_uk_index_t out_stride0,
+    iree_uk_index_t out_size0, iree_uk_index_t out_size1, iree_uk_index_t M,
+    iree_uk_index_t N, iree_uk_index_t K, int32_t M0, int32_t N0, int32_t K0,
+    uint32_t flags, const uint64_t* cpu_data);
+IREE_UK_AMD_EXPORT void iree_uk_amd_mmt4d_unpack_p(
+    const iree_uk_amd_mmt4d_unpack_params_t* params);
+
+/*===----------------------------------------------------------------------===*/
 /* HAL executable plugin face                                                  */
 /*===----------------------------------------------------------------------===*/
 

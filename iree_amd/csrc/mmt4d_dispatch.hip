@@ -5,10 +5,11 @@
 #include "uk_hip_abi.h"
 
 extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
-    const iree_uk_mmt4d_params_t* p, void* stream);
+    const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
+    void* stream);
 extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(
-    const iree_uk_mmt4d_params_t* p, void* stream, int forced_variant,
-    const char** kernel_name);
+    const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
+    void* stream, int forced_variant, const char** kernel_name);
 extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
                                                     int32_t K0, uint32_t flags);
 
@@ -19,6 +20,7 @@ extern "C" int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0,
 }
 
 extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
+                                            const iree_uk_amd_rowmajor_out_t* rowmajor,
                                             void* stream, int kernel_mode,
                                             const char** kernel_name) {
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC &&
@@ -26,10 +28,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
     const int forced = kernel_mode >= IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
                            ? kernel_mode - IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
                            : 0;
-    int st = iree_uk_amd_hip_launch_mmt4d_mfma(p, stream, forced, kernel_name);
+    int st = iree_uk_amd_hip_launch_mmt4d_mfma(p, rowmajor, stream, forced, kernel_name);
     // A negative status means "shape not served after all"; fall through.
     if (st >= 0) return st;
   }
   *kernel_name = "mmt4d_generic";
-  return iree_uk_amd_hip_launch_mmt4d_generic(p, stream);
+  return iree_uk_amd_hip_launch_mmt4d_generic(p, rowmajor, stream);
 }

@@ -39,7 +39,12 @@ struct Mmt4dArgs {
   const char* lhs;
   const char* rhs;
   char* out;
-  int64_t lhs_stride_bytes, rhs_stride_bytes, out_stride_elems;
+  int64_t lhs_stride_bytes, rhs_stride_bytes;
+  // Output element (i, j, i0, j0) is out[i*out_s_i + i0*out_s_i0 + j*out_s_j + j0]
+  // (elements): the tiled layout, or a row-major matrix for the fused
+  // mmt4d + unpack, of which only out_rows x out_cols elements exist.
+  int64_t out_s_i, out_s_i0, out_s_j;
+  int64_t out_rows, out_cols;
   int64_t M, N, K;
   int32_t M0, N0, K0;
   uint32_t accumulate, skip_round;
@@ -62,7 +67,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_generic_kernel(Mmt4dArgs a) {
     const int32_t j0 = (int32_t)(t - (int64_t)i0 * a.N0);
     const char* lp = a.lhs + i * a.lhs_stride_bytes;
     const char* rp = a.rhs + j * a.rhs_stride_bytes;
-    const int64_t o = i * a.out_stride_elems + rem;
+    if (i * a.M0 + i0 >= a.out_rows || j * a.N0 + j0 >= a.out_cols) continue;
+    const int64_t o = i * a.out_s_i + i0 * a.out_s_i0 + j * a.out_s_j + j0;
     const int32_t M0 = a.M0, N0 = a.N0, K0 = a.K0;
 
     if constexpr (KIND == Kind::kS8S8 || KIND == Kind::kS16S16 || KIND == Kind::kS16S8) {
@@ -165,7 +171,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_generic_kernel(Mmt4dArgs a) {
 }  // namespace
 
 extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
-    const iree_uk_mmt4d_params_t* p, void* stream_v) {
+    const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
+    void* stream_v) {
   hipStream_t stream = (hipStream_t)stream_v;
   int lhs_bits, rhs_bits, out_bytes;
   Kind kind;
@@ -189,7 +196,19 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
   a.out = (char*)p->out_buffer + p->out_offset * out_bytes;
   a.lhs_stride_bytes = p->lhs_stride0 * lhs_bits / 8;
   a.rhs_stride_bytes = p->rhs_stride0 * rhs_bits / 8;
-  a.out_stride_elems = p->out_stride0;
+  if (rowmajor) {
+    a.out_s_i0 = rowmajor->stride0;
+    a.out_s_i = rowmajor->stride0 * p->M0;
+    a.out_s_j = p->N0;
+    a.out_rows = rowmajor->size0;
+    a.out_cols = rowmajor->size1;
+  } else {
+    a.out_s_i = p->out_stride0;
+    a.out_s_i0 = p->N0;
+    a.out_s_j = (int64_t)p->M0 * p->N0;
+    a.out_rows = p->M * p->M0;
+    a.out_cols = p->N * p->N0;
+  }
   a.M = p->M; a.N = p->N; a.K = p->K;
   a.M0 = p->M0; a.N0 = p->N0; a.K0 = p->K0;
   a.accumulate = (p->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0;

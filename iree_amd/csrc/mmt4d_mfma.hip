@@ -68,6 +68,7 @@ extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
 // Returns a HIP status (>= 0), or -1 when the call is not served after all
 // (operands not 16-byte aligned, spans beyond 2 GiB, ...).
 extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p,
+                                                 const iree_uk_amd_rowmajor_out_t* rowmajor,
                                                  void* stream_v, int forced_variant,
                                                  const char** kernel_name) {
   Elem e;
@@ -82,7 +83,21 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
   pr.out = (char*)p->out_buffer + p->out_offset * ob;
   pr.lhs_stride = p->lhs_stride0 * eb;
   pr.rhs_stride = p->rhs_stride0 * eb;
-  pr.out_stride = p->out_stride0 * ob;
+  if (rowmajor) {
+    // Row m of panel pl is matrix row pl * M0 + m; column panels follow each
+    // other inside a row.
+    pr.out_sm0 = rowmajor->stride0 * ob;
+    pr.out_stride = pr.out_sm0 * p->M0;
+    pr.out_spn = (int64_t)p->N0 * ob;
+    pr.out_rows = rowmajor->size0;
+    pr.out_cols = rowmajor->size1;
+  } else {
+    pr.out_stride = p->out_stride0 * ob;
+    pr.out_sm0 = (int64_t)p->N0 * ob;
+    pr.out_spn = (int64_t)p->M0 * p->N0 * ob;
+    pr.out_rows = p->M * p->M0;
+    pr.out_cols = p->N * p->N0;
+  }
   // 16-byte vector loads need 16-byte aligned panels.
   if (((uintptr_t)pr.lhs | (uintptr_t)pr.rhs | (uint64_t)pr.lhs_stride |
        (uint64_t)pr.rhs_stride) & 15) {

@@ -57,8 +57,11 @@ typedef uint16_t v4u16 __attribute__((ext_vector_type(4)));
 template <typename Acc, typename T>
 struct Out32 {
   static constexpr int kOutBytes = 4;
-  static __device__ __forceinline__ Acc load4(const char* p) { return *reinterpret_cast<const Acc*>(p); }
-  static __device__ __forceinline__ void store4(char* p, Acc v) { *reinterpret_cast<Acc*>(p) = v; }
+  // 4-byte alignment is all these need (gfx950 under HSA takes dword-aligned
+  // wide accesses); row-major outputs with odd row lengths rely on it.
+  typedef Acc Acc4 __attribute__((aligned(4)));
+  static __device__ __forceinline__ Acc load4(const char* p) { return *reinterpret_cast<const Acc4*>(p); }
+  static __device__ __forceinline__ void store4(char* p, Acc v) { *reinterpret_cast<Acc4*>(p) = v; }
   static __device__ __forceinline__ T load1(const char* p) { return *reinterpret_cast<const T*>(p); }
   static __device__ __forceinline__ void store1(char* p, T v) { *reinterpret_cast<T*>(p) = v; }
 };
@@ -157,7 +160,10 @@ struct Args {
   char* out;
   int64_t lhs_stride;  // bytes between LHS panels
   int64_t rhs_stride;  // bytes between RHS panels
-  int64_t out_stride;  // bytes between rows of output tiles
+  int64_t out_stride;  // bytes between output row panels (tiled: rows of tiles; row-major: M0 rows)
+  uint32_t out_sm0;    // bytes between rows inside a panel (tiled: N0 * elem; row-major: row pitch)
+  uint32_t out_spn;    // bytes between column panels (tiled: M0 * N0 * elem; row-major: N0 * elem)
+  int32_t out_rows, out_cols;  // rows / columns that exist, from this problem's origin
   int32_t M1, N1, K1;
   int32_t M0, N0;
   int32_t rb;          // bytes per tile row (K0 * element size), power of two
@@ -168,7 +174,7 @@ struct Args {
   uint32_t accumulate;
   uint32_t tail;       // 1 when the last K step is partial
   uint32_t band;       // workgroup rows per rasterization band
-  uint32_t vec_out;    // 1: 4 consecutive columns of a row are contiguous, 16-byte aligned
+  uint32_t vec_out;    // 1: 4 consecutive columns of a row are contiguous (and aligned enough)
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that
@@ -357,33 +363,48 @@ void mmt4d_mfma_kernel(Args a) {
   // contiguously). `vec_out` is 0 when that does not hold or the output is not
   // 16-byte aligned; elements then move one by one.
   Acc acc[TM][TN];
+  // Output element (row, col) of the workgroup's block, with pl = row / M0,
+  // m0 = row % M0, pc = col / N0, n0 = col % N0, lives at
+  //   out + (pm0 + pl) * out_stride + m0 * out_sm0 + (pn0 + pc) * out_spn + n0 * elem,
+  // which covers both the tiled [M1][N1][M0][N0] output and a plain row-major
+  // matrix (the fused mmt4d + unpack). Rows and columns at or beyond
+  // out_rows / out_cols do not exist (row-major output of a ragged problem).
   auto for_each_output = [&](auto f4, auto f1) {
     // The lane coordinates pass through an empty asm so that the address
     // arithmetic of the prologue (ACCUMULATE loads) and of the epilogue
     // (stores) is not shared: shared, it would stay live across the K loop.
     uint32_t oq = q, orr = r;
     asm volatile("" : "+v"(oq), "+v"(orr));
-    char* out_base = a.out + (int64_t)pm0 * a.out_stride + (int64_t)pn0 * a.M0 * a.N0 * OB;
-    const uint32_t tile_bytes = (uint32_t)(a.M0 * a.N0 * OB);
+    char* out_base = a.out + (int64_t)pm0 * a.out_stride + (int64_t)pn0 * a.out_spn;
+    const int row_origin = pm0 * a.M0, col_origin = pn0 * a.N0;
     if (a.vec_out) {
       uint32_t col_off[TN];
-      bool col_ok[TN];
+      int col_n[TN];  // how many of the 4 columns exist
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
         const int col = (wn * TN + tn) * 16 + 4 * (int)oq;
         const int pl = col / a.N0, n0 = col - pl * a.N0;
-        col_ok[tn] = pl < a.bpn && pn0 + pl < a.N1;
-        col_off[tn] = (uint32_t)pl * tile_bytes + (uint32_t)n0 * OB;
+        const bool ok = pl < a.bpn && pn0 + pl < a.N1;
+        const int left = a.out_cols - (col_origin + col);
+        col_n[tn] = ok ? (left >= 4 ? 4 : (left > 0 ? left : 0)) : 0;
+        col_off[tn] = (uint32_t)pl * a.out_spn + (uint32_t)n0 * OB;
       }
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
         const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
-        const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
-        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * OB);
+        const bool row_ok = pl < a.bpm && pm0 + pl < a.M1 && row_origin + row < a.out_rows;
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)m0 * a.out_sm0;
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
-          if (row_ok && col_ok[tn]) f4(tm, tn, out_base + (row_off + col_off[tn]));
+          if (row_ok && col_n[tn] == 4) {
+            f4(tm, tn, out_base + (row_off + col_off[tn]));
+          } else if (row_ok && col_n[tn] > 0) {
+            // the matrix ends inside this group of four columns
+#pragma unroll
+            for (int e = 0; e < 3; ++e)
+              if (e < col_n[tn]) f1(tm, tn, e, out_base + (row_off + col_off[tn] + e * OB));
+          }
         }
         // Keep the unrolled rows from being hoisted together.
         __builtin_amdgcn_sched_barrier(0);
@@ -393,16 +414,16 @@ void mmt4d_mfma_kernel(Args a) {
       for (int tm = 0; tm < TM; ++tm) {
         const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
-        const bool row_ok = pl < a.bpm && pm0 + pl < a.M1;
-        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)(m0 * a.N0 * OB);
+        const bool row_ok = pl < a.bpm && pm0 + pl < a.M1 && row_origin + row < a.out_rows;
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)m0 * a.out_sm0;
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int col = (wn * TN + tn) * 16 + 4 * (int)oq + e;
             const int pc = col / a.N0, n0 = col - pc * a.N0;
-            if (row_ok && pc < a.bpn && pn0 + pc < a.N1)
-              f1(tm, tn, e, out_base + (row_off + (uint32_t)pc * tile_bytes + (uint32_t)n0 * OB));
+            if (row_ok && pc < a.bpn && pn0 + pc < a.N1 && col_origin + col < a.out_cols)
+              f1(tm, tn, e, out_base + (row_off + (uint32_t)pc * a.out_spn + (uint32_t)n0 * OB));
           }
           __builtin_amdgcn_sched_barrier(0);
         }

@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <climits>
 
 #include "mmt4d_mfma_kernel.h"
 #include "uk_device_common.h"
@@ -20,7 +21,12 @@ struct Problem {
   const char* lhs;
   const char* rhs;
   char* out;
-  int64_t lhs_stride, rhs_stride, out_stride;  // bytes
+  int64_t lhs_stride, rhs_stride, out_stride;  // bytes between row panels
+  // Output addressing beyond the panel stride (see Args in the kernel header):
+  // bytes between rows inside a panel and between column panels, and how many
+  // rows / columns exist counted from this problem's origin.
+  int64_t out_sm0, out_spn;
+  int64_t out_rows, out_cols;
   int32_t M1, N1, K1, M0, N0;
   int32_t rb, lrb;  // bytes per tile row and its log2
   bool accumulate;
@@ -44,6 +50,10 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   a.lhs_stride = p.lhs_stride;
   a.rhs_stride = p.rhs_stride;
   a.out_stride = p.out_stride;
+  a.out_sm0 = (uint32_t)p.out_sm0;
+  a.out_spn = (uint32_t)p.out_spn;
+  a.out_rows = (int32_t)std::min<int64_t>(p.out_rows, INT32_MAX);
+  a.out_cols = (int32_t)std::min<int64_t>(p.out_cols, INT32_MAX);
   a.M1 = p.M1; a.N1 = p.N1; a.K1 = kt_count;
   a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
   a.bpm = SH::BM / p.M0;
@@ -60,16 +70,20 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   a.accumulate = accumulate;
   a.band = 4;
   // Four consecutive output columns of one row are contiguous when they lie in
-  // one tile row (N0 % 4 == 0), or when tiles are single rows (M0 == 1: the
-  // tiles of a row then follow each other) and the row ends on a multiple of 4.
-  a.vec_out = (p.N0 % 4 == 0 || (p.M0 == 1 && ((int64_t)p.N1 * p.N0) % 4 == 0)) &&
-              ((uintptr_t)p.out % (4 * ElemTraits<E>::Out::kOutBytes)) == 0 &&
-              p.out_stride % (4 * ElemTraits<E>::Out::kOutBytes) == 0;
+  // one tile row (N0 % 4 == 0) or when column panels follow each other without
+  // a gap (row-major output, or tiles that are single rows). 4-byte outputs
+  // need no more alignment than their own; 2-byte outputs move as 8-byte
+  // vectors and need that alignment.
+  constexpr int OB = ElemTraits<E>::Out::kOutBytes;
+  const bool contiguous4 = p.N0 % 4 == 0 || p.out_spn == (int64_t)p.N0 * OB;
+  const bool aligned4 = OB == 4 || (((uintptr_t)p.out | (uint64_t)p.out_stride |
+                                     (uint64_t)p.out_sm0 | (uint64_t)p.out_spn) % 8) == 0;
+  a.vec_out = contiguous4 && aligned4;
   // 32-bit offsets inside a workgroup's share of each operand.
   const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
   const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
-  constexpr int OB = ElemTraits<E>::Out::kOutBytes;
-  const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.N1 * p.M0 * p.N0 * OB;
+  const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.M0 * p.out_sm0 +
+                         (int64_t)p.N1 * p.out_spn;
   if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31)) return -1;
   auto kernel = mmt4d_mfma_kernel<E, RBC, TM, TN, WGM, WGN, NKK, PIPE>;
   if (SH::kLdsBytes > 64 * 1024) {
@@ -165,7 +179,8 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
       if (split_n) {  // columns [main_n, N1), all rows
         q = p;
         q.rhs = p.rhs + (int64_t)main_n * p.rhs_stride;
-        q.out = p.out + (int64_t)main_n * p.M0 * p.N0 * ElemTraits<E>::Out::kOutBytes;
+        q.out = p.out + (int64_t)main_n * p.out_spn;
+        q.out_cols = p.out_cols - (int64_t)main_n * p.N0;
         q.N1 = p.N1 - main_n;
         st = launch_class<E, RBC>(q, 0, stream, &strip_name);
         // The main part has run: "not served" must not reach the caller, who
@@ -176,6 +191,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         q = p;
         q.lhs = p.lhs + (int64_t)main_m * p.lhs_stride;
         q.out = p.out + (int64_t)main_m * p.out_stride;
+        q.out_rows = p.out_rows - (int64_t)main_m * p.M0;
         q.M1 = p.M1 - main_m;
         q.N1 = main_n;
         st = launch_class<E, RBC>(q, 0, stream, &strip_name);

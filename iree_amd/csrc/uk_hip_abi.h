@@ -25,7 +25,18 @@ int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* params,
 int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* params,
                                   void* stream, int kernel_mode,
                                   const char** kernel_name);
+/* Where an mmt4d result goes when it is not the tiled [M][N][M0][N0] buffer
+ * that the params describe: a row-major matrix of size0 x size1 elements,
+ * `stride0` elements between rows, starting at out_buffer + out_offset (the
+ * fused mmt4d + unpack). Elements of tiles beyond size0 x size1 are dropped. */
+typedef struct iree_uk_amd_rowmajor_out_t {
+  int64_t stride0;
+  int64_t size0, size1;
+} iree_uk_amd_rowmajor_out_t;
+
+/* `rowmajor` NULL: the result is stored tiled, as iree_uk_mmt4d does. */
 int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* params,
+                                 const iree_uk_amd_rowmajor_out_t* rowmajor,
                                  void* stream, int kernel_mode,
                                  const char** kernel_name);
 

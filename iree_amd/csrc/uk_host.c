@@ -251,15 +251,11 @@ uint32_t iree_uk_mmt4d_info(int32_t M0, int32_t N0, int32_t K0, uint32_t flags,
   return iree_uk_mmt4d_info_p(&params);
 }
 
-void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
-  tls_status = 0;
-  tls_kernel_name = "";
-  if (!mmt4d_validate(params)) return;
-  /* mmt4d.c:106-114 */
-  if (params->M == 0 || params->N == 0 ||
-      (params->K == 0 && (params->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE))) {
-    return;
-  }
+/* Runs a validated call. `rowmajor` NULL: the tiled result of iree_uk_mmt4d;
+ * otherwise the result goes to the row-major matrix it describes (at
+ * out_buffer + out_offset) and params->out_stride0 is not used. */
+static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
+                      const iree_uk_amd_rowmajor_out_t* rowmajor) {
   /* mmt4d.c:126-139: without the fallback flag only an architecture-specific
    * (here: MFMA) kernel may serve the call. */
   if (!(params->flags &
@@ -272,6 +268,8 @@ void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
   mmt4d_bits_t bits;
   mmt4d_type_bits(params->flags, &bits);
   iree_uk_mmt4d_params_t p = *params;
+  iree_uk_amd_rowmajor_out_t rm;
+  if (rowmajor) rm = *rowmajor;
   const int out_bytes = bits.out_bits / 8;
   staged_t lhs = {(char*)p.lhs_buffer + p.lhs_offset * bits.lhs_bits / 8,
                   p.lhs_stride0 * bits.lhs_bits / 8,
@@ -282,6 +280,11 @@ void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
   staged_t out = {(char*)p.out_buffer + p.out_offset * out_bytes,
                   p.out_stride0 * out_bytes, p.N * p.M0 * p.N0 * out_bytes,
                   p.M, 0};
+  if (rowmajor) {
+    out.pitch = rm.stride0 * out_bytes;
+    out.row_bytes = rm.size1 * out_bytes;
+    out.rows = rm.size0;
+  }
   int st = stage_in(&lhs, 1);
   if (!st) st = stage_in(&rhs, 1);
   if (!st) {
@@ -302,9 +305,10 @@ void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
       p.out_buffer = out.device;
       p.out_offset = 0;
       p.out_stride0 = p.N * p.M0 * p.N0;
+      rm.stride0 = rm.size1;
     }
-    st = iree_uk_amd_hip_launch_mmt4d(&p, tls_stream, tls_kernel_mode,
-                                      &tls_kernel_name);
+    st = iree_uk_amd_hip_launch_mmt4d(&p, rowmajor ? &rm : 0, tls_stream,
+                                      tls_kernel_mode, &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
   if (lhs.device || rhs.device || out.device) {
@@ -315,6 +319,65 @@ void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
   stage_free(&rhs);
   stage_free(&out);
   tls_status = st;
+}
+
+void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
+  tls_status = 0;
+  tls_kernel_name = "";
+  if (!mmt4d_validate(params)) return;
+  /* mmt4d.c:106-114 */
+  if (params->M == 0 || params->N == 0 ||
+      (params->K == 0 && (params->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE))) {
+    return;
+  }
+  mmt4d_run(params, 0);
+}
+
+/* Fused mmt4d + unpack: validation is that of the two calls it stands for. */
+static int mmt4d_unpack_validate(const iree_uk_amd_mmt4d_unpack_params_t* p,
+                                 const iree_uk_mmt4d_params_t* mm) {
+  if (!mmt4d_validate(mm)) return 0;
+  UK_REQUIRE(p->out_size0 >= 0 && p->out_size0 <= p->M * p->M0);
+  UK_REQUIRE(p->out_size1 >= 0 && p->out_size1 <= p->N * p->N0);
+  return 1;
+}
+
+void iree_uk_amd_mmt4d_unpack_p(const iree_uk_amd_mmt4d_unpack_params_t* params) {
+  tls_status = 0;
+  tls_kernel_name = "";
+  const iree_uk_mmt4d_params_t mm = {
+      params->lhs_buffer, params->lhs_offset, params->lhs_stride0,
+      params->rhs_buffer, params->rhs_offset, params->rhs_stride0,
+      params->out_buffer, params->out_offset, /*out_stride0=*/0,
+      params->M, params->N, params->K, params->M0, params->N0, params->K0,
+      params->flags, params->cpu_data};
+  if (!mmt4d_unpack_validate(params, &mm)) return;
+  /* The early returns of the two calls (mmt4d.c:106-114, unpack.c:84-86). */
+  if (params->M == 0 || params->N == 0 || params->out_size0 == 0 ||
+      params->out_size1 == 0 ||
+      (params->K == 0 && (params->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE))) {
+    return;
+  }
+  const iree_uk_amd_rowmajor_out_t rm = {params->out_stride0, params->out_size0,
+                                         params->out_size1};
+  mmt4d_run(&mm, &rm);
+}
+
+void iree_uk_amd_mmt4d_unpack(const void* lhs_buffer, iree_uk_index_t lhs_offset,
+                              iree_uk_index_t lhs_stride0, const void* rhs_buffer,
+                              iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0,
+                              void* out_buffer, iree_uk_index_t out_offset,
+                              iree_uk_index_t out_stride0, iree_uk_index_t out_size0,
+                              iree_uk_index_t out_size1, iree_uk_index_t M,
+                              iree_uk_index_t N, iree_uk_index_t K, int32_t M0,
+                              int32_t N0, int32_t K0, uint32_t flags,
+                              const uint64_t* cpu_data) {
+  iree_uk_amd_mmt4d_unpack_params_t params = {
+      lhs_buffer, lhs_offset, lhs_stride0, rhs_buffer, rhs_offset, rhs_stride0,
+      out_buffer, out_offset, out_stride0, out_size0,  out_size1,  M,
+      N,          K,          M0,          N0,         K0,         flags,
+      cpu_data};
+  iree_uk_amd_mmt4d_unpack_p(&params);
 }
 
 void iree_uk_mmt4d(const void* lhs_buffer, iree_uk_index_t lhs_offset,

@@ -146,6 +146,18 @@ class Runner:
         nbytes = (M1 * K1 * M0 * K0 + N1 * K1 * N0 * K0) * in_es + out_bytes
         return Op("mmt4d", launch, 2.0 * M * N * K, float(nbytes), "mfma", dtype)
 
+    def _mmt4d_unpack_op(self, lhs4, rhs4, out, M, N, M1, N1, K1, M0, N0, K0, type_flag, dtype,
+                         in_es):
+        """The fused call: operands tiled, result row-major M x N."""
+        lib = self.lib
+        lp, rp, op_ = lhs4.data_ptr(), rhs4.data_ptr(), out.data_ptr()
+
+        def launch():
+            lib.mmt4d_unpack(lp, 0, K1 * M0 * K0, rp, 0, K1 * N0 * K0, op_, 0, N, M, N,
+                             M1, N1, K1, M0, N0, K0, type_flag)
+        nbytes = (M1 * K1 * M0 * K0 + N1 * K1 * N0 * K0) * in_es + M * N * 4
+        return Op("mmt4d", launch, 2.0 * M * N * K1 * K0, float(nbytes), "mfma", dtype)
+
     # --------------------------------------------------------------- workloads
     def workload(self, name: str) -> Workload:
         torch = self.torch
@@ -168,6 +180,24 @@ class Runner:
                             ops, 2.0 * M * N * K, sum(o.bytes for o in ops), "f16",
                             dict(a=a, bt=bt, lhs4=lhs4, rhs4=rhs4, out4=out4, out=out,
                                  M=M, N=N, K=K, M0=M0, N0=N0, K0=K0))
+        if name in ("c2_f16_fused_4096", "c2_f16_fused_ragged"):
+            # The same chain with the fused mmt4d + unpack entry point.
+            M, N, K = (4096, 4096, 4096) if name.endswith("4096") else (4095, 4097, 4096)
+            M0 = N0 = K0 = 16
+            M1, N1, K1 = -(-M // M0), -(-N // N0), K // K0
+            a = self.normal((M, K), torch.float16, 1)
+            bt = self.normal((N, K), torch.float16, 2)
+            lhs4 = self.empty(M1 * K1 * M0 * K0, torch.float16)
+            rhs4 = self.empty(N1 * K1 * N0 * K0, torch.float16)
+            out = self.empty(M * N, torch.float32)
+            ops = [self._pack_op("pack_lhs", a, M, K, lhs4, M0, K0, uk.PACK_TYPE_F16F16, 2),
+                   self._pack_op("pack_rhs", bt, N, K, rhs4, N0, K0, uk.PACK_TYPE_F16F16, 2),
+                   self._mmt4d_unpack_op(lhs4, rhs4, out, M, N, M1, N1, K1, M0, N0, K0,
+                                         uk.MMT4D_TYPE_F16F16F32, "f16", 2)]
+            return Workload(name, f"pack->fused mmt4d+unpack f16xf16->f32 M={M} N={N} K={K} "
+                            "tiles 16x16x16", ops, 2.0 * M * N * K, sum(o.bytes for o in ops),
+                            "f16", dict(a=a, bt=bt, lhs4=lhs4, rhs4=rhs4, out=out, M=M, N=N, K=K,
+                                        M0=M0, N0=N0, K0=K0))
         if name.startswith("s8_mmt4d_"):
             # s8_mmt4d_<size>_k<K0>, tiles 16x16xK0, packed operands filled directly.
             _, _, size, k0 = name.split("_")

@@ -138,6 +138,10 @@ class UKernelLibrary:
                                      _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                      _u32, _vp]
         L.iree_uk_unpack.restype = None
+        L.iree_uk_amd_mmt4d_unpack.argtypes = [_vp, _i64, _i64, _vp, _i64, _i64, _vp,
+                                               _i64, _i64, _i64, _i64, _i64, _i64,
+                                               _i64, _i32, _i32, _i32, _u32, _vp]
+        L.iree_uk_amd_mmt4d_unpack.restype = None
         L.iree_uk_amd_last_status.restype = ctypes.c_int
         L.iree_uk_amd_last_status_string.restype = ctypes.c_char_p
         L.iree_uk_amd_last_kernel_name.restype = ctypes.c_char_p
@@ -183,6 +187,16 @@ class UKernelLibrary:
                                 out_offset, out_stride0, out_stride1, in_size0,
                                 in_size1, in_size2, in_size3, out_size0,
                                 out_size1, flags, cpu_data)
+        self._check()
+
+    def mmt4d_unpack(self, lhs, lhs_offset, lhs_stride0, rhs, rhs_offset, rhs_stride0,
+                     out, out_offset, out_stride0, out_size0, out_size1, M, N, K,
+                     M0, N0, K0, flags, cpu_data=None):
+        """mmt4d straight into a row-major out_size0 x out_size1 matrix."""
+        self.lib.iree_uk_amd_mmt4d_unpack(lhs, lhs_offset, lhs_stride0, rhs, rhs_offset,
+                                          rhs_stride0, out, out_offset, out_stride0,
+                                          out_size0, out_size1, M, N, K, M0, N0, K0,
+                                          flags, cpu_data)
         self._check()
 
     # --------------------------------------------------------------- control

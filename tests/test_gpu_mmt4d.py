@@ -276,3 +276,53 @@ def test_entry_points_from_concurrent_threads(gpu, oracle):
     assert np.array_equal(got_host[rows * tile_row:], out0[rows * tile_row:])   # other slabs untouched
     assert np.array_equal(got_dev[rows * tile_row:], want[rows * tile_row:])
     assert np.array_equal(got_dev[:rows * tile_row], out0[:rows * tile_row])
+
+
+@pytest.mark.parametrize("mode", [uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_GENERIC,
+                                  uk.KERNEL_MODE_MFMA_VARIANT + 1])
+@pytest.mark.parametrize("tf,M0,N0,K0", [
+    (uk.MMT4D_TYPE_S8S8S32, 16, 16, 16), (uk.MMT4D_TYPE_S8S8S32, 16, 16, 2),
+    (uk.MMT4D_TYPE_S8S8S32, 8, 32, 4), (uk.MMT4D_TYPE_F16F16F32, 16, 16, 8),
+    (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1), (uk.MMT4D_TYPE_S16S16S32, 4, 6, 3)])
+def test_fused_mmt4d_unpack_equals_the_two_calls(gpu, oracle, tf, M0, N0, K0, mode):
+    """iree_uk_amd_mmt4d_unpack == mmt4d into a tiled temporary + unpack of it,
+    bit for bit (inputs are the reference tests' small integers, so every f32
+    partial sum is exact), including ragged sizes, loose row pitch, a nonzero
+    offset, ACCUMULATE, and bytes outside the matrix left untouched."""
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    lk, rk, ok = T.MMT4D_KINDS[tf]
+    unpack_tf = uk.UNPACK_TYPE_I32I32 if ok == "s32" else uk.UNPACK_TYPE_F32F32
+    shapes = [(3, 2, 5, 0, 0), (17, 18, 9, 5, 3), (1, 1, 1, 0, 15), (33, 5, 40, 15, 0)]
+    for si, (M1, N1, K1, cut0, cut1) in enumerate(shapes):
+        for acc in (0, 1):
+            rows, cols = M1 * M0 - min(cut0, M0 - 1), N1 * N0 - min(cut1, N0 - 1)
+            pitch, off = cols + 16 * (si % 2), 16 * ((si + acc) % 2)
+            c = T.Mmt4dCase(tf | 0x200 | (uk.MMT4D_ACCUMULATE if acc else 0), M1, N1, K1, M0, N0,
+                            K0, K1 * M0 * K0, K1 * N0 * K0, N1 * M0 * N0, 0, 0, 0)
+            rng = np.random.default_rng(100 * si + acc)
+            lhs, rhs, _ = T.make_mmt4d_buffers(c, rng)
+            out0 = rng.integers(-9, 9, off + rows * pitch).astype(np.int32)
+            if ok != "s32":
+                out0 = out0.astype(np.float32).view(np.int32)
+            # oracle: pack the accumulator matrix, mmt4d, unpack
+            tiled = np.zeros(M1 * N1 * M0 * N0, np.int32)
+            if acc:
+                oracle.pack(out0, off, pitch, 1, tiled, 0, N1 * M0 * N0, M0 * N0, rows, cols,
+                            M1, N1, M0, N0, 0, uk.PACK_TYPE_I32I32)
+            G.run_mmt4d_case(oracle, c, lhs, rhs, tiled.view(np.uint8))
+            want = out0.copy()
+            oracle.unpack(tiled, 0, N1 * M0 * N0, M0 * N0, want, off, pitch, 1, M1, N1, M0, N0,
+                          rows, cols, unpack_tf)
+            d = [T.DeviceBytes(torch, x) for x in (lhs, rhs, out0)]
+            lib.mmt4d_unpack(d[0].ptr, 0, c.lhs_stride0, d[1].ptr, 0, c.rhs_stride0, d[2].ptr, off,
+                             pitch, rows, cols, M1, N1, K1, M0, N0, K0, c.flags)
+            lib.synchronize()
+            got = d[2].numpy().view(np.int32)
+            assert np.array_equal(got, want), (tf, M0, N0, K0, M1, N1, K1, acc, lib.last_kernel_name())
+            # host pointers (staged) give the same
+            host = out0.copy()
+            lib.mmt4d_unpack(lhs.ctypes.data, 0, c.lhs_stride0, rhs.ctypes.data, 0, c.rhs_stride0,
+                             host.ctypes.data, off, pitch, rows, cols, M1, N1, K1, M0, N0, K0,
+                             c.flags)
+            assert np.array_equal(host, want)
