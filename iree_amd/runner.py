@@ -310,7 +310,14 @@ class Runner:
         on the launch stream (iree_uk_amd_timing_begin/end), which timestamps
         the kernel itself."""
         torch = self.torch
+        import time
         with torch.cuda.stream(self.stream):
+            # Same clock-settle phase as run_steps, then the warm-up launches.
+            t_settle = time.perf_counter()
+            while time.perf_counter() - t_settle < self.settle_seconds:
+                for _ in range(4):
+                    op.launch()
+                self.stream.synchronize()
             for _ in range(warmup):
                 op.launch()
             op.kernel = self.lib.last_kernel_name()
