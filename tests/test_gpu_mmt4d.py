@@ -326,3 +326,42 @@ def test_fused_mmt4d_unpack_equals_the_two_calls(gpu, oracle, tf, M0, N0, K0, mo
                              host.ctypes.data, off, pitch, rows, cols, M1, N1, K1, M0, N0, K0,
                              c.flags)
             assert np.array_equal(host, want)
+
+
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_fused_mmt4d_unpack_with_remainder_strips(gpu, accumulate):
+    """A shape large enough for the 256x256 variant and ragged against it in M
+    and N (so the strips are split off), with a K remainder: the fused call
+    must equal mmt4d + unpack on the GPU (both halves are pinned against the
+    oracle by the tests above) and, on a sample of rows, the integer product."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    M1, N1, K1, M0, N0, K0 = 241, 273, 5, 16, 16, 16
+    rows, cols = M1 * M0 - 3, N1 * N0 - 5
+    g = torch.Generator(device="cuda"); g.manual_seed(7)
+    lhs = torch.randint(-128, 128, (M1, K1, M0, K0), generator=g, device="cuda", dtype=torch.int8)
+    rhs = torch.randint(-128, 128, (N1, K1, N0, K0), generator=g, device="cuda", dtype=torch.int8)
+    init = torch.randint(-1000, 1000, (rows, cols), generator=g, device="cuda", dtype=torch.int32)
+    flags = uk.MMT4D_TYPE_S8S8S32 | (uk.MMT4D_ACCUMULATE if accumulate else 0)
+    # the two reference calls (accumulator packed first when accumulating)
+    tiled = torch.zeros(M1 * N1 * M0 * N0, device="cuda", dtype=torch.int32)
+    if accumulate:
+        lib.pack(init.data_ptr(), 0, cols, 1, tiled.data_ptr(), 0, N1 * M0 * N0, M0 * N0, rows, cols,
+                 M1, N1, M0, N0, 0, uk.PACK_TYPE_I32I32)
+    lib.mmt4d(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, tiled.data_ptr(), 0,
+              N1 * M0 * N0, M1, N1, K1, M0, N0, K0, flags)
+    assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256")
+    want = init.clone()
+    lib.unpack(tiled.data_ptr(), 0, N1 * M0 * N0, M0 * N0, want.data_ptr(), 0, cols, 1, M1, N1, M0, N0,
+               rows, cols, uk.UNPACK_TYPE_I32I32)
+    got = init.clone()
+    lib.mmt4d_unpack(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, got.data_ptr(),
+                     0, cols, rows, cols, M1, N1, K1, M0, N0, K0, flags)
+    assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256")
+    lib.synchronize()
+    assert torch.equal(got, want)
+    # closed form on the last rows (they cross the row strip)
+    a = lhs.permute(0, 2, 1, 3).reshape(M1 * M0, K1 * K0)[rows - 40:rows].cpu().numpy().astype(np.int64)
+    b = rhs.permute(0, 2, 1, 3).reshape(N1 * N0, K1 * K0)[:cols].cpu().numpy().astype(np.int64)
+    ref = a @ b.T + (init[rows - 40:].cpu().numpy() if accumulate else 0)
+    assert np.array_equal(got[rows - 40:].cpu().numpy(), ref.astype(np.int32))
