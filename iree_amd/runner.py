@@ -34,6 +34,7 @@ class Op:
     bound: str = "hbm"        # "hbm" | "mfma"
     dtype: str = ""
     kernel: str = ""          # filled after the first launch
+    external: bool = False    # True: not a ukernel call (a harness-side torch op)
 
 
 @dataclasses.dataclass
@@ -264,10 +265,28 @@ class Runner:
                                 uk.MMT4D_TYPE_S8S8S32, "s8", 1, accumulate=True,
                                 logical=(Mlog, N, K))
             op.bound = "hbm"
-            return Workload(name, "mmt4d s8 decode M=16(32) K=4096 N=14336 tiles 32x16x8 ACCUMULATE",
-                            [op], op.flops, op.bytes, "s8",
-                            dict(act=act, w=w, lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1,
-                                 K1=K1, M0=M0, N0=N0, K0=K0))
+            # The layer's epilogue is not a ukernel: per-row (activation) and
+            # per-column (weight) scales applied to the s32 accumulators of the
+            # 16 real rows, out[m][n] = float(acc[m][n]) * scale_m[m] * scale_n[n],
+            # as one torch expression on the tiled buffer.
+            scale_m = torch.rand(Mlog, generator=self._gen(15), device="cuda") * 0.02 + 0.001
+            scale_n = torch.rand(N, generator=self._gen(16), device="cuda") * 0.02 + 0.001
+            y = torch.empty(Mlog, N, device="cuda", dtype=torch.float32)
+            acc_view = out4.view(N1, M0, N0)[:, :Mlog, :].permute(1, 0, 2)  # [m][n1][n0]
+            scale = (scale_m[:, None] * scale_n[None, :]).view(Mlog, N1, N0)
+            y_view = y.view(Mlog, N1, N0)
+            stream = self.stream
+
+            def epilogue():
+                with torch.cuda.stream(stream):
+                    torch.mul(acc_view, scale, out=y_view)  # one kernel: s32 * f32 -> f32
+            ep = Op("scale_epilogue", epilogue, 0.0, float(Mlog * N * 8), "hbm", "f32",
+                    kernel="torch (harness, not a ukernel)", external=True)
+            return Workload(name, "mmt4d s8 decode M=16(32) K=4096 N=14336 tiles 32x16x8 ACCUMULATE "
+                            "+ per-row/per-column scale epilogue",
+                            [op, ep], op.flops, op.bytes, "s8",
+                            dict(act=act, w=w, lhs4=lhs4, rhs4=rhs4, out4=out4, y=y, scale_m=scale_m,
+                                 scale_n=scale_n, M1=M1, N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
         if name == "c4_f8_prefill":
             M, K, N = 2048, 8192, 28672
             M0, N0, K0 = 16, 16, 32
@@ -311,6 +330,19 @@ class Runner:
         the kernel itself."""
         torch = self.torch
         import time
+        if op.external:
+            with torch.cuda.stream(self.stream):
+                for _ in range(warmup):
+                    op.launch()
+                evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                       for _ in range(iters)]
+                for a, b in evs:
+                    a.record(self.stream)
+                    op.launch()
+                    b.record(self.stream)
+            self.stream.synchronize()
+            us = [a.elapsed_time(b) * 1e3 for a, b in evs]
+            return sum(us) / len(us), min(us), sorted(us)[len(us) // 2]
         with torch.cuda.stream(self.stream):
             # Same clock-settle phase as run_steps, then the warm-up launches.
             t_settle = time.perf_counter()
@@ -372,10 +404,10 @@ class Runner:
             for _ in range(warmup):
                 for op in wl.ops:
                     op.launch()
-                    op.kernel = self.lib.last_kernel_name()
             for op in wl.ops:
                 op.launch()
-                op.kernel = self.lib.last_kernel_name()
+                if not op.external:
+                    op.kernel = self.lib.last_kernel_name()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(steps):
