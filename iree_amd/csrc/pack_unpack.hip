@@ -807,6 +807,10 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
     // widen along dim 1 (more, longer 2-D row segments) up to the target
     while (G0 * G1 * tile_bytes * 2 <= kTarget) G1 *= 2;
   } else {
+    // Tiles of one tile row are contiguous on the tiled side, so widening
+    // along dim 1 lengthens the segments of both sides; do that up to 1 KB of
+    // matrix row, then add tile rows.
+    while (G0 * G1 * tile_bytes * 2 <= kTarget && G1 * v.tile1 * es < 1024 && G1 < v.outer1) G1 *= 2;
     while (G0 * G1 * tile_bytes * 2 <= kTarget) G0 *= 2;
   }
   G0 = std::min<int64_t>(G0, std::max<int64_t>(v.outer0, 1));
