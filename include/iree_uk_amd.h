@@ -345,6 +345,88 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);
 IREE_UK_AMD_EXPORT const char* iree_uk_amd_version(void);
 
 /*===----------------------------------------------------------------------===*/
+/* conv_nchwc                                                                  */
+/*===----------------------------------------------------------------------===*/
+
+/* The convolution ukernel of the same reference library
+ * (runtime/src/iree/builtins/ukernel/conv_nchwc.h:14-31), kept so that the
+ * library stands in for all of iree/builtins/ukernel/api.h. It is served by a
+ * scalar kernel (one thread per output element, the reference's accumulation
+ * order): correct for every shape, not tuned.
+ *
+ * input [N][IC_outer][IH][IW][c0], filter [OC_outer][IC_outer][FH][FW][c0][k0],
+ * output [N][OC_outer][OH][OW][k0]; the named strides are in elements.
+ * Flag values: exported_bits.h:113-124. */
+enum {
+  IREE_UK_FLAG_CONV_NCHWC_TYPE_MASK = 0xFF,
+  IREE_UK_FLAG_CONV_NCHWC_TYPE_NONE = 0x00,
+  IREE_UK_FLAG_CONV_NCHWC_TYPE_F32F32F32 = 0x01,
+  IREE_UK_FLAG_CONV_NCHWC_TYPE_END = 0x02,
+  IREE_UK_FLAG_CONV_NCHWC_ACCUMULATE = 0x100,
+  IREE_UK_FLAG_CONV_NCHWC_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION = 0x200,
+  IREE_UK_FLAG_CONV_NCHWC_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION = 0x1,
+};
+
+/* Replaces iree_uk_conv_nchwc_params_t (conv_nchwc_internal.h:12-46); field
+ * order is the reference's, `ow_count` (a per-tile value its driver loop sets)
+ * included and ignored. */
+typedef struct iree_uk_conv_nchwc_params_t {
+  const void* input_buffer;
+  iree_uk_index_t input_offset;
+  iree_uk_index_t input_stride_n;
+  iree_uk_index_t input_stride_ic_outer;
+  iree_uk_index_t input_stride_h;
+  const void* filter_buffer;
+  iree_uk_index_t filter_offset;
+  iree_uk_index_t filter_stride_oc_outer;
+  iree_uk_index_t filter_stride_ic_outer;
+  iree_uk_index_t filter_stride_fh;
+  void* output_buffer;
+  iree_uk_index_t output_offset;
+  iree_uk_index_t output_stride_n;
+  iree_uk_index_t output_stride_oc_outer;
+  iree_uk_index_t output_stride_oh;
+  iree_uk_index_t N;
+  iree_uk_index_t OC_outer;
+  iree_uk_index_t OH;
+  iree_uk_index_t OW;
+  iree_uk_index_t IC_outer;
+  iree_uk_index_t FH;
+  iree_uk_index_t FW;
+  int32_t k0;
+  int32_t c0;
+  int32_t stride_h;
+  int32_t stride_w;
+  uint32_t flags;
+  iree_uk_index_t ow_count;
+  const uint64_t* cpu_data;
+} iree_uk_conv_nchwc_params_t;
+
+/* Replaces iree_uk_conv_nchwc (conv_nchwc.h:14-27, conv_nchwc.c:157-198). */
+IREE_UK_AMD_EXPORT void iree_uk_conv_nchwc(
+    const void* input_buffer, iree_uk_index_t input_offset,
+    iree_uk_index_t input_stride_n, iree_uk_index_t input_stride_ic_outer,
+    iree_uk_index_t input_stride_h, const void* filter_buffer,
+    iree_uk_index_t filter_offset, iree_uk_index_t filter_stride_oc_outer,
+    iree_uk_index_t filter_stride_ic_outer, iree_uk_index_t filter_stride_fh,
+    void* output_buffer, iree_uk_index_t output_offset,
+    iree_uk_index_t output_stride_n, iree_uk_index_t output_stride_oc_outer,
+    iree_uk_index_t output_stride_oh, iree_uk_index_t N,
+    iree_uk_index_t OC_outer, iree_uk_index_t OH, iree_uk_index_t OW,
+    iree_uk_index_t IC_outer, iree_uk_index_t FH, iree_uk_index_t FW,
+    int32_t k0, int32_t c0, int32_t stride_h, int32_t stride_w, uint32_t flags,
+    const uint64_t* cpu_data);
+/* Replaces iree_uk_conv_nchwc_p (conv_nchwc_internal.h:48, conv_nchwc.c:132-155). */
+IREE_UK_AMD_EXPORT void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params);
+/* Replace iree_uk_conv_nchwc_info (conv_nchwc.h:29-31, conv_nchwc.c:210-218) and
+ * iree_uk_conv_nchwc_info_p (conv_nchwc.c:200-208): 0, there is no tuned
+ * kernel, so callers must pass ALLOW_GENERIC_FALLBACK_TILE_FUNCTION. */
+IREE_UK_AMD_EXPORT uint32_t iree_uk_conv_nchwc_info(int32_t k0, int32_t c0, uint32_t flags,
+                                                    const uint64_t* cpu_data);
+IREE_UK_AMD_EXPORT uint32_t iree_uk_conv_nchwc_info_p(
+    const iree_uk_conv_nchwc_params_t* params);
+
+/*===----------------------------------------------------------------------===*/
 /* Fused mmt4d + unpack                                                        */
 /*===----------------------------------------------------------------------===*/
 

@@ -588,6 +588,130 @@ void iree_uk_unpack(const void* in_buffer, iree_uk_index_t in_offset,
 }
 
 /*---------------------------------------------------------------------------
+ * conv_nchwc
+ *-------------------------------------------------------------------------*/
+
+/* conv_nchwc.c:12-40 */
+static int conv_nchwc_validate(const iree_uk_conv_nchwc_params_t* p) {
+  const uint32_t allflags =
+      IREE_UK_FLAG_CONV_NCHWC_TYPE_MASK | IREE_UK_FLAG_CONV_NCHWC_ACCUMULATE |
+      IREE_UK_FLAG_CONV_NCHWC_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION;
+  UK_REQUIRE(!(p->flags & ~allflags));
+  const uint32_t type_bits = p->flags & IREE_UK_FLAG_CONV_NCHWC_TYPE_MASK;
+  UK_REQUIRE(type_bits > 0 && type_bits < IREE_UK_FLAG_CONV_NCHWC_TYPE_END);
+  UK_REQUIRE(fits_unsigned_bits(p->N, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->OC_outer, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->OH, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->OW, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->IC_outer, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->FH, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->FW, 31));
+  UK_REQUIRE(fits_unsigned_bits(p->k0, 15));
+  UK_REQUIRE(fits_unsigned_bits(p->c0, 15));
+  UK_REQUIRE(p->k0 > 0 && p->c0 > 0);
+  UK_REQUIRE(p->stride_h > 0 && p->stride_w > 0);
+  return 1;
+}
+
+uint32_t iree_uk_conv_nchwc_info_p(const iree_uk_conv_nchwc_params_t* params) {
+  (void)params;
+  return 0; /* served by the scalar kernel only */
+}
+
+uint32_t iree_uk_conv_nchwc_info(int32_t k0, int32_t c0, uint32_t flags,
+                                 const uint64_t* cpu_data) {
+  (void)k0; (void)c0; (void)flags; (void)cpu_data;
+  return 0;
+}
+
+void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params) {
+  tls_status = 0;
+  tls_kernel_name = "";
+  if (!conv_nchwc_validate(params)) return;
+  /* conv_nchwc.c:42-53 */
+  if (params->N == 0 || params->OC_outer == 0 || params->OH == 0 ||
+      params->OW == 0) {
+    return;
+  }
+  const int no_taps =
+      params->IC_outer == 0 || params->FH == 0 || params->FW == 0;
+  if (no_taps && (params->flags & IREE_UK_FLAG_CONV_NCHWC_ACCUMULATE)) return;
+  /* conv_nchwc.c:139-152 */
+  if (!(params->flags &
+        IREE_UK_FLAG_CONV_NCHWC_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)) {
+    assert_fail(__FILE__, __LINE__, __func__,
+                "no target-specific tile function, and fallback not enabled.");
+    return;
+  }
+  iree_uk_conv_nchwc_params_t p = *params;
+  /* Host operands are staged as the contiguous element range they span; the
+   * output range travels to the device and back whole, so the elements
+   * between its rows come back as they were. */
+  const int64_t H = (p.OH - 1) * p.stride_h + p.FH;
+  const int64_t W = (p.OW - 1) * p.stride_w + p.FW;
+  const int64_t in_span =
+      no_taps ? 0
+              : (p.N - 1) * p.input_stride_n +
+                    (p.IC_outer - 1) * p.input_stride_ic_outer +
+                    (H - 1) * p.input_stride_h + W * p.c0;
+  const int64_t f_span =
+      no_taps ? 0
+              : (p.OC_outer - 1) * p.filter_stride_oc_outer +
+                    (p.IC_outer - 1) * p.filter_stride_ic_outer +
+                    (p.FH - 1) * p.filter_stride_fh + p.FW * (int64_t)p.c0 * p.k0;
+  const int64_t out_span = (p.N - 1) * p.output_stride_n +
+                           (p.OC_outer - 1) * p.output_stride_oc_outer +
+                           (p.OH - 1) * p.output_stride_oh + p.OW * (int64_t)p.k0;
+  staged_t in = {(char*)p.input_buffer + p.input_offset * 4, in_span * 4,
+                 in_span * 4, in_span > 0 ? 1 : 0, 0};
+  staged_t flt = {(char*)p.filter_buffer + p.filter_offset * 4, f_span * 4,
+                  f_span * 4, f_span > 0 ? 1 : 0, 0};
+  staged_t out = {(char*)p.output_buffer + p.output_offset * 4, out_span * 4,
+                  out_span * 4, 1, 0};
+  int st = stage_in(&in, 1);
+  if (!st) st = stage_in(&flt, 1);
+  if (!st) st = stage_in(&out, 1);
+  if (!st) {
+    if (in.device) { p.input_buffer = in.device; p.input_offset = 0; }
+    if (flt.device) { p.filter_buffer = flt.device; p.filter_offset = 0; }
+    if (out.device) { p.output_buffer = out.device; p.output_offset = 0; }
+    st = iree_uk_amd_hip_launch_conv_nchwc(&p, tls_stream, &tls_kernel_name);
+  }
+  if (!st) st = stage_out(&out);
+  if (in.device || flt.device || out.device) {
+    int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
+    if (!st) st = st2;
+  }
+  stage_free(&in);
+  stage_free(&flt);
+  stage_free(&out);
+  tls_status = st;
+}
+
+void iree_uk_conv_nchwc(
+    const void* input_buffer, iree_uk_index_t input_offset,
+    iree_uk_index_t input_stride_n, iree_uk_index_t input_stride_ic_outer,
+    iree_uk_index_t input_stride_h, const void* filter_buffer,
+    iree_uk_index_t filter_offset, iree_uk_index_t filter_stride_oc_outer,
+    iree_uk_index_t filter_stride_ic_outer, iree_uk_index_t filter_stride_fh,
+    void* output_buffer, iree_uk_index_t output_offset,
+    iree_uk_index_t output_stride_n, iree_uk_index_t output_stride_oc_outer,
+    iree_uk_index_t output_stride_oh, iree_uk_index_t N,
+    iree_uk_index_t OC_outer, iree_uk_index_t OH, iree_uk_index_t OW,
+    iree_uk_index_t IC_outer, iree_uk_index_t FH, iree_uk_index_t FW,
+    int32_t k0, int32_t c0, int32_t stride_h, int32_t stride_w, uint32_t flags,
+    const uint64_t* cpu_data) {
+  iree_uk_conv_nchwc_params_t params = {
+      input_buffer, input_offset, input_stride_n, input_stride_ic_outer,
+      input_stride_h, filter_buffer, filter_offset, filter_stride_oc_outer,
+      filter_stride_ic_outer, filter_stride_fh, output_buffer, output_offset,
+      output_stride_n, output_stride_oc_outer, output_stride_oh, N, OC_outer,
+      OH, OW, IC_outer, FH, FW, k0, c0, stride_h, stride_w, flags,
+      /*ow_count=*/0, cpu_data};
+  iree_uk_conv_nchwc_p(&params);
+}
+
+/*---------------------------------------------------------------------------
  * query_tile_sizes
  *-------------------------------------------------------------------------*/
 

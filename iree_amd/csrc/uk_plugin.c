@@ -1,5 +1,6 @@
 // HAL executable plugin face of the library: lets an unmodified IREE runtime
-// route the `iree_uk_mmt4d`, `iree_uk_pack` and `iree_uk_unpack` imports of
+// route the `iree_uk_mmt4d`, `iree_uk_pack`, `iree_uk_unpack` (and
+// `iree_uk_conv_nchwc`) imports of
 // compiled LLVMCPU programs to the GPU implementation
 // (`--executable_plugin=libiree_uk_amd.so`).
 //
@@ -103,6 +104,35 @@ static int pack_thunk(void* params_ptr, void* context, void* reserved) {
   iree_uk_pack_p(&((const pack_import_t*)params_ptr)->p);
   return iree_uk_amd_last_status() ? 1 : 0;
 }
+/* conv_nchwc: the arguments of the flat entry point in order (the params
+ * struct has one more, internal, field, so it cannot be overlaid). */
+typedef struct {
+  int32_t unused_result;
+  const void* input_buffer;
+  iree_uk_index_t input_offset, input_stride_n, input_stride_ic_outer, input_stride_h;
+  const void* filter_buffer;
+  iree_uk_index_t filter_offset, filter_stride_oc_outer, filter_stride_ic_outer, filter_stride_fh;
+  void* output_buffer;
+  iree_uk_index_t output_offset, output_stride_n, output_stride_oc_outer, output_stride_oh;
+  iree_uk_index_t N, OC_outer, OH, OW, IC_outer, FH, FW;
+  int32_t k0, c0, stride_h, stride_w;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} conv_import_t;
+
+static int conv_thunk(void* params_ptr, void* context, void* reserved) {
+  (void)context; (void)reserved;
+  const conv_import_t* a = (const conv_import_t*)params_ptr;
+  iree_uk_conv_nchwc(a->input_buffer, a->input_offset, a->input_stride_n,
+                     a->input_stride_ic_outer, a->input_stride_h, a->filter_buffer,
+                     a->filter_offset, a->filter_stride_oc_outer, a->filter_stride_ic_outer,
+                     a->filter_stride_fh, a->output_buffer, a->output_offset, a->output_stride_n,
+                     a->output_stride_oc_outer, a->output_stride_oh, a->N, a->OC_outer, a->OH,
+                     a->OW, a->IC_outer, a->FH, a->FW, a->k0, a->c0, a->stride_h, a->stride_w,
+                     a->flags, a->cpu_data);
+  return iree_uk_amd_last_status() ? 1 : 0;
+}
+
 static int unpack_thunk(void* params_ptr, void* context, void* reserved) {
   (void)context; (void)reserved;
   iree_uk_unpack_p(&((const unpack_import_t*)params_ptr)->p);
@@ -132,6 +162,7 @@ static uk_plugin_status_t plugin_resolve(void* self,
                                          uint32_t* out_resolution) {
   (void)self;
   static const struct { const char* name; void* fn; } table[] = {
+      {"iree_uk_conv_nchwc", (void*)conv_thunk},
       {"iree_uk_mmt4d", (void*)mmt4d_thunk},
       {"iree_uk_pack", (void*)pack_thunk},
       {"iree_uk_unpack", (void*)unpack_thunk},

@@ -142,6 +142,10 @@ class UKernelLibrary:
                                                _i64, _i64, _i64, _i64, _i64, _i64,
                                                _i64, _i32, _i32, _i32, _u32, _vp]
         L.iree_uk_amd_mmt4d_unpack.restype = None
+        L.iree_uk_conv_nchwc.argtypes = ([_vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64,
+                                          _vp, _i64, _i64, _i64, _i64] + [_i64] * 7 +
+                                         [_i32] * 4 + [_u32, _vp])
+        L.iree_uk_conv_nchwc.restype = None
         L.iree_uk_amd_last_status.restype = ctypes.c_int
         L.iree_uk_amd_last_status_string.restype = ctypes.c_char_p
         L.iree_uk_amd_last_kernel_name.restype = ctypes.c_char_p
@@ -197,6 +201,19 @@ class UKernelLibrary:
                                           rhs_stride0, out, out_offset, out_stride0,
                                           out_size0, out_size1, M, N, K, M0, N0, K0,
                                           flags, cpu_data)
+        self._check()
+
+    def conv_nchwc(self, inp, input_offset, input_stride_n, input_stride_ic_outer,
+                   input_stride_h, flt, filter_offset, filter_stride_oc_outer,
+                   filter_stride_ic_outer, filter_stride_fh, out, output_offset,
+                   output_stride_n, output_stride_oc_outer, output_stride_oh, N, OC_outer, OH,
+                   OW, IC_outer, FH, FW, k0, c0, stride_h, stride_w, flags, cpu_data=None):
+        self.lib.iree_uk_conv_nchwc(inp, input_offset, input_stride_n, input_stride_ic_outer,
+                                    input_stride_h, flt, filter_offset, filter_stride_oc_outer,
+                                    filter_stride_ic_outer, filter_stride_fh, out, output_offset,
+                                    output_stride_n, output_stride_oc_outer, output_stride_oh, N,
+                                    OC_outer, OH, OW, IC_outer, FH, FW, k0, c0, stride_h,
+                                    stride_w, flags, cpu_data)
         self._check()
 
     # --------------------------------------------------------------- control

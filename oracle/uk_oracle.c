@@ -17,7 +17,10 @@
  *   f16/bf16 <-> f32: runtime/src/iree/builtins/ukernel/common.h:665-792;
  *   f8E4M3FN -> f32 : runtime/src/iree/base/internal/math.h:324-362,557-560;
  *   f8 matmul       : tools/testing/e2e/iree-e2e-matmul-test.cc:123-142
- *                     (decode both operands, accumulate sequentially in f32).
+ *                     (decode both operands, accumulate sequentially in f32);
+ *   conv_nchwc      : runtime/src/iree/builtins/ukernel/conv_nchwc.c:42-130
+ *                     (early-outs, pointer arithmetic) and
+ *                     conv_nchwc_tile_generic.c:11-61 (the loop nest).
  *
  * Pinning status (what each function is checked against, in tests/):
  *   uk_oracle_pack / uk_oracle_unpack : golden tensors of
@@ -33,6 +36,11 @@
  *   uk_oracle_mmt4d with the f8 type : the reference has no f8 ukernel; the
  *       function is pinned by the decode table plus the f32 loop above, and
  *       by exactness on inputs whose products and sums are exact in f32.
+ *
+ *   uk_oracle_conv_nchwc : the independent per-pixel definition of
+ *       tools/conv_nchwc_test.c:13-87 restated in numpy (tests), a direct
+ *       convolution closed form on dense tensors, and randomized sweeps
+ *       against the compiled reference (oracle/_ref).
  *
  * Compile with -ffp-contract=off so that `acc += a*b` is a separate multiply
  * and add, which is what the reference generic build does on baseline x86-64.
@@ -474,5 +482,55 @@ UK_ORACLE_EXPORT int uk_oracle_unpack(
                  in + (in_offset + a0 * sl0 + a1 * sl1 + b0 * sl2 + b1 * sl3) * es,
                  es);
         }
+  return 0;
+}
+
+
+/* conv_nchwc, f32 only (the reference has no other type):
+ * input [N][IC_outer][IH][IW][c0], filter [OC_outer][IC_outer][FH][FW][c0][k0],
+ * output [N][OC_outer][OH][OW][k0], strides in elements for the outer
+ * dimensions as named; IW and FW steps are c0 and c0*k0. Accumulation order
+ * (ic_outer, fh, fw, ci) per output element as in
+ * conv_nchwc_tile_generic.c:34-57. Returns non-zero for an unknown type. */
+UK_ORACLE_EXPORT int uk_oracle_conv_nchwc(
+    const void* input_buffer, int64_t input_offset, int64_t input_stride_n,
+    int64_t input_stride_ic_outer, int64_t input_stride_h, const void* filter_buffer,
+    int64_t filter_offset, int64_t filter_stride_oc_outer, int64_t filter_stride_ic_outer,
+    int64_t filter_stride_fh, void* output_buffer, int64_t output_offset,
+    int64_t output_stride_n, int64_t output_stride_oc_outer, int64_t output_stride_oh,
+    int64_t N, int64_t OC_outer, int64_t OH, int64_t OW, int64_t IC_outer, int64_t FH,
+    int64_t FW, int32_t k0, int32_t c0, int32_t stride_h, int32_t stride_w, uint32_t flags,
+    const uint64_t* cpu_data) {
+  (void)cpu_data;
+  if ((flags & kTypeMask) != 0x01) return 1; /* exported_bits.h:113-116 */
+  const int accumulate = (flags & 0x100) != 0; /* exported_bits.h:119 */
+  /* conv_nchwc.c:42-53 */
+  if (N == 0 || OC_outer == 0 || OH == 0 || OW == 0) return 0;
+  if ((IC_outer == 0 || FH == 0 || FW == 0) && accumulate) return 0;
+  const float* in = (const float*)input_buffer + input_offset;
+  const float* f = (const float*)filter_buffer + filter_offset;
+  float* out = (float*)output_buffer + output_offset;
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t oc = 0; oc < OC_outer; ++oc)
+      for (int64_t oh = 0; oh < OH; ++oh)
+        for (int64_t ow = 0; ow < OW; ++ow)
+          for (int32_t ko = 0; ko < k0; ++ko) {
+            float* o = out + n * output_stride_n + oc * output_stride_oc_outer +
+                       oh * output_stride_oh + ow * k0 + ko;
+            float acc = accumulate ? *o : 0.f;
+            for (int64_t ic = 0; ic < IC_outer; ++ic)
+              for (int64_t fh = 0; fh < FH; ++fh)
+                for (int64_t fw = 0; fw < FW; ++fw)
+                  for (int32_t ci = 0; ci < c0; ++ci) {
+                    const float iv = in[n * input_stride_n + ic * input_stride_ic_outer +
+                                        (oh * stride_h + fh) * input_stride_h +
+                                        (ow * stride_w + fw) * c0 + ci];
+                    const float fv = f[oc * filter_stride_oc_outer + ic * filter_stride_ic_outer +
+                                       fh * filter_stride_fh + fw * (int64_t)c0 * k0 +
+                                       (int64_t)ci * k0 + ko];
+                    acc += iv * fv;
+                  }
+            *o = acc;
+          }
   return 0;
 }

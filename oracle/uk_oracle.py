@@ -42,6 +42,8 @@ _PACK_ARGS = [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
               _i64, _i64, _i64, _u64, _u32, _vp]
 _UNPACK_ARGS = [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
                 _i64, _i64, _i64, _u32, _vp]
+_CONV_ARGS = ([_vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
+               _i64] + [_i64] * 7 + [_i32] * 4 + [_u32, _vp])
 
 # Bit positions of cpu_data[0] on x86-64
 # (runtime/src/iree/schemas/cpu_feature_bits.inl:85-117), keyed by the
@@ -110,8 +112,10 @@ class Checker:
         self._mmt4d = getattr(self.lib, names[0])
         self._pack = getattr(self.lib, names[1])
         self._unpack = getattr(self.lib, names[2])
+        self._conv = getattr(self.lib, "uk_oracle_conv_nchwc" if kind == "oracle"
+                             else "iree_uk_conv_nchwc")
         for fn, args in ((self._mmt4d, _MMT4D_ARGS), (self._pack, _PACK_ARGS),
-                         (self._unpack, _UNPACK_ARGS)):
+                         (self._unpack, _UNPACK_ARGS), (self._conv, _CONV_ARGS)):
             fn.argtypes = args
             fn.restype = restype
         if kind == "oracle":
@@ -173,6 +177,23 @@ class Checker:
                          out_size0, out_size1, flags, _ptr(self.cpu_data))
         if self.kind == "oracle" and r != 0:
             raise ValueError(f"oracle unpack rejected flags {flags:#x}")
+
+    def conv_nchwc(self, inp, input_offset, input_stride_n, input_stride_ic_outer,
+                   input_stride_h, flt, filter_offset, filter_stride_oc_outer,
+                   filter_stride_ic_outer, filter_stride_fh, out, output_offset,
+                   output_stride_n, output_stride_oc_outer, output_stride_oh, N, OC_outer, OH,
+                   OW, IC_outer, FH, FW, k0, c0, stride_h, stride_w, flags, in_shift=0,
+                   filter_shift=0, out_shift=0):
+        """Positional arguments of iree_uk_conv_nchwc
+        (runtime/src/iree/builtins/ukernel/conv_nchwc.h:14-27)."""
+        r = self._conv(_ptr(inp, in_shift), input_offset, input_stride_n, input_stride_ic_outer,
+                       input_stride_h, _ptr(flt, filter_shift), filter_offset,
+                       filter_stride_oc_outer, filter_stride_ic_outer, filter_stride_fh,
+                       _ptr(out, out_shift), output_offset, output_stride_n,
+                       output_stride_oc_outer, output_stride_oh, N, OC_outer, OH, OW, IC_outer,
+                       FH, FW, k0, c0, stride_h, stride_w, flags, _ptr(self.cpu_data))
+        if self.kind == "oracle" and r != 0:
+            raise ValueError(f"oracle conv_nchwc rejected flags {flags:#x}")
 
     # -- threaded mmt4d: slabs of M (or N when M is small) through the
     # offset/stride parameters, the way IREE's task system slices work -------

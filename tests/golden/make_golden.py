@@ -108,6 +108,20 @@ def sweep_digests(chk) -> dict:
     return digests
 
 
+def conv_digests(chk) -> dict:
+    """case index -> digest of the whole output buffer for the seeded conv_nchwc
+    sweep (small-integer and N(0,1) inputs), computed with checker `chk`."""
+    import conv_testing as C
+    digests = {}
+    for ci, c in enumerate(C.cases(seed=31)):
+        for exact in (True, False):
+            rng = np.random.default_rng(7000 + ci)
+            inp, flt, out = C.buffers(c, rng, exact=exact)
+            C.run(chk, c, inp, flt, out)
+            digests[f"conv/{ci}/{int(exact)}"] = _digest(out)
+    return digests
+
+
 def known_answers(ref) -> dict:
     kat = {"pack": [], "unpack": [], "mmt4d_s8": []}
     x = np.array([[10 * i + j for j in range(5)] for i in range(3)], dtype=np.int8)
@@ -143,7 +157,9 @@ def main():
         json.dump(known_answers(ref), f, indent=1)
     with open(os.path.join(HERE, "reference_sweep.json"), "w") as f:
         json.dump(sweep_digests(ref), f, indent=0, sort_keys=True)
-    print("wrote reference_kat.json, reference_sweep.json")
+    with open(os.path.join(HERE, "reference_conv.json"), "w") as f:
+        json.dump(conv_digests(ref), f, indent=0, sort_keys=True)
+    print("wrote reference_kat.json, reference_sweep.json, reference_conv.json")
 
 
 if __name__ == "__main__":
