@@ -99,8 +99,9 @@ def test_query_versions_and_header(lib):
 
 def test_resolve_required_optional_and_preset(lib):
     plugin = _query(lib, 1).contents
-    st, res, ptrs = _resolve(plugin, ["iree_uk_mmt4d", "iree_uk_pack", "iree_uk_unpack"])
-    assert st == 0 and res == 0 and all(ptrs) and len(set(ptrs)) == 3
+    st, res, ptrs = _resolve(plugin, ["iree_uk_conv_nchwc", "iree_uk_mmt4d", "iree_uk_pack",
+                                      "iree_uk_unpack"])
+    assert st == 0 and res == 0 and all(ptrs) and len(set(ptrs)) == 4
     # optional and unknown: OK with the MISSING_OPTIONAL bit, entry left NULL
     st, res, ptrs = _resolve(plugin, ["?iree_uk_conv", "?iree_uk_mmt4d"])
     assert st == 0 and res == 1 and ptrs[0] is None and ptrs[1]
