@@ -115,6 +115,107 @@ def cpu_baseline_c2(keep: dict, target_seconds: float = 12.0) -> dict:
     }, out4, slab
 
 
+def _host_bytes(t):
+    """A device tensor as a flat numpy byte view on the host."""
+    import torch
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def _mmt4d_type_flag(dtype: str, uk):
+    return {"s8": uk.MMT4D_TYPE_S8S8S32, "f16": uk.MMT4D_TYPE_F16F16F32,
+            "bf16": uk.MMT4D_TYPE_BF16BF16F32, "f32": uk.MMT4D_TYPE_F32F32F32,
+            "f8": uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32}[dtype]
+
+
+def cpu_baseline_extra(wl, target_seconds: float = 3.0):
+    """The CPU path beside an `extra` workload, on a bounded sample: the
+    compiled reference with the host's ISA paths enabled where it has the type
+    (kind "reference"; s8 16x16x2 and bf16 16x16x2 then run its AVX-512
+    VNNI / BF16 tiles), the C restatement for f8 (kind "port"). mmt4d runs on
+    a slab of tile rows (or columns when M is one tile) over all threads, sized
+    from a calibration run and extrapolated; pack / unpack run single-threaded
+    on a slab of rows. None for workloads it does not cover."""
+    import numpy as np
+    from oracle import uk_oracle
+    from iree_amd import ukernel as uk
+
+    keep = wl.keep
+    T = cpu_threads()
+    have_ref = uk_oracle.Checker.reference_available()
+    if wl.name.startswith("c5_pack"):
+        chk = uk_oracle.Checker("reference" if have_ref else "oracle")
+        chk.use_host_cpu_features(True)
+        rows, cols = keep["rows"], keep["cols"]
+        slab_rows = min(rows, 16 * 96)               # 96 tile rows of 16
+        x = keep["x"][:slab_rows].cpu().numpy().reshape(-1)
+        o0 = slab_rows // 16
+        packed = np.zeros(o0 * cols * 16, np.float32)
+        flags = uk.PACK_TYPE_F32F32 | uk.PACK_TRANSPOSE_OUTER
+        t0 = time.perf_counter()
+        # TRANSPOSE_OUTER: stored [cols][o0][16][1]
+        chk.pack(x, 0, cols, 1, packed, 0, o0 * 16, 16, slab_rows, cols, cols, o0, 16, 1,
+                 0xBF800000, flags)
+        t_pack = time.perf_counter() - t0
+        back = np.zeros(slab_rows * cols, np.float32)
+        t0 = time.perf_counter()
+        chk.unpack(packed, 0, o0 * 16, 16, back, 0, cols, 1, cols, o0, 16, 1, slab_rows, cols,
+                   uk.UNPACK_TYPE_F32F32 | uk.UNPACK_TRANSPOSE_OUTER)
+        t_un = time.perf_counter() - t0
+        ok = bool(np.array_equal(back, x))
+        nbytes = 2.0 * slab_rows * cols * 4
+        return {"value": round(2 * nbytes / (t_pack + t_un) / 1e9, 3), "unit": "GB/s", "cores": 1,
+                "kind": "reference" if have_ref else "port",
+                "sample": f"pack + unpack of the first {slab_rows} of {rows} rows, 1 thread "
+                          f"({t_pack:.2f} s + {t_un:.2f} s); round trip exact: {ok}"}
+    if "lhs4" not in keep or "M1" not in keep and "M" not in keep:
+        return None
+    dtype = wl.dtype
+    if dtype not in ("s8", "f16", "bf16", "f32", "f8"):
+        return None
+    kind = "reference" if (have_ref and dtype != "f8") else "port"
+    chk = uk_oracle.Checker("reference" if kind == "reference" else "oracle")
+    chk.use_host_cpu_features(True)
+    M0, N0, K0 = keep["M0"], keep["N0"], keep["K0"]
+    if "M1" in keep:
+        M1, N1, K1 = keep["M1"], keep["N1"], keep["K1"]
+    else:
+        M1, N1, K1 = -(-keep["M"] // M0), -(-keep["N"] // N0), keep["K"] // K0
+    flags = _mmt4d_type_flag(dtype, uk) | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
+    lhs = _host_bytes(keep["lhs4"])
+    rhs = _host_bytes(keep["rhs4"])
+    out = np.zeros(M1 * N1 * M0 * N0, np.int32 if dtype == "s8" else np.float32)
+    ls, rs, os_ = K1 * M0 * K0, K1 * N0 * K0, N1 * M0 * N0
+
+    def run(m_tiles, n_tiles):
+        t0 = time.perf_counter()
+        chk.mmt4d_threaded(T, lhs, ls, rhs, rs, out, os_, m_tiles, n_tiles, K1, M0, N0, K0, flags)
+        return time.perf_counter() - t0
+
+    # Calibrate on a small rectangle of tiles, then size the sample: whole tile
+    # rows when a few of them fit the time budget, else part of T tile rows.
+    if M1 >= T:
+        n_cal = min(N1, 2 * T)
+        t_cal = run(T, n_cal)
+        tiles = (T * n_cal / max(t_cal, 1e-4)) * target_seconds
+        if tiles >= T * N1:
+            rows = int(min(M1, (tiles / N1) // T * T))
+            cols = N1
+        else:
+            rows, cols = T, int(max(n_cal, min(N1, tiles // T)))
+        t = run(rows, cols)
+        frac, what = rows * cols / (M1 * N1), f"{rows}/{M1} M tile-rows x {cols}/{N1} N tile-columns"
+    else:         # one (or few) tile rows: slab of N tile columns
+        n_cal = min(N1, 4 * T)
+        t_cal = run(M1, n_cal)
+        cols = int(max(n_cal, min(N1, n_cal * round(target_seconds / max(t_cal, 1e-4)))))
+        t = run(M1, cols)
+        frac, what = cols / N1, f"{M1}/{M1} M tile-rows x {cols}/{N1} N tile-columns"
+    return {"value": round(wl.ops[[o.name for o in wl.ops].index("mmt4d")].flops * frac / t / 1e12, 6),
+            "unit": "TFLOP/s", "cores": T, "kind": kind,
+            "sample": f"mmt4d only, on {what} over {T} threads ({t:.2f} s), host ISA paths enabled; "
+                      "extrapolated linearly to the whole problem"}
+
+
 def verify_c2(runner, keep, cpu_out4, slab) -> dict:
     """GPU result of the timed chain against the CPU checker on the slab the
     baseline computed: max|gpu-ref|/max|ref| must be <= 1e-2 (f16 inputs, f32
@@ -213,6 +314,11 @@ def main() -> int:
             if w.flops:
                 # sum of the kernels' device times (no launch gaps)
                 entry["chain_TFLOPs"] = round(w.flops / (total_us * 1e-6) / 1e12, 3)
+            if not args.no_cpu:
+                try:
+                    entry["cpu_baseline"] = cpu_baseline_extra(w)
+                except Exception as e:  # the baseline is a reported aside, never fatal
+                    entry["cpu_baseline"] = {"error": repr(e)}
             extra[name] = entry
             del w
         result["extra"] = extra
