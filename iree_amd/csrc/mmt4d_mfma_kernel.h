@@ -285,6 +285,11 @@ void mmt4d_mfma_kernel(Args a) {
   uint32_t skt[NU];      // bytes between consecutive loads of a unit
   int32_t kt0[NU];       // K-tile index of the first load at step 0
   uint32_t loff[NU];     // LDS offset (within a stage) of the unit's first store
+  // Regrouping loaders only: false for a unit whose rows lie beyond the
+  // operand's LDS image. That happens when the tile height does not divide
+  // the block (e.g. M0 = 24 in a 64-row block: the units of a third, partial
+  // panel would land on rows 48..71); such a unit loads but must not store.
+  bool lds_ok[NU];
 #pragma unroll
   for (int i = 0; i < NU; ++i) {
     const int blk = wave + i * NW;
@@ -313,6 +318,7 @@ void mmt4d_mfma_kernel(Args a) {
       voff[i] = (uint32_t)pl * (uint32_t)xstride + ktl * kt_bytes + (m0 << lrb) +
                 (kb & ((1u << lrb) - 1));
       skt[i] = 0;
+      lds_ok[i] = true;
       loff[i] = image + (uint32_t)xblk * 1024 + lane * 16;
     } else {
       // Units in order [panel][chunk g][row group]; the unit's R loads read
@@ -328,6 +334,7 @@ void mmt4d_mfma_kernel(Args a) {
       voff[i] = (uint32_t)pl * (uint32_t)xstride + g * kt_bytes + mg * 16;
       skt[i] = NCH * kt_bytes;
       const uint32_t row = (uint32_t)pl * X0 + mg * R;  // first of R rows
+      lds_ok[i] = row + R <= (uint32_t)(is_b ? BN : BM);
       const uint32_t rr = row & 15;  // R divides 16: the R rows share a block
       // Slot of row rr + j is (rr + j) ^ mask; R <= 8 and rr % R == 0, so j
       // only touches the low bits and the store applies j ^ ... itself.
@@ -469,6 +476,7 @@ void mmt4d_mfma_kernel(Args a) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       if (!EVEN && wave + i * NW >= BLOCKS) continue;
+      if (RBC < 16 && !lds_ok[i]) continue;
       if constexpr (RBC >= 16) {
         *reinterpret_cast<v4i*>(base + loff[i]) = src[i][0];
       } else {
@@ -577,6 +585,7 @@ void mmt4d_mfma_kernel(Args a) {
         for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k) {
           const int i = k / R, j = k % R;
           if (!EVEN && wave + i * NW >= BLOCKS) continue;
+          if (RBC < 16 && !lds_ok[i]) continue;
           char* dst = lds + st_write + (RBC >= 16 ? loff[i] : (loff[i] ^ (uint32_t)(j * 16)));
           *reinterpret_cast<v4i*>(dst) = RBC >= 16 ? regs[P ^ 1][i][0] : outp[i][j];
         }

@@ -60,6 +60,11 @@ MFMA_TILES = [
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 128),
     (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 4),
     (uk.MMT4D_TYPE_F32F32F32, 8, 8, 2), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 32),
+    # tile heights that do not divide the workgroup tiles (a partial panel at
+    # the end of each block), with regrouping and with direct loaders
+    (uk.MMT4D_TYPE_S8S8S32, 24, 16, 4), (uk.MMT4D_TYPE_S8S8S32, 16, 24, 2),
+    (uk.MMT4D_TYPE_F16F16F32, 24, 48, 2), (uk.MMT4D_TYPE_S8S8S32, 40, 24, 16),
+    (uk.MMT4D_TYPE_BF16BF16F32, 12, 20, 4), (uk.MMT4D_TYPE_F32F32F32, 24, 40, 1),
 ]
 
 

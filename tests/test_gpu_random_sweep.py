@@ -1,0 +1,126 @@
+"""Seeded random sweeps of pack / unpack / mmt4d on the GPU against the oracle,
+through the C-ABI: shapes, tile sizes, strides, offsets and flags drawn at
+random (mid-size, so that the streaming, tiled and generic kernels and several
+MFMA variants are all reached), whole destination buffers compared bit for
+bit. Complements the reference's own test grids with shapes they do not hold."""
+import numpy as np
+import pytest
+
+import uk_testing as T
+from golden import make_golden as G
+from iree_amd import ukernel as uk
+
+pytestmark = pytest.mark.gpu
+
+PACK_TYPES = [uk.PACK_TYPE_F32F32, uk.PACK_TYPE_I8I8, uk.PACK_TYPE_I32I32, uk.PACK_TYPE_F16F16,
+              uk.PACK_TYPE_BF16BF16]
+UNPACK_TYPES = [uk.UNPACK_TYPE_F32F32, uk.UNPACK_TYPE_I32I32, uk.UNPACK_TYPE_F16F16,
+                uk.UNPACK_TYPE_BF16BF16]
+TILE_SIDES = [1, 2, 3, 4, 6, 8, 16, 32, 64]
+
+
+def _pack_case(rng, tf):
+    es = uk.PACK_TYPE_BYTES[tf]
+    while True:
+        t0, t1 = (int(rng.choice(TILE_SIDES)) for _ in range(2))
+        if t0 * t1 * es <= 4096:
+            break
+    o0, o1 = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+    ti, to = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+    flags = tf | (uk.PACK_TRANSPOSE_INNER if ti else 0) | (uk.PACK_TRANSPOSE_OUTER if to else 0)
+    lt0, lt1 = (t1, t0) if ti else (t0, t1)            # logical tile along matrix dims 0, 1
+    lo0, lo1 = (o1, o0) if to else (o0, o1)            # logical outer counts
+    in0 = max(0, lo0 * lt0 - int(rng.integers(0, lt0 + 3)))
+    in1 = max(0, lo1 * lt1 - int(rng.integers(0, lt1 + 3)))
+    in_stride1 = 1 if rng.integers(0, 4) else 2
+    in_stride0 = in1 * in_stride1 + int(rng.choice([0, 0, 1, 4, 16]))
+    out_stride0 = o1 * t0 * t1 + int(rng.choice([0, 0, 1, 4, 16]))
+    return T.PackCase(flags, in0, in1, o0, o1, t0, t1, in_stride0, in_stride1, out_stride0,
+                      int(rng.choice([0, 1, 4, 16])), int(rng.choice([0, 1, 4, 16])),
+                      int(rng.integers(0, 2 ** 63)))
+
+
+def _unpack_case(rng, tf):
+    es = uk.PACK_TYPE_BYTES[tf]
+    while True:
+        t0, t1 = (int(rng.choice(TILE_SIDES)) for _ in range(2))
+        if t0 * t1 * es <= 4096:
+            break
+    i0, i1 = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+    ti, to = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+    flags = tf | (uk.UNPACK_TRANSPOSE_INNER if ti else 0) | (uk.UNPACK_TRANSPOSE_OUTER if to else 0)
+    lt0, lt1 = (t1, t0) if ti else (t0, t1)
+    lo0, lo1 = (i1, i0) if to else (i0, i1)
+    out0 = max(1, lo0 * lt0 - int(rng.integers(0, lt0)))
+    out1 = max(1, lo1 * lt1 - int(rng.integers(0, lt1)))
+    out_stride1 = 1 if rng.integers(0, 4) else 2
+    out_stride0 = out1 * out_stride1 + int(rng.choice([0, 0, 1, 4, 16]))
+    in_stride0 = i1 * t0 * t1 + int(rng.choice([0, 0, 1, 4, 16]))
+    return T.UnpackCase(flags, i0, i1, t0, t1, out0, out1, in_stride0, out_stride0, out_stride1,
+                        int(rng.choice([0, 1, 4, 16])), int(rng.choice([0, 1, 4, 16])))
+
+
+def test_pack_random_sweep(gpu, oracle):
+    lib, torch = gpu
+    rng = np.random.default_rng(2024)
+    kernels = set()
+    for ci in range(160):
+        c = _pack_case(rng, PACK_TYPES[ci % len(PACK_TYPES)])
+        inp, out = T.make_pack_buffers(c, np.random.default_rng(ci))
+        want = out.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        got = T.gpu_pack(lib, torch, c, inp, out)
+        assert np.array_equal(got, want), (ci, c, lib.last_kernel_name())
+        kernels.add(lib.last_kernel_name())
+    assert {"pack_stream", "pack_generic"} <= kernels, kernels
+
+
+def test_unpack_random_sweep(gpu, oracle):
+    lib, torch = gpu
+    rng = np.random.default_rng(2025)
+    kernels = set()
+    for ci in range(160):
+        c = _unpack_case(rng, UNPACK_TYPES[ci % len(UNPACK_TYPES)])
+        inp, out = T.make_unpack_buffers(c, np.random.default_rng(ci))
+        want = out.copy()
+        G.run_unpack_case(oracle, c, inp, want)
+        got = T.gpu_unpack(lib, torch, c, inp, out)
+        assert np.array_equal(got, want), (ci, c, lib.last_kernel_name())
+        kernels.add(lib.last_kernel_name())
+    assert {"unpack_stream", "unpack_generic"} <= kernels, kernels
+
+
+MMT4D_TYPES = [uk.MMT4D_TYPE_S8S8S32, uk.MMT4D_TYPE_F16F16F32, uk.MMT4D_TYPE_BF16BF16F32,
+               uk.MMT4D_TYPE_F32F32F32, uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, uk.MMT4D_TYPE_S16S16S32,
+               uk.MMT4D_TYPE_S8S4S32, uk.MMT4D_TYPE_F16F16F16, uk.MMT4D_TYPE_BF16BF16BF16]
+
+
+def test_mmt4d_random_sweep(gpu, oracle):
+    """Inputs are small integers (exact in every type), so any summation order
+    must give the oracle's bits; tile shapes include ones no MFMA kernel takes."""
+    lib, torch = gpu
+    rng = np.random.default_rng(2026)
+    kernels = set()
+    for ci in range(180):
+        tf = MMT4D_TYPES[ci % len(MMT4D_TYPES)]
+        lb = uk.MMT4D_TYPE_BITS[tf][0]
+        rbits = uk.MMT4D_TYPE_BITS[tf][1]
+        M0, N0 = int(rng.choice([1, 2, 4, 8, 16, 24, 32, 64])), int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        K0 = int(rng.choice([1, 2, 4, 8, 16, 32]))
+        if rbits == 4:
+            K0 = max(2, K0)
+        if tf == uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32:
+            K0 = max(16, K0)
+        M, N, K = int(rng.integers(0, 12)), int(rng.integers(0, 12)), int(rng.integers(0, 40))
+        extra = uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS if rng.integers(0, 2) and lb == 16 else 0
+        acc = uk.MMT4D_ACCUMULATE if rng.integers(0, 2) else 0
+        slack = int(rng.choice([0, 16]))
+        c = T.Mmt4dCase(tf | extra | acc, M, N, K, M0, N0, K0, K * M0 * K0 + slack,
+                        K * N0 * K0 + slack, N * M0 * N0 + slack, slack, 0, slack)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert np.array_equal(got, want), (ci, c, lib.last_kernel_name())
+        kernels.add(lib.last_kernel_name())
+    assert "mmt4d_generic" in kernels and any(k.startswith("mmt4d_mfma") for k in kernels), kernels
