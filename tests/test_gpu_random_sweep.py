@@ -124,3 +124,71 @@ def test_mmt4d_random_sweep(gpu, oracle):
         assert np.array_equal(got, want), (ci, c, lib.last_kernel_name())
         kernels.add(lib.last_kernel_name())
     assert "mmt4d_generic" in kernels and any(k.startswith("mmt4d_mfma") for k in kernels), kernels
+
+
+def test_mmt4d_random_sweep_larger_shapes_and_forced_variants(gpu, oracle):
+    """Tile counts large enough for the 128x128 / 256x256 workgroup shapes
+    (several workgroups, ragged against them), a random forced variant per
+    case, MFMA-served tile shapes only (incl. heights that do not divide the
+    workgroup tile), K with and without a remainder against the pipeline step."""
+    lib, torch = gpu
+    rng = np.random.default_rng(2027)
+    types = [uk.MMT4D_TYPE_S8S8S32, uk.MMT4D_TYPE_F16F16F32, uk.MMT4D_TYPE_BF16BF16F32,
+             uk.MMT4D_TYPE_F32F32F32, uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32]
+    done = 0
+    for ci in range(400):
+        tf = types[ci % len(types)]
+        eb = uk.MMT4D_TYPE_BITS[tf][0] // 8
+        M0, N0 = int(rng.choice([4, 8, 12, 16, 24, 32, 48, 64])), int(rng.choice([4, 8, 16, 20, 32, 64]))
+        K0 = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        if not lib.mmt4d_info(M0, N0, K0, tf):
+            continue
+        M, N = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        K = int(rng.integers(1, max(2, 600 // (K0 * eb))))
+        acc = uk.MMT4D_ACCUMULATE if rng.integers(0, 2) else 0
+        c = T.Mmt4dCase(tf | acc, M, N, K, M0, N0, K0, K * M0 * K0 + 16, K * N0 * K0,
+                        N * M0 * N0 + 16, 16, 0, 0)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        variant = int(rng.integers(0, 5))
+        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (ci, c, variant, lib.last_kernel_name())
+        assert lib.last_kernel_name().startswith("mmt4d_mfma"), (ci, c, lib.last_kernel_name())
+        done += 1
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    assert done >= 120, done
+
+
+def test_pack_unpack_random_round_trips_multi_block(gpu):
+    """Sizes of several blocks per dimension: pack must equal numpy's
+    pad + reshape + transpose and unpack must invert it, for random tiles,
+    transposes and ragged sizes."""
+    lib, torch = gpu
+    rng = np.random.default_rng(2028)
+    for ci in range(40):
+        dtype, tf = [(np.float32, uk.PACK_TYPE_F32F32), (np.int8, uk.PACK_TYPE_I8I8),
+                     (np.float16, uk.PACK_TYPE_F16F16), (np.int32, uk.PACK_TYPE_I32I32)][ci % 4]
+        t0, t1 = int(rng.choice([1, 4, 8, 16, 32])), int(rng.choice([1, 2, 8, 16, 32]))
+        ti, to = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        shape = (int(rng.integers(1, 700)), int(rng.integers(1, 700)))
+        x = rng.integers(-100, 100, shape).astype(dtype)
+        pad_val = dtype(-3)
+        pad_bits = int(np.array([pad_val]).view({1: np.uint8, 2: np.uint16, 4: np.uint32}[x.itemsize])[0])
+        want4 = T.numpy_pack(x, t0, t1, ti, to, pad_val)
+        o0, o1, o2, o3 = want4.shape
+        d_x = torch.from_numpy(x).cuda()
+        d_p = torch.zeros(want4.size * x.itemsize, dtype=torch.uint8, device="cuda")
+        flags = tf | (0x100 if ti else 0) | (0x200 if to else 0)
+        lib.pack(d_x.data_ptr(), 0, shape[1], 1, d_p.data_ptr(), 0, o1 * o2 * o3, o2 * o3, shape[0],
+                 shape[1], o0, o1, o2, o3, pad_bits, flags)
+        got4 = d_p.cpu().numpy().view(dtype).reshape(want4.shape)
+        assert np.array_equal(got4, want4), (ci, shape, t0, t1, ti, to, lib.last_kernel_name())
+        if tf == uk.PACK_TYPE_I8I8:
+            continue  # unpack has no 1-byte type
+        d_y = torch.full((x.size * x.itemsize,), 0x5A, dtype=torch.uint8, device="cuda")
+        lib.unpack(d_p.data_ptr(), 0, o1 * o2 * o3, o2 * o3, d_y.data_ptr(), 0, shape[1], 1, o0, o1,
+                   o2, o3, shape[0], shape[1], flags)
+        back = d_y.cpu().numpy().view(dtype).reshape(shape)
+        assert np.array_equal(back, x), (ci, shape, t0, t1, ti, to, lib.last_kernel_name())
