@@ -26,8 +26,17 @@
 // them: [row block of 16][group of 4 K-slices][slice q][row r][16 bytes], so an
 // operand fetch is one ds_read_b128 per lane over a contiguous KiB.
 //
-// Pipeline: double-buffered LDS; global loads run PF steps ahead of the MFMAs
-// through PF register sets; one barrier per K step.
+// Pipelines (template parameter PIPE), one barrier per K step in all of them:
+//   0  two LDS stages, both operands through LDS, global loads one step
+//      ahead, zero-filled K tail (any K);
+//   1  three LDS stages, both operands through LDS, loads three steps ahead
+//      through two register sets, fragments one step ahead;
+//   2  LHS as in 1, RHS fragments loaded by each wave straight from global
+//      memory into registers one step ahead (row bytes >= 16 only);
+//   3  as 2 with every prefetch one step deeper (three register sets, three
+//      RHS fragment buffers), unrolled by three.
+// Pipelines 1-3 need K in whole steps; the launcher gives a K remainder to a
+// second, accumulating launch of a PIPE 0 variant.
 #ifndef IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
 #define IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
 
@@ -231,8 +240,7 @@ __device__ __forceinline__ void block_of_workgroup(uint32_t wg, const Args& a,
 }
 
 // TM x TN accumulator blocks per wave, WGM x WGN waves per workgroup, NKK MFMA
-// K-groups per pipeline step. PIPE 0: two LDS stages, loads one step ahead.
-// PIPE 1: three LDS stages, loads three steps ahead, fragments one step ahead.
+// K-groups per pipeline step, PIPE as described at the top of this file.
 // RBC: 16 = row bytes >= 16 (direct), 8/4/2 = regrouping loaders.
 template <Elem E, int RBC, int TM, int TN, int WGM, int WGN, int NKK, int PIPE>
 __global__ __launch_bounds__(WGM* WGN * 64)
