@@ -473,6 +473,69 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_mmt4d_unpack_p(
     const iree_uk_amd_mmt4d_unpack_params_t* params);
 
 /*===----------------------------------------------------------------------===*/
+/* Fused mmt4d + dequantizing unpack                                           */
+/*===----------------------------------------------------------------------===*/
+
+/* No counterpart in the reference (a quantized linear layer there is mmt4d,
+ * unpack and a compiler-generated elementwise dispatch): mmt4d of a type with
+ * a 32-bit accumulator (s32 or f32 out type), whose result goes into a
+ * row-major f32 out_size0 x out_size1 matrix as
+ *
+ *   out[i][j] = (float)(acc0[i][j] + sum_k lhs[i][k] * rhs[j][k])
+ *               * row_scale[i] * col_scale[j]
+ *
+ * evaluated in f32 from left to right (convert, multiply by the row scale,
+ * multiply by the column scale). `row_scale` has out_size0 and `col_scale`
+ * out_size1 f32 entries; either may be NULL and then reads as 1. acc0 is 0, or
+ * with IREE_UK_FLAG_MMT4D_ACCUMULATE the tiled [M][N][M0][N0] buffer
+ * `acc_buffer` of the mmt4d out type (`acc_offset` and `acc_stride0` in
+ * elements, as out_offset / out_stride0 of iree_uk_mmt4d), which is only read.
+ * For the integer types the result equals, bit for bit, iree_uk_mmt4d into the
+ * accumulator buffer, iree_uk_unpack and the scaling above. Unlike
+ * iree_uk_mmt4d, K == 0 with ACCUMULATE still writes the (scaled) matrix.
+ * Operand arguments, tile sizes and flags are otherwise those of
+ * iree_uk_mmt4d; out_size0 <= M*M0 and out_size1 <= N*N0. */
+typedef struct iree_uk_amd_mmt4d_dequant_unpack_params_t {
+  const void* lhs_buffer;
+  iree_uk_index_t lhs_offset;
+  iree_uk_index_t lhs_stride0;
+  const void* rhs_buffer;
+  iree_uk_index_t rhs_offset;
+  iree_uk_index_t rhs_stride0;
+  const void* acc_buffer;
+  iree_uk_index_t acc_offset;
+  iree_uk_index_t acc_stride0;
+  void* out_buffer;
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t out_size0;
+  iree_uk_index_t out_size1;
+  const float* row_scale;
+  const float* col_scale;
+  iree_uk_index_t M;
+  iree_uk_index_t N;
+  iree_uk_index_t K;
+  int32_t M0;
+  int32_t N0;
+  int32_t K0;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_amd_mmt4d_dequant_unpack_params_t;
+
+IREE_UK_AMD_EXPORT void iree_uk_amd_mmt4d_dequant_unpack(
+    const void* lhs_buffer, iree_uk_index_t lhs_offset,
+    iree_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0,
+    const void* acc_buffer, iree_uk_index_t acc_offset,
+    iree_uk_index_t acc_stride0, void* out_buffer, iree_uk_index_t out_offset,
+    iree_uk_index_t out_stride0, iree_uk_index_t out_size0,
+    iree_uk_index_t out_size1, const float* row_scale, const float* col_scale,
+    iree_uk_index_t M, iree_uk_index_t N, iree_uk_index_t K, int32_t M0,
+    int32_t N0, int32_t K0, uint32_t flags, const uint64_t* cpu_data);
+IREE_UK_AMD_EXPORT void iree_uk_amd_mmt4d_dequant_unpack_p(
+    const iree_uk_amd_mmt4d_dequant_unpack_params_t* params);
+
+/*===----------------------------------------------------------------------===*/
 /* HAL executable plugin face                                                  */
 /*===----------------------------------------------------------------------===*/
 

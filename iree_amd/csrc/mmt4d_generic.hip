@@ -45,6 +45,15 @@ struct Mmt4dArgs {
   // mmt4d + unpack, of which only out_rows x out_cols elements exist.
   int64_t out_s_i, out_s_i0, out_s_j;
   int64_t out_rows, out_cols;
+  // Dequantizing store (32-bit accumulator kinds only): the output is f32,
+  // (float)acc * row_scale[row] * col_scale[col] with a null scale reading as
+  // 1, and ACCUMULATE reads the tiled buffer `acc` (acc_s_i elements between
+  // rows of tiles) instead of the output.
+  uint32_t dequant;
+  const char* acc;
+  int64_t acc_s_i;
+  const float* row_scale;
+  const float* col_scale;
   int64_t M, N, K;
   int32_t M0, N0, K0;
   uint32_t accumulate, skip_round;
@@ -70,10 +79,18 @@ __global__ __launch_bounds__(kThreads) void mmt4d_generic_kernel(Mmt4dArgs a) {
     if (i * a.M0 + i0 >= a.out_rows || j * a.N0 + j0 >= a.out_cols) continue;
     const int64_t o = i * a.out_s_i + i0 * a.out_s_i0 + j * a.out_s_j + j0;
     const int32_t M0 = a.M0, N0 = a.N0, K0 = a.K0;
+    // Where the initial accumulator is read, and what the finished one becomes.
+    const char* acc_base = a.dequant ? a.acc : a.out;
+    const int64_t ai = a.dequant ? i * a.acc_s_i + j * tile + t : o;
+    auto scaled = [&](float v) {
+      const float rs = a.row_scale ? a.row_scale[i * M0 + i0] : 1.0f;
+      const float cs = a.col_scale ? a.col_scale[j * N0 + j0] : 1.0f;
+      return v * rs * cs;
+    };
 
     if constexpr (KIND == Kind::kS8S8 || KIND == Kind::kS16S16 || KIND == Kind::kS16S8) {
       int32_t* out = reinterpret_cast<int32_t*>(a.out);
-      uint32_t acc = a.accumulate ? (uint32_t)out[o] : 0u;
+      uint32_t acc = a.accumulate ? (uint32_t) reinterpret_cast<const int32_t*>(acc_base)[ai] : 0u;
       for (int64_t k = 0; k < a.K; ++k) {
         for (int32_t k0 = 0; k0 < K0; ++k0) {
           const int64_t li = (k * M0 + i0) * K0 + k0;
@@ -86,11 +103,12 @@ __global__ __launch_bounds__(kThreads) void mmt4d_generic_kernel(Mmt4dArgs a) {
           acc += (uint32_t)(l * r);
         }
       }
-      out[o] = (int32_t)acc;
+      if (a.dequant) reinterpret_cast<float*>(a.out)[o] = scaled((float)(int32_t)acc);
+      else out[o] = (int32_t)acc;
     } else if constexpr (KIND == Kind::kS8S4 || KIND == Kind::kS16U4) {
       // Two 4-bit rhs values per byte, low nibble first.
       int32_t* out = reinterpret_cast<int32_t*>(a.out);
-      uint32_t acc = a.accumulate ? (uint32_t)out[o] : 0u;
+      uint32_t acc = a.accumulate ? (uint32_t) reinterpret_cast<const int32_t*>(acc_base)[ai] : 0u;
       const int32_t K0h = K0 / 2;
       const uint8_t* r8 = reinterpret_cast<const uint8_t*>(rp);
       for (int64_t k = 0; k < a.K; ++k) {
@@ -113,11 +131,12 @@ __global__ __launch_bounds__(kThreads) void mmt4d_generic_kernel(Mmt4dArgs a) {
           acc += (uint32_t)(l0 * r0 + l1 * r1);
         }
       }
-      out[o] = (int32_t)acc;
+      if (a.dequant) reinterpret_cast<float*>(a.out)[o] = scaled((float)(int32_t)acc);
+      else out[o] = (int32_t)acc;
     } else if constexpr (KIND == Kind::kF32 || KIND == Kind::kF16F32 ||
                          KIND == Kind::kBF16F32 || KIND == Kind::kF8F32) {
       float* out = reinterpret_cast<float*>(a.out);
-      float acc = a.accumulate ? out[o] : 0.f;
+      float acc = a.accumulate ? reinterpret_cast<const float*>(acc_base)[ai] : 0.f;
       for (int64_t k = 0; k < a.K; ++k) {
         for (int32_t k0 = 0; k0 < K0; ++k0) {
           const int64_t li = (k * M0 + i0) * K0 + k0;
@@ -139,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_generic_kernel(Mmt4dArgs a) {
           acc += l * r;
         }
       }
-      out[o] = acc;
+      out[o] = a.dequant ? scaled(acc) : acc;
     } else {
       // f16 / bf16 results, with or without rounding the running sum to the
       // 16-bit type after every multiply-add.
@@ -208,6 +227,18 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_generic(
     a.out_s_j = (int64_t)p->M0 * p->N0;
     a.out_rows = p->M * p->M0;
     a.out_cols = p->N * p->N0;
+  }
+  a.dequant = 0;
+  a.acc = nullptr;
+  a.acc_s_i = 0;
+  a.row_scale = a.col_scale = nullptr;
+  if (rowmajor && rowmajor->dequant) {
+    if (out_bytes != 4) return (int)hipErrorInvalidValue;
+    a.dequant = 1;
+    a.acc = (const char*)rowmajor->acc;
+    a.acc_s_i = rowmajor->acc_stride0;
+    a.row_scale = rowmajor->row_scale;
+    a.col_scale = rowmajor->col_scale;
   }
   a.M = p->M; a.N = p->N; a.K = p->K;
   a.M0 = p->M0; a.N0 = p->N0; a.K0 = p->K0;

@@ -98,6 +98,25 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     pr.out_rows = p->M * p->M0;
     pr.out_cols = p->N * p->N0;
   }
+  pr.acc = pr.out;
+  pr.acc_stride = pr.out_stride;
+  pr.acc_sm0 = pr.out_sm0;
+  pr.acc_spn = pr.out_spn;
+  pr.dequant = false;
+  pr.row_scale = pr.col_scale = nullptr;
+  if (rowmajor && rowmajor->dequant) {
+    if (ob != 4) return -1;
+    pr.dequant = true;
+    pr.row_scale = rowmajor->row_scale;
+    pr.col_scale = rowmajor->col_scale;
+    if (p->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) {
+      pr.acc = (const char*)rowmajor->acc;
+      pr.acc_stride = rowmajor->acc_stride0 * ob;
+      pr.acc_sm0 = (int64_t)p->N0 * ob;
+      pr.acc_spn = (int64_t)p->M0 * p->N0 * ob;
+      if ((uintptr_t)pr.acc & 3) return -1;
+    }
+  }
   // 16-byte vector loads need 16-byte aligned panels.
   if (((uintptr_t)pr.lhs | (uintptr_t)pr.rhs | (uint64_t)pr.lhs_stride |
        (uint64_t)pr.rhs_stride) & 15) {

@@ -34,7 +34,10 @@
 //   2  LHS as in 1, RHS fragments loaded by each wave straight from global
 //      memory into registers one step ahead (row bytes >= 16 only);
 //   3  as 2 with every prefetch one step deeper (three register sets, three
-//      RHS fragment buffers), unrolled by three.
+//      RHS fragment buffers), unrolled by three;
+//   4  as 0 with the global loads three steps ahead through three register
+//      sets (any K): for M-thin problems, which are bound by memory latency
+//      and want as many bytes in flight per workgroup as registers allow.
 // Pipelines 1-3 need K in whole steps; the launcher gives a K remainder to a
 // second, accumulating launch of a PIPE 0 variant.
 #ifndef IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
@@ -184,6 +187,20 @@ struct Args {
   uint32_t tail;       // 1 when the last K step is partial
   uint32_t band;       // workgroup rows per rasterization band
   uint32_t vec_out;    // 1: 4 consecutive columns of a row are contiguous (and aligned enough)
+  // Where ACCUMULATE reads the initial accumulators: the same four-stride
+  // addressing as the output. It is the output itself except in the first
+  // launch of a dequantizing call, which reads a tiled accumulator buffer and
+  // writes a row-major matrix.
+  const char* acc;
+  int64_t acc_stride;
+  uint32_t acc_sm0, acc_spn;
+  // Dequantizing store (4-byte outputs only), applied by the launch that
+  // finishes K: element (row, col) becomes
+  //   (float)acc * row_scale[row] * col_scale[col]   (a NULL scale reads as 1)
+  // with row / col counted from this problem's origin.
+  uint32_t dequant;
+  const float* row_scale;
+  const float* col_scale;
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that
@@ -259,11 +276,12 @@ void mmt4d_mfma_kernel(Args a) {
   constexpr int R = RBC >= 16 ? 1 : 16 / RBC;
   // A loader block is 64 units (one per lane); a unit is R loads + R stores.
   constexpr int BLOCKS_A = BM * NCH / R / 64;
-  // PIPE 2 keeps only the LHS in LDS; RHS fragments come straight from global.
-  constexpr int BLOCKS = (PIPE >= 2 ? BM : BM + BN) * NCH / R / 64;
+  // PIPE 2 and 3 keep only the LHS in LDS; RHS fragments come straight from global.
+  constexpr bool RHS_DIRECT = PIPE == 2 || PIPE == 3;
+  constexpr int BLOCKS = (RHS_DIRECT ? BM : BM + BN) * NCH / R / 64;
   constexpr int NU = (BLOCKS + NW - 1) / NW;
   constexpr int IMAGE_A = BM * KS;
-  constexpr int STAGE = (PIPE >= 2 ? BM : BM + BN) * KS;
+  constexpr int STAGE = (RHS_DIRECT ? BM : BM + BN) * KS;
   static_assert((BM * NCH / R) % 64 == 0 && (BN * NCH / R) % 64 == 0, "block split");
   // When the blocks do not divide evenly over the waves, the surplus (wave, i)
   // slots are idle: they load from a valid address and skip the store.
@@ -384,13 +402,14 @@ void mmt4d_mfma_kernel(Args a) {
   // which covers both the tiled [M1][N1][M0][N0] output and a plain row-major
   // matrix (the fused mmt4d + unpack). Rows and columns at or beyond
   // out_rows / out_cols do not exist (row-major output of a ragged problem).
-  auto for_each_output = [&](auto f4, auto f1) {
+  auto for_each_output = [&](const char* base, int64_t s_panel, uint32_t s_m0, uint32_t s_pn,
+                             auto f4, auto f1) {
     // The lane coordinates pass through an empty asm so that the address
     // arithmetic of the prologue (ACCUMULATE loads) and of the epilogue
     // (stores) is not shared: shared, it would stay live across the K loop.
     uint32_t oq = q, orr = r;
     asm volatile("" : "+v"(oq), "+v"(orr));
-    char* out_base = a.out + (int64_t)pm0 * a.out_stride + (int64_t)pn0 * a.out_spn;
+    char* out_base = const_cast<char*>(base) + (int64_t)pm0 * s_panel + (int64_t)pn0 * s_pn;
     const int row_origin = pm0 * a.M0, col_origin = pn0 * a.N0;
     if (a.vec_out) {
       uint32_t col_off[TN];
@@ -402,14 +421,14 @@ void mmt4d_mfma_kernel(Args a) {
         const bool ok = pl < a.bpn && pn0 + pl < a.N1;
         const int left = a.out_cols - (col_origin + col);
         col_n[tn] = ok ? (left >= 4 ? 4 : (left > 0 ? left : 0)) : 0;
-        col_off[tn] = (uint32_t)pl * a.out_spn + (uint32_t)n0 * OB;
+        col_off[tn] = (uint32_t)pl * s_pn + (uint32_t)n0 * OB;
       }
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) {
         const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
         const bool row_ok = pl < a.bpm && pm0 + pl < a.M1 && row_origin + row < a.out_rows;
-        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)m0 * a.out_sm0;
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)s_panel + (uint32_t)m0 * s_m0;
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
           if (row_ok && col_n[tn] == 4) {
@@ -430,7 +449,7 @@ void mmt4d_mfma_kernel(Args a) {
         const int row = (wm * TM + tm) * 16 + (int)orr;
         const int pl = row / a.M0, m0 = row - pl * a.M0;
         const bool row_ok = pl < a.bpm && pm0 + pl < a.M1 && row_origin + row < a.out_rows;
-        const uint32_t row_off = (uint32_t)pl * (uint32_t)a.out_stride + (uint32_t)m0 * a.out_sm0;
+        const uint32_t row_off = (uint32_t)pl * (uint32_t)s_panel + (uint32_t)m0 * s_m0;
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
 #pragma unroll
@@ -438,7 +457,7 @@ void mmt4d_mfma_kernel(Args a) {
             const int col = (wn * TN + tn) * 16 + 4 * (int)oq + e;
             const int pc = col / a.N0, n0 = col - pc * a.N0;
             if (row_ok && pc < a.bpn && pn0 + pc < a.N1 && col_origin + col < a.out_cols)
-              f1(tm, tn, e, out_base + (row_off + (uint32_t)pc * a.out_spn + (uint32_t)n0 * OB));
+              f1(tm, tn, e, out_base + (row_off + (uint32_t)pc * s_pn + (uint32_t)n0 * OB));
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -450,7 +469,8 @@ void mmt4d_mfma_kernel(Args a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
   if (a.accumulate) {
-    for_each_output([&](int tm, int tn, char* p) { acc[tm][tn] = Out::load4(p); },
+    for_each_output(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn,
+                    [&](int tm, int tn, char* p) { acc[tm][tn] = Out::load4(p); },
                     [&](int tm, int tn, int e, char* p) { acc[tm][tn][e] = Out::load1(p); });
   }
 
@@ -544,6 +564,52 @@ void mmt4d_mfma_kernel(Args a) {
       if (s < last) store_lds(regs, cur ^ STAGE);
       __syncthreads();
     }
+  } else if constexpr (PIPE == 4) {
+    // Two LDS stages as in PIPE 0, three register sets: iteration s issues the
+    // global loads of step s+3 into the set that step s occupied, computes
+    // step s from LDS and stores step s+1 (loaded two iterations ago) for the
+    // next iteration. Unrolled by three so that the set index is static.
+    constexpr int D = 3;
+    v4i regs[D][NU][R];
+    // Workgroups walk K from different starting steps (the sum over K is
+    // order-free for the instruction): in lockstep from step 0 they would all
+    // read the same offset of their panels at the same time, and panels are a
+    // power-of-two distance apart, which concentrates the requests on a few
+    // memory channels.
+    const int rot = (int)(blockIdx.x % (uint32_t)a.steps);
+    auto load_step = [&](v4i (&dst)[NU][R], int s) {
+      int ks = s + rot;
+      if (ks >= a.steps) ks -= a.steps;
+      if (has_tail && ks == last) load_global(dst, ks, true);
+      else load_global(dst, ks, false);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      if (d <= last) load_step(regs[d], d);
+    }
+    store_lds(regs[0], 0);
+    __syncthreads();
+    auto iteration = [&](int s, auto phase) {
+      constexpr int P = decltype(phase)::value;
+      const uint32_t cur = (s & 1) * STAGE;
+      if (s + D <= last) load_step(regs[P], s + D);
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        v4i fa[TM][HALVES], fb[TN][HALVES];
+        read_frags(fa, fb, cur, kk);
+        mfmas(fa, fb);
+      }
+      if (s < last) store_lds(regs[(P + 1) % D], cur ^ STAGE);
+      __syncthreads();
+    };
+    int s = 0;
+    for (; s + 2 < a.steps; s += 3) {
+      iteration(s, std::integral_constant<int, 0>{});
+      iteration(s + 1, std::integral_constant<int, 1>{});
+      iteration(s + 2, std::integral_constant<int, 2>{});
+    }
+    if (s < a.steps) iteration(s, std::integral_constant<int, 0>{});
+    if (s + 1 < a.steps) iteration(s + 1, std::integral_constant<int, 1>{});
   } else if constexpr (PIPE == 1) {
     // Three LDS stages, two register sets. In iteration s a wave runs the
     // MFMAs of step s row by row (tm) and, between rows, issues everything
@@ -804,7 +870,46 @@ void mmt4d_mfma_kernel(Args a) {
     if (s + 1 < a.steps) iteration(s + 1, std::integral_constant<int, 1>{});
   }
   // ---- epilogue -----------------------------------------------------------
-  for_each_output([&](int tm, int tn, char* p) { Out::store4(p, acc[tm][tn]); },
+  if constexpr (OB == 4) {
+    if (a.dequant) {
+      // Scales of this lane's rows and columns; indices beyond the matrix are
+      // clamped (their elements are never stored).
+      uint32_t oq = q, orr = r;
+      asm volatile("" : "+v"(oq), "+v"(orr));
+      const int row_origin = pm0 * a.M0, col_origin = pn0 * a.N0;
+      float sm[TM];
+      v4f sn[TN];
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) {
+        const int row = max(min(row_origin + (wm * TM + tm) * 16 + (int)orr, a.out_rows - 1), 0);
+        sm[tm] = a.row_scale ? a.row_scale[row] : 1.0f;
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int col =
+              max(min(col_origin + (wn * TN + tn) * 16 + 4 * (int)oq + e, a.out_cols - 1), 0);
+          sn[tn][e] = a.col_scale ? a.col_scale[col] : 1.0f;
+        }
+      }
+      typedef v4f v4f_a4 __attribute__((aligned(4)));
+      for_each_output(
+          a.out, a.out_stride, a.out_sm0, a.out_spn,
+          [&](int tm, int tn, char* p) {
+            v4f v = __builtin_convertvector(acc[tm][tn], v4f);
+            v = v * sm[tm];
+            v = v * sn[tn];
+            *reinterpret_cast<v4f_a4*>(p) = v;
+          },
+          [&](int tm, int tn, int e, char* p) {
+            *reinterpret_cast<float*>(p) = (float)acc[tm][tn][e] * sm[tm] * sn[tn][e];
+          });
+      return;
+    }
+  }
+  for_each_output(a.out, a.out_stride, a.out_sm0, a.out_spn,
+                  [&](int tm, int tn, char* p) { Out::store4(p, acc[tm][tn]); },
                   [&](int tm, int tn, int e, char* p) { Out::store1(p, acc[tm][tn][e]); });
 }
 
@@ -815,7 +920,7 @@ struct Shape {
   static constexpr int BM = WGM * TM * 16;
   static constexpr int BN = WGN * TN * 16;
   static constexpr size_t kLdsBytes =
-      (PIPE ? 3 : 2) * (size_t)(PIPE >= 2 ? BM : BM + BN) * KS;
+      (PIPE == 0 || PIPE == 4 ? 2 : 3) * (size_t)(PIPE == 2 || PIPE == 3 ? BM : BM + BN) * KS;
 };
 
 }  // namespace uk_mfma

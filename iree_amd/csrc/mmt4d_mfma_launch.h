@@ -7,9 +7,11 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <climits>
 
 #include "mmt4d_mfma_kernel.h"
+#include "mmt4d_mfma_thin.h"
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
 #include "uk_launch.h"
@@ -27,6 +29,14 @@ struct Problem {
   // rows / columns exist counted from this problem's origin.
   int64_t out_sm0, out_spn;
   int64_t out_rows, out_cols;
+  // Initial accumulators for ACCUMULATE, addressed like the output (the output
+  // itself unless `dequant`), and the dequantizing store's scales, indexed
+  // from this problem's origin (either may be null).
+  const char* acc;
+  int64_t acc_stride, acc_sm0, acc_spn;
+  bool dequant;
+  const float* row_scale;
+  const float* col_scale;
   int32_t M1, N1, K1, M0, N0;
   int32_t rb, lrb;  // bytes per tile row and its log2
   bool accumulate;
@@ -42,6 +52,7 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   if (p.rb > SH::KS) return -1;                       // a tile row must fit one step
   if (p.M0 > SH::BM || p.N0 > SH::BN) return -1;      // at least one whole panel
   if (p.M0 % R || p.N0 % R) return -1;                // pieces hold whole rows
+  if (p.out_rows <= 0 || p.out_cols <= 0) return 0;   // a strip beyond the matrix: nothing to store
   Args a;
   const int64_t kt_bytes_m = (int64_t)p.M0 << p.lrb, kt_bytes_n = (int64_t)p.N0 << p.lrb;
   a.lhs = p.lhs + kt_begin * kt_bytes_m;
@@ -66,8 +77,19 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   a.steps = (int32_t)uk::ceil_div(k_bytes, SH::KS);
   if (a.steps < 1) a.steps = 1;
   a.tail = (k_bytes % SH::KS) != 0;
-  if (PIPE != 0 && (a.tail || kt_count == 0)) return -1;
+  if (PIPE != 0 && PIPE != 4 && (a.tail || kt_count == 0)) return -1;
   a.accumulate = accumulate;
+  // A launch that starts K reads the caller's accumulators; a later one
+  // continues from what the previous launch left in the output. Only the
+  // launch that finishes K applies the dequantizing store.
+  const bool first = kt_begin == 0;
+  a.acc = first ? p.acc : p.out;
+  a.acc_stride = first ? p.acc_stride : p.out_stride;
+  a.acc_sm0 = (uint32_t)(first ? p.acc_sm0 : p.out_sm0);
+  a.acc_spn = (uint32_t)(first ? p.acc_spn : p.out_spn);
+  a.dequant = p.dequant && kt_begin + kt_count == p.K1;
+  a.row_scale = p.row_scale;
+  a.col_scale = p.col_scale;
   a.band = 4;
   // Four consecutive output columns of one row are contiguous when they lie in
   // one tile row (N0 % 4 == 0) or when column panels follow each other without
@@ -75,16 +97,25 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   // need no more alignment than their own; 2-byte outputs move as 8-byte
   // vectors and need that alignment.
   constexpr int OB = ElemTraits<E>::Out::kOutBytes;
-  const bool contiguous4 = p.N0 % 4 == 0 || p.out_spn == (int64_t)p.N0 * OB;
-  const bool aligned4 = OB == 4 || (((uintptr_t)p.out | (uint64_t)p.out_stride |
-                                     (uint64_t)p.out_sm0 | (uint64_t)p.out_spn) % 8) == 0;
-  a.vec_out = contiguous4 && aligned4;
+  auto vector_ok = [&](const char* base, int64_t stride, int64_t sm0, int64_t spn) {
+    const bool contiguous4 = p.N0 % 4 == 0 || spn == (int64_t)p.N0 * OB;
+    const bool aligned4 = OB == 4 || (((uintptr_t)base | (uint64_t)stride | (uint64_t)sm0 |
+                                       (uint64_t)spn) % 8) == 0;
+    return contiguous4 && aligned4;
+  };
+  a.vec_out = vector_ok(p.out, p.out_stride, p.out_sm0, p.out_spn) &&
+              (!accumulate || vector_ok(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn));
   // 32-bit offsets inside a workgroup's share of each operand.
   const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
   const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
   const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.M0 * p.out_sm0 +
                          (int64_t)p.N1 * p.out_spn;
-  if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31)) return -1;
+  const int64_t span_a = (int64_t)a.bpm * a.acc_stride + (int64_t)p.M0 * a.acc_sm0 +
+                         (int64_t)p.N1 * a.acc_spn;
+  if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31) ||
+      span_a >= (1ll << 31)) {
+    return -1;
+  }
   auto kernel = mmt4d_mfma_kernel<E, RBC, TM, TN, WGM, WGN, NKK, PIPE>;
   if (SH::kLdsBytes > 64 * 1024) {
     // Raising the dynamic LDS limit is a per-function setting; do it once.
@@ -95,6 +126,50 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   }
   uk::launch(2, kernel, dim3((uint32_t)(grid_m * grid_n)), dim3(WGM * WGN * 64),
              SH::kLdsBytes, stream, a);
+  return (int)hipGetLastError();
+}
+
+// Launches the M-thin kernel (mmt4d_mfma_thin.h) over all of K. Returns a HIP
+// status, or -1 if it cannot serve the shape.
+template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
+int launch_thin(const Problem& p, hipStream_t stream) {
+  constexpr int KS = 64 * ElemTraits<E>::kHalves;
+  constexpr int OB = ElemTraits<E>::Out::kOutBytes;
+  if (p.rb > KS || p.rb < 8) return -1;
+  const int64_t k_bytes = (int64_t)p.K1 << p.lrb;
+  if (k_bytes == 0 || k_bytes % KS) return -1;
+  if (p.out_rows <= 0 || p.out_cols <= 0) return 0;
+  Args a{};
+  a.lhs = p.lhs; a.rhs = p.rhs; a.out = p.out;
+  a.lhs_stride = p.lhs_stride; a.rhs_stride = p.rhs_stride; a.out_stride = p.out_stride;
+  a.out_sm0 = (uint32_t)p.out_sm0; a.out_spn = (uint32_t)p.out_spn;
+  a.out_rows = (int32_t)std::min<int64_t>(p.out_rows, INT32_MAX);
+  a.out_cols = (int32_t)std::min<int64_t>(p.out_cols, INT32_MAX);
+  a.M1 = p.M1; a.N1 = p.N1; a.K1 = p.K1; a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
+  const int64_t grid_m = uk::ceil_div((int64_t)p.M1 * p.M0, TM * 16);
+  const int64_t grid_n = uk::ceil_div((int64_t)p.N1 * p.N0, TN * 16);
+  if (grid_m * grid_n >= (1ll << 31) || p.out_sm0 >= (1ll << 32) || p.out_spn >= (1ll << 32)) return -1;
+  a.grid_m = (int32_t)grid_m;
+  a.grid_n = (int32_t)grid_n;
+  a.steps = (int32_t)(k_bytes / KS);
+  a.accumulate = p.accumulate;
+  a.acc = p.acc; a.acc_stride = p.acc_stride;
+  a.acc_sm0 = (uint32_t)p.acc_sm0; a.acc_spn = (uint32_t)p.acc_spn;
+  a.dequant = p.dequant; a.row_scale = p.row_scale; a.col_scale = p.col_scale;
+  auto vector_ok = [&](const char* base, int64_t stride, int64_t sm0, int64_t spn) {
+    const bool contiguous4 = p.N0 % 4 == 0 || spn == (int64_t)p.N0 * OB;
+    const bool aligned4 = OB == 4 || (((uintptr_t)base | (uint64_t)stride | (uint64_t)sm0 |
+                                       (uint64_t)spn) % 8) == 0;
+    return contiguous4 && aligned4;
+  };
+  a.vec_out = vector_ok(p.out, p.out_stride, p.out_sm0, p.out_spn) &&
+              (!p.accumulate || vector_ok(p.acc, p.acc_stride, p.acc_sm0, p.acc_spn));
+  // 32-bit operand offsets inside a workgroup's panels.
+  const int64_t span_m = (int64_t)(TM * 16 / p.M0 + 2) * p.lhs_stride + k_bytes * p.M0;
+  const int64_t span_n = (int64_t)(TN * 16 / p.N0 + 2) * p.rhs_stride + k_bytes * p.N0;
+  if (span_m >= (1ll << 31) || span_n >= (1ll << 31)) return -1;
+  uk::launch(2, mmt4d_thin_kernel<E, RBC, TM, TN, KSPLIT, D>, dim3((uint32_t)(grid_m * grid_n)),
+             dim3(KSPLIT * 64), 0, stream, a);
   return (int)hipGetLastError();
 }
 
@@ -114,8 +189,12 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //         occupy the 256 CUs;
 // `forced` (1 big, 2 mid, 3 small, 4 skinny; 0 = choose) overrides the size
 // heuristic for tests and tuning.
-//   skinny 32 rows x 64 columns: M-thin (decode-shaped) problems, which are
-//         bound by streaming the RHS and want every CU pulling on it.
+//   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
+//         streaming the RHS: the barrier-free kernel of mmt4d_mfma_thin.h (16,
+//         32 or 64 rows x 32 columns per workgroup, K split over its 4 waves)
+//         when rows are at least 8 bytes wide and K is a whole number of
+//         steps, else 32 rows x 64 columns through LDS with loads three steps
+//         ahead.
 template <Elem E, int RBC>
 int launch_class(const Problem& p, int forced, hipStream_t stream, const char** name) {
   constexpr int H = ElemTraits<E>::kHalves;
@@ -128,7 +207,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   int choice;
   if (forced >= 1 && forced <= 4) {
     choice = forced;
-  } else if (rows_m <= 32 && workgroups(p, 32, 64) >= 1) {
+  } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
     choice = 4;
   } else if (workgroups(p, 256, 256) >= 192) {
     choice = 1;
@@ -180,6 +259,8 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         q = p;
         q.rhs = p.rhs + (int64_t)main_n * p.rhs_stride;
         q.out = p.out + (int64_t)main_n * p.out_spn;
+        q.acc = p.acc + (int64_t)main_n * p.acc_spn;
+        if (p.col_scale) q.col_scale = p.col_scale + (int64_t)main_n * p.N0;
         q.out_cols = p.out_cols - (int64_t)main_n * p.N0;
         q.N1 = p.N1 - main_n;
         st = launch_class<E, RBC>(q, 0, stream, &strip_name);
@@ -191,6 +272,8 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         q = p;
         q.lhs = p.lhs + (int64_t)main_m * p.lhs_stride;
         q.out = p.out + (int64_t)main_m * p.out_stride;
+        q.acc = p.acc + (int64_t)main_m * p.acc_stride;
+        if (p.row_scale) q.row_scale = p.row_scale + (int64_t)main_m * p.M0;
         q.out_rows = p.out_rows - (int64_t)main_m * p.M0;
         q.M1 = p.M1 - main_m;
         q.N1 = main_n;
@@ -218,12 +301,24 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 2;
   }
   if (choice == 4) {
+    if constexpr (RBC >= 8) {
+      int st;
+      if (rows_m <= 16) {
+        st = launch_thin<E, RBC, 1, 2, 4, 4>(p, stream);
+      } else if (rows_m <= 32) {
+        st = launch_thin<E, RBC, 2, 2, 4, 4>(p, stream);
+      } else {
+        st = launch_thin<E, RBC, 4, 2, 4, 3>(p, stream);
+      }
+      if (st >= 0) { *name = "mmt4d_mfma_thin"; return st; }
+    }
     // With 2-byte rows a 16-byte piece spans 8 rows and 32 rows do not fill a
     // loader block; that combination takes the 64x64 variant.
     if constexpr (RBC != 2) {
       // 256 bytes of K per step: these problems are bound by memory latency,
-      // and a longer step keeps more bytes in flight per workgroup.
-      int st = launch_variant<E, RBC, 2, 1, 1, 4, 4 / H, 0>(p, 0, p.K1, p.accumulate, stream);
+      // and a longer step keeps more bytes in flight per workgroup, as do the
+      // three steps of loads ahead of the MFMAs.
+      int st = launch_variant<E, RBC, 2, 1, 1, 4, 4 / H, 4>(p, 0, p.K1, p.accumulate, stream);
       if (st >= 0) { *name = "mmt4d_mfma_32x64"; return st; }
     }
     choice = 3;

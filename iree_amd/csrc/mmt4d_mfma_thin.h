@@ -1,0 +1,267 @@
+// mmt4d on the gfx950 matrix cores for M-thin (decode-shaped) problems: a few
+// rows of LHS against a long RHS. Such a call streams the RHS once and is
+// bound by memory, so the kernel is built around keeping loads in flight:
+//
+//   * no LDS staging and no barrier in the K loop. A workgroup owns TM x TN
+//     output blocks of 16x16; its KSPLIT waves take the 64-byte K steps round
+//     robin (wave w: steps w, w + KSPLIT, ...), so together they read the
+//     workgroup's RHS panels front to back;
+//   * each lane loads its MFMA operands straight from global memory, the RHS
+//     from HBM and the (small, shared) LHS from L2, D steps ahead of the MFMAs
+//     through D register buffers;
+//   * the KSPLIT partial accumulators meet in LDS once, at the end, and wave 0
+//     adds them in wave order and stores.
+//
+// Operand layout, K-order freedom of the MFMA and the output addressing are
+// those of mmt4d_mfma_kernel.h, whose Args this kernel takes. Row widths of 16
+// bytes and more load one 16-byte piece per operand; 8-byte rows load the two
+// 8-byte halves from two K-tiles (chunk g of a step holds K-tiles g and
+// g + 4). K must be a whole number of steps.
+#ifndef IREE_UK_AMD_MMT4D_MFMA_THIN_H_
+#define IREE_UK_AMD_MMT4D_MFMA_THIN_H_
+
+#include "mmt4d_mfma_kernel.h"
+
+namespace uk_mfma {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
+__global__ __launch_bounds__(KSPLIT * 64)
+void mmt4d_thin_kernel(Args a) {
+  using TT = ElemTraits<E>;
+  using Acc = typename TT::Acc;
+  using Out = typename TT::Out;
+  constexpr int OB = Out::kOutBytes;
+  constexpr int HALVES = TT::kHalves;
+  constexpr int NCH = 4 * HALVES;             // 16-byte chunks per row per step
+  constexpr int KS = NCH * 16;                // bytes of K per row per step
+  constexpr int PIECES = RBC >= 16 ? 1 : 2;   // loads per 16-byte operand
+  static_assert(RBC >= 8, "rows narrower than 8 bytes take the LDS kernels");
+
+  __shared__ v4i partial[KSPLIT > 1 ? KSPLIT - 1 : 1][TM * TN][64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t q = lane >> 4, r = lane & 15;
+  const int bm = (int)(blockIdx.x / (uint32_t)a.grid_n);
+  const int bn = (int)(blockIdx.x - (uint32_t)bm * a.grid_n);
+  const int lrb = a.lrb;
+  const uint32_t kt_m = (uint32_t)a.M0 << lrb, kt_n = (uint32_t)a.N0 << lrb;
+  const uint32_t kts_per_step = KS >> lrb;
+  const uint32_t sstep_a = kts_per_step * kt_m, sstep_b = kts_per_step * kt_n;
+
+  // Byte offset of the lane's piece(s) of block row `x` (a row of 16 rows of
+  // the M or N dimension) at K step 0; 0 for rows outside the problem, whose
+  // (valid) bytes only reach accumulators that are never stored.
+  // Offsets are 32-bit and relative to the first panel the workgroup touches.
+  const int pa0 = bm * TM * 16 / a.M0, pb0 = bn * TN * 16 / a.N0;
+  const char* base_a = a.lhs + (int64_t)pa0 * a.lhs_stride;
+  const char* base_b = a.rhs + (int64_t)pb0 * a.rhs_stride;
+  auto operand_offsets = [&](uint32_t (&off)[HALVES][PIECES], int x, int X0, int X1, int p0,
+                             int64_t stride, uint32_t kt_bytes) {
+    const uint32_t row = (uint32_t)x * 16 + r;
+    const uint32_t pabs = row / (uint32_t)X0;
+    const uint32_t x0 = row - pabs * X0;
+    const bool ok = (int)pabs < X1;
+    const uint32_t pl = pabs - (uint32_t)p0;
+#pragma unroll
+    for (int h = 0; h < HALVES; ++h) {
+      const uint32_t g = (uint32_t)h * 4 + q;
+#pragma unroll
+      for (int t = 0; t < PIECES; ++t) {
+        uint32_t o;
+        if constexpr (RBC >= 16) {
+          const uint32_t kb = g * 16;
+          o = (kb >> lrb) * kt_bytes + (x0 << lrb) + (kb & ((1u << lrb) - 1));
+        } else {
+          o = (g + (uint32_t)t * NCH) * kt_bytes + x0 * 8;
+        }
+        off[h][t] = ok ? pl * (uint32_t)stride + o : 0u;
+      }
+    }
+  };
+  uint32_t offa[TM][HALVES][PIECES], offb[TN][HALVES][PIECES];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+    operand_offsets(offa[tm], bm * TM + tm, a.M0, a.M1, pa0, a.lhs_stride, kt_m);
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)
+    operand_offsets(offb[tn], bn * TN + tn, a.N0, a.N1, pb0, a.rhs_stride, kt_n);
+
+  auto load_operand = [&](const char* base, const uint32_t (&off)[PIECES], uint32_t adv) {
+    if constexpr (RBC >= 16) {
+      return *reinterpret_cast<const v4i*>(base + (off[0] + adv));
+    } else {
+      const v2i lo = *reinterpret_cast<const v2i*>(base + (off[0] + adv));
+      const v2i hi = *reinterpret_cast<const v2i*>(base + (off[1] + adv));
+      return v4i{lo[0], lo[1], hi[0], hi[1]};
+    }
+  };
+  v4i fa[D][TM][HALVES], fb[D][TN][HALVES];
+  // Local step i of this wave is K step wave + i * KSPLIT.
+  auto load_step = [&](int d, int i) {
+    const uint32_t s = (uint32_t)(wave + i * KSPLIT);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h) fb[d][tn][h] = load_operand(base_b, offb[tn][h], s * sstep_b);
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h) fa[d][tm][h] = load_operand(base_a, offa[tm][h], s * sstep_a);
+  };
+
+  // ---- output addressing (see for_each_output in mmt4d_mfma_kernel.h) ------
+  // Lane (q, r) of block (tm, tn) holds output row r, columns 4q..4q+3.
+  auto for_each_output = [&](const char* base, int64_t s_panel, uint32_t s_m0, uint32_t s_pn,
+                             auto f4, auto f1) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const int row = (bm * TM + tm) * 16 + (int)r;
+      const int pl = row / a.M0, m0 = row - pl * a.M0;
+      const bool row_ok = pl < a.M1 && row < a.out_rows;
+      char* row_base = const_cast<char*>(base) + (int64_t)pl * s_panel + (int64_t)m0 * s_m0;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const int col = (bn * TN + tn) * 16 + 4 * (int)q;
+        if (a.vec_out) {
+          const int pc = col / a.N0, n0 = col - pc * a.N0;
+          const int left = a.out_cols - col;
+          char* p = row_base + (int64_t)pc * s_pn + (int64_t)n0 * OB;
+          if (row_ok && pc < a.N1 && left >= 4) {
+            f4(tm, tn, p);
+          } else if (row_ok && pc < a.N1) {
+#pragma unroll
+            for (int e = 0; e < 3; ++e)
+              if (e < left) f1(tm, tn, e, p + e * OB);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int c = col + e;
+            const int pc = c / a.N0, n0 = c - pc * a.N0;
+            if (row_ok && pc < a.N1 && c < a.out_cols)
+              f1(tm, tn, e, row_base + (int64_t)pc * s_pn + (int64_t)n0 * OB);
+          }
+        }
+      }
+    }
+  };
+
+  Acc acc[TM][TN];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
+
+  // ---- K loop ---------------------------------------------------------------
+  const int my_steps = (a.steps - wave + KSPLIT - 1) / KSPLIT;
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < my_steps) load_step(d, d);
+  // Wave 0, which stores, fetches what the store needs now, under the K loop:
+  // the initial accumulators and the scales of the dequantizing store (indices
+  // beyond the matrix are clamped; their elements are never stored).
+  float sm[TM];
+  v4f sn[TN];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) sm[tm] = 1.0f;
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) sn[tn] = v4f{1.0f, 1.0f, 1.0f, 1.0f};
+  if (wave == 0) {
+    if (a.accumulate) {
+      for_each_output(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn,
+                      [&](int tm, int tn, char* p) { acc[tm][tn] = Out::load4(p); },
+                      [&](int tm, int tn, int e, char* p) { acc[tm][tn][e] = Out::load1(p); });
+    }
+    if (OB == 4 && a.dequant) {
+      if (a.row_scale) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          sm[tm] = a.row_scale[max(min((bm * TM + tm) * 16 + (int)r, a.out_rows - 1), 0)];
+      }
+      if (a.col_scale) {
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            sn[tn][e] =
+                a.col_scale[max(min((bn * TN + tn) * 16 + 4 * (int)q + e, a.out_cols - 1), 0)];
+      }
+    }
+  }
+  auto compute = [&](int d) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fb[d][tn], fa[d][tm], acc[tm][tn]);
+  };
+  int i = 0;
+  // Steady state: every step computed is followed by the load of the step D
+  // further on, which exists.
+  for (; i + 2 * D <= my_steps; i += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      compute(d);
+      load_step(d, i + d + D);
+    }
+  }
+  // Fewer than 2 D steps left: the same with bounds.
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    if (i + d < my_steps) {
+      compute(d);
+      if (i + d + D < my_steps) load_step(d, i + d + D);
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (i + D + d < my_steps) compute(d);
+
+  // ---- meet the partial sums ---------------------------------------------------
+  if constexpr (KSPLIT > 1) {
+    if (wave > 0) {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          partial[wave - 1][tm * TN + tn][lane] = __builtin_bit_cast(v4i, acc[tm][tn]);
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < KSPLIT - 1; ++w)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] += __builtin_bit_cast(Acc, partial[w][tm * TN + tn][lane]);
+  }
+
+  // ---- store --------------------------------------------------------------------
+  if constexpr (OB == 4) {
+    if (a.dequant) {
+      typedef v4f v4f_a4 __attribute__((aligned(4)));
+      for_each_output(
+          a.out, a.out_stride, a.out_sm0, a.out_spn,
+          [&](int tm, int tn, char* p) {
+            v4f v = __builtin_convertvector(acc[tm][tn], v4f);
+            v = v * sm[tm];
+            v = v * sn[tn];
+            *reinterpret_cast<v4f_a4*>(p) = v;
+          },
+          [&](int tm, int tn, int e, char* p) {
+            *reinterpret_cast<float*>(p) = (float)acc[tm][tn][e] * sm[tm] * sn[tn][e];
+          });
+      return;
+    }
+  }
+  for_each_output(a.out, a.out_stride, a.out_sm0, a.out_spn,
+                  [&](int tm, int tn, char* p) { Out::store4(p, acc[tm][tn]); },
+                  [&](int tm, int tn, int e, char* p) { Out::store1(p, acc[tm][tn][e]); });
+}
+
+}  // namespace uk_mfma
+
+#endif  // IREE_UK_AMD_MMT4D_MFMA_THIN_H_

@@ -32,6 +32,17 @@ int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* params,
 typedef struct iree_uk_amd_rowmajor_out_t {
   int64_t stride0;
   int64_t size0, size1;
+  /* Dequantizing store (iree_uk_amd_mmt4d_dequant_unpack); `dequant` 0: none
+   * and the fields below are not read. The matrix is f32; element (i, j) is
+   * (float)acc * row_scale[i] * col_scale[j], a NULL scale reading as 1. With
+   * ACCUMULATE the initial accumulators come from the tiled [M][N][M0][N0]
+   * buffer `acc` (first element, offset applied; `acc_stride0` elements
+   * between rows of tiles), not from the matrix. */
+  int dequant;
+  const float* row_scale;
+  const float* col_scale;
+  const void* acc;
+  int64_t acc_stride0;
 } iree_uk_amd_rowmajor_out_t;
 
 /* `rowmajor` NULL: the result is stored tiled, as iree_uk_mmt4d does. */

@@ -270,6 +270,7 @@ static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
   iree_uk_mmt4d_params_t p = *params;
   iree_uk_amd_rowmajor_out_t rm;
   if (rowmajor) rm = *rowmajor;
+  else memset(&rm, 0, sizeof rm);
   const int out_bytes = bits.out_bits / 8;
   staged_t lhs = {(char*)p.lhs_buffer + p.lhs_offset * bits.lhs_bits / 8,
                   p.lhs_stride0 * bits.lhs_bits / 8,
@@ -285,12 +286,42 @@ static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
     out.row_bytes = rm.size1 * out_bytes;
     out.rows = rm.size0;
   }
+  /* Dequantizing store: the matrix is written in full and never read; the
+   * initial accumulators (ACCUMULATE) come from a tiled buffer of their own. */
+  const int dequant = rowmajor && rm.dequant;
+  const int accumulate = (p.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0;
+  staged_t acc = {0, 0, 0, 0, 0}, rscale = {0, 0, 0, 0, 0}, cscale = {0, 0, 0, 0, 0};
+  if (dequant) {
+    if (accumulate) {
+      acc.host_base = (char*)rm.acc;
+      acc.pitch = rm.acc_stride0 * out_bytes;
+      acc.row_bytes = p.N * p.M0 * p.N0 * out_bytes;
+      acc.rows = p.M;
+    }
+    if (rm.row_scale) {
+      rscale.host_base = (char*)rm.row_scale;
+      rscale.pitch = rscale.row_bytes = rm.size0 * (int64_t)sizeof(float);
+      rscale.rows = 1;
+    }
+    if (rm.col_scale) {
+      cscale.host_base = (char*)rm.col_scale;
+      cscale.pitch = cscale.row_bytes = rm.size1 * (int64_t)sizeof(float);
+      cscale.rows = 1;
+    }
+  }
   int st = stage_in(&lhs, 1);
   if (!st) st = stage_in(&rhs, 1);
+  if (!st) st = stage_in(&out, accumulate && !dequant);
+  if (!st) st = stage_in(&acc, 1);
+  if (!st) st = stage_in(&rscale, 1);
+  if (!st) st = stage_in(&cscale, 1);
   if (!st) {
-    st = stage_in(&out, (p.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0);
-  }
-  if (!st) {
+    if (acc.device) {
+      rm.acc = acc.device;
+      rm.acc_stride0 = p.N * p.M0 * p.N0;
+    }
+    if (rscale.device) rm.row_scale = (const float*)rscale.device;
+    if (cscale.device) rm.col_scale = (const float*)cscale.device;
     if (lhs.device) {
       p.lhs_buffer = lhs.device;
       p.lhs_offset = 0;
@@ -311,13 +342,17 @@ static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
                                       tls_kernel_mode, &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
-  if (lhs.device || rhs.device || out.device) {
+  if (lhs.device || rhs.device || out.device || acc.device || rscale.device ||
+      cscale.device) {
     int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
     if (!st) st = st2;
   }
   stage_free(&lhs);
   stage_free(&rhs);
   stage_free(&out);
+  stage_free(&acc);
+  stage_free(&rscale);
+  stage_free(&cscale);
   tls_status = st;
 }
 
@@ -358,8 +393,11 @@ void iree_uk_amd_mmt4d_unpack_p(const iree_uk_amd_mmt4d_unpack_params_t* params)
       (params->K == 0 && (params->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE))) {
     return;
   }
-  const iree_uk_amd_rowmajor_out_t rm = {params->out_stride0, params->out_size0,
-                                         params->out_size1};
+  iree_uk_amd_rowmajor_out_t rm;
+  memset(&rm, 0, sizeof rm);
+  rm.stride0 = params->out_stride0;
+  rm.size0 = params->out_size0;
+  rm.size1 = params->out_size1;
   mmt4d_run(&mm, &rm);
 }
 
@@ -378,6 +416,69 @@ void iree_uk_amd_mmt4d_unpack(const void* lhs_buffer, iree_uk_index_t lhs_offset
       N,          K,          M0,          N0,         K0,         flags,
       cpu_data};
   iree_uk_amd_mmt4d_unpack_p(&params);
+}
+
+/* Fused mmt4d + dequantizing unpack: a 32-bit accumulator type, a matrix
+ * inside the tiles, and an accumulator buffer whenever one is to be read. */
+static int mmt4d_dequant_validate(
+    const iree_uk_amd_mmt4d_dequant_unpack_params_t* p,
+    const iree_uk_mmt4d_params_t* mm) {
+  if (!mmt4d_validate(mm)) return 0;
+  mmt4d_bits_t bits;
+  mmt4d_type_bits(mm->flags, &bits);
+  UK_REQUIRE(bits.out_bits == 32);
+  UK_REQUIRE(p->out_size0 >= 0 && p->out_size0 <= p->M * p->M0);
+  UK_REQUIRE(p->out_size1 >= 0 && p->out_size1 <= p->N * p->N0);
+  UK_REQUIRE(!(p->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) || p->acc_buffer != 0);
+  return 1;
+}
+
+void iree_uk_amd_mmt4d_dequant_unpack_p(
+    const iree_uk_amd_mmt4d_dequant_unpack_params_t* params) {
+  tls_status = 0;
+  tls_kernel_name = "";
+  const iree_uk_mmt4d_params_t mm = {
+      params->lhs_buffer, params->lhs_offset, params->lhs_stride0,
+      params->rhs_buffer, params->rhs_offset, params->rhs_stride0,
+      params->out_buffer, params->out_offset, /*out_stride0=*/0,
+      params->M, params->N, params->K, params->M0, params->N0, params->K0,
+      params->flags, params->cpu_data};
+  if (!mmt4d_dequant_validate(params, &mm)) return;
+  /* Nothing to write. Unlike iree_uk_mmt4d, K == 0 with ACCUMULATE is not a
+   * no-op here: the accumulators still have to reach the matrix, scaled. */
+  if (params->M == 0 || params->N == 0 || params->out_size0 == 0 ||
+      params->out_size1 == 0) {
+    return;
+  }
+  iree_uk_amd_rowmajor_out_t rm;
+  memset(&rm, 0, sizeof rm);
+  rm.stride0 = params->out_stride0;
+  rm.size0 = params->out_size0;
+  rm.size1 = params->out_size1;
+  rm.dequant = 1;
+  rm.row_scale = params->row_scale;
+  rm.col_scale = params->col_scale;
+  if (params->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) {
+    rm.acc = (const char*)params->acc_buffer + params->acc_offset * 4;
+    rm.acc_stride0 = params->acc_stride0;
+  }
+  mmt4d_run(&mm, &rm);
+}
+
+void iree_uk_amd_mmt4d_dequant_unpack(
+    const void* lhs_buffer, iree_uk_index_t lhs_offset, iree_uk_index_t lhs_stride0,
+    const void* rhs_buffer, iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0,
+    const void* acc_buffer, iree_uk_index_t acc_offset, iree_uk_index_t acc_stride0,
+    void* out_buffer, iree_uk_index_t out_offset, iree_uk_index_t out_stride0,
+    iree_uk_index_t out_size0, iree_uk_index_t out_size1, const float* row_scale,
+    const float* col_scale, iree_uk_index_t M, iree_uk_index_t N, iree_uk_index_t K,
+    int32_t M0, int32_t N0, int32_t K0, uint32_t flags, const uint64_t* cpu_data) {
+  iree_uk_amd_mmt4d_dequant_unpack_params_t params = {
+      lhs_buffer, lhs_offset, lhs_stride0, rhs_buffer, rhs_offset, rhs_stride0,
+      acc_buffer, acc_offset, acc_stride0, out_buffer, out_offset, out_stride0,
+      out_size0,  out_size1,  row_scale,   col_scale,  M,          N,
+      K,          M0,         N0,          K0,         flags,      cpu_data};
+  iree_uk_amd_mmt4d_dequant_unpack_p(&params);
 }
 
 void iree_uk_mmt4d(const void* lhs_buffer, iree_uk_index_t lhs_offset,

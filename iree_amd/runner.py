@@ -287,6 +287,32 @@ class Runner:
                             [op, ep], op.flops, op.bytes, "s8",
                             dict(act=act, w=w, lhs4=lhs4, rhs4=rhs4, out4=out4, y=y, scale_m=scale_m,
                                  scale_n=scale_n, M1=M1, N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
+        if name == "c3_s8_decode_fused":
+            # The same layer through the fused entry point: accumulators read
+            # from the tiled s32 buffer, result scaled into the row-major f32
+            # matrix by the mmt4d kernel itself (no separate epilogue pass).
+            base = self.workload("c3_s8_decode")
+            t = base.keep
+            Mlog, N = t["act"].shape[0], t["w"].shape[0]
+            M1, N1, K1, M0, N0, K0 = (t[k] for k in ("M1", "N1", "K1", "M0", "N0", "K0"))
+            y = torch.empty(Mlog, N, device="cuda", dtype=torch.float32)
+            lib = self.lib
+            ptrs = [t[k].data_ptr() for k in ("lhs4", "rhs4", "out4", "scale_m", "scale_n")]
+            yp = y.data_ptr()
+            flags = uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE
+
+            def launch():
+                lib.mmt4d_dequant_unpack(ptrs[0], 0, K1 * M0 * K0, ptrs[1], 0, K1 * N0 * K0,
+                                         ptrs[2], 0, N1 * M0 * N0, yp, 0, N, Mlog, N,
+                                         ptrs[3], ptrs[4], M1, N1, K1, M0, N0, K0, flags)
+            nbytes = (M1 * K1 * M0 * K0 + N1 * K1 * N0 * K0 + M1 * N1 * M0 * N0 * 4 +
+                      Mlog * N * 4 + (Mlog + N) * 4)
+            op = Op("mmt4d", launch, base.flops, float(nbytes), "hbm", "s8")
+            tensors = dict(t)
+            tensors["y_fused"] = y
+            return Workload(name, "fused mmt4d + dequantizing unpack, s8 decode M=16(32) K=4096 N=14336 "
+                            "tiles 32x16x8 ACCUMULATE, per-row/per-column scales",
+                            [op], base.flops, float(nbytes), "s8", tensors)
         if name == "c4_f8_prefill":
             M, K, N = 2048, 8192, 28672
             M0, N0, K0 = 16, 16, 32

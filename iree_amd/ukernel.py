@@ -142,6 +142,10 @@ class UKernelLibrary:
                                                _i64, _i64, _i64, _i64, _i64, _i64,
                                                _i64, _i32, _i32, _i32, _u32, _vp]
         L.iree_uk_amd_mmt4d_unpack.restype = None
+        L.iree_uk_amd_mmt4d_dequant_unpack.argtypes = (
+            [_vp, _i64, _i64] * 4 + [_i64, _i64, _vp, _vp, _i64, _i64, _i64,
+                                     _i32, _i32, _i32, _u32, _vp])
+        L.iree_uk_amd_mmt4d_dequant_unpack.restype = None
         L.iree_uk_conv_nchwc.argtypes = ([_vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64,
                                           _vp, _i64, _i64, _i64, _i64] + [_i64] * 7 +
                                          [_i32] * 4 + [_u32, _vp])
@@ -201,6 +205,18 @@ class UKernelLibrary:
                                           rhs_stride0, out, out_offset, out_stride0,
                                           out_size0, out_size1, M, N, K, M0, N0, K0,
                                           flags, cpu_data)
+        self._check()
+
+    def mmt4d_dequant_unpack(self, lhs, lhs_offset, lhs_stride0, rhs, rhs_offset, rhs_stride0,
+                             acc, acc_offset, acc_stride0, out, out_offset, out_stride0,
+                             out_size0, out_size1, row_scale, col_scale, M, N, K,
+                             M0, N0, K0, flags, cpu_data=None):
+        """mmt4d into a row-major f32 matrix, scaled per row and per column;
+        `acc` is the tiled accumulator input read with ACCUMULATE."""
+        self.lib.iree_uk_amd_mmt4d_dequant_unpack(
+            lhs, lhs_offset, lhs_stride0, rhs, rhs_offset, rhs_stride0, acc, acc_offset,
+            acc_stride0, out, out_offset, out_stride0, out_size0, out_size1, row_scale,
+            col_scale, M, N, K, M0, N0, K0, flags, cpu_data)
         self._check()
 
     def conv_nchwc(self, inp, input_offset, input_stride_n, input_stride_ic_outer,
