@@ -201,6 +201,13 @@ struct Args {
   uint32_t dequant;
   const float* row_scale;
   const float* col_scale;
+  // mmt4d_mfma_thin.h only: bytes between consecutive columns inside a tile
+  // row (the element size, unless the launcher has swapped the operands and
+  // with them the meaning of rows and columns), and whether the column scale
+  // is applied before the row scale (again the swapped case, which must keep
+  // the caller's order of the two multiplications).
+  uint32_t out_sn0, acc_sn0;
+  uint32_t col_scale_first;
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that

@@ -131,10 +131,27 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
 
 // Launches the M-thin kernel (mmt4d_mfma_thin.h) over all of K. Returns a HIP
 // status, or -1 if it cannot serve the shape.
+// `swapped`: the caller's problem is N-thin and is computed as its transpose
+// (out^T = rhs * lhs^T): the kernel's rows are the caller's columns.
 template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
-int launch_thin(const Problem& p, hipStream_t stream) {
+int launch_thin(const Problem& caller, bool swapped, hipStream_t stream) {
+  constexpr int OBYTES = ElemTraits<E>::Out::kOutBytes;
+  Problem p = caller;
+  if (swapped) {
+    std::swap(p.lhs, p.rhs);
+    std::swap(p.lhs_stride, p.rhs_stride);
+    std::swap(p.M1, p.N1);
+    std::swap(p.M0, p.N0);
+    std::swap(p.out_rows, p.out_cols);
+    std::swap(p.row_scale, p.col_scale);
+    // Element (row i, col j) of the caller sits at
+    //   (i / M0) * stride + (i % M0) * sm0 + (j / N0) * spn + (j % N0) * elem;
+    // the kernel's row is j and its column is i.
+    std::swap(p.out_stride, p.out_spn);
+    std::swap(p.acc_stride, p.acc_spn);
+  }
   constexpr int KS = 64 * ElemTraits<E>::kHalves;
-  constexpr int OB = ElemTraits<E>::Out::kOutBytes;
+  constexpr int OB = OBYTES;
   if (p.rb > KS || p.rb < 8) return -1;
   const int64_t k_bytes = (int64_t)p.K1 << p.lrb;
   if (k_bytes == 0 || k_bytes % KS) return -1;
@@ -142,27 +159,35 @@ int launch_thin(const Problem& p, hipStream_t stream) {
   Args a{};
   a.lhs = p.lhs; a.rhs = p.rhs; a.out = p.out;
   a.lhs_stride = p.lhs_stride; a.rhs_stride = p.rhs_stride; a.out_stride = p.out_stride;
-  a.out_sm0 = (uint32_t)p.out_sm0; a.out_spn = (uint32_t)p.out_spn;
+  a.out_sm0 = (uint32_t)(swapped ? OBYTES : p.out_sm0);
+  a.out_sn0 = (uint32_t)(swapped ? p.out_sm0 : OBYTES);
+  a.out_spn = (uint32_t)p.out_spn;
   a.out_rows = (int32_t)std::min<int64_t>(p.out_rows, INT32_MAX);
   a.out_cols = (int32_t)std::min<int64_t>(p.out_cols, INT32_MAX);
   a.M1 = p.M1; a.N1 = p.N1; a.K1 = p.K1; a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
   const int64_t grid_m = uk::ceil_div((int64_t)p.M1 * p.M0, TM * 16);
   const int64_t grid_n = uk::ceil_div((int64_t)p.N1 * p.N0, TN * 16);
-  if (grid_m * grid_n >= (1ll << 31) || p.out_sm0 >= (1ll << 32) || p.out_spn >= (1ll << 32)) return -1;
+  if (grid_m * grid_n >= (1ll << 31) || p.out_sm0 >= (1ll << 32) || p.out_spn >= (1ll << 32) ||
+      p.acc_sm0 >= (1ll << 32) || p.acc_spn >= (1ll << 32)) {
+    return -1;
+  }
   a.grid_m = (int32_t)grid_m;
   a.grid_n = (int32_t)grid_n;
   a.steps = (int32_t)(k_bytes / KS);
   a.accumulate = p.accumulate;
   a.acc = p.acc; a.acc_stride = p.acc_stride;
-  a.acc_sm0 = (uint32_t)p.acc_sm0; a.acc_spn = (uint32_t)p.acc_spn;
+  a.acc_sm0 = (uint32_t)(swapped ? OBYTES : p.acc_sm0);
+  a.acc_sn0 = (uint32_t)(swapped ? p.acc_sm0 : OBYTES);
+  a.acc_spn = (uint32_t)p.acc_spn;
   a.dequant = p.dequant; a.row_scale = p.row_scale; a.col_scale = p.col_scale;
+  a.col_scale_first = swapped;
   auto vector_ok = [&](const char* base, int64_t stride, int64_t sm0, int64_t spn) {
     const bool contiguous4 = p.N0 % 4 == 0 || spn == (int64_t)p.N0 * OB;
     const bool aligned4 = OB == 4 || (((uintptr_t)base | (uint64_t)stride | (uint64_t)sm0 |
                                        (uint64_t)spn) % 8) == 0;
     return contiguous4 && aligned4;
   };
-  a.vec_out = vector_ok(p.out, p.out_stride, p.out_sm0, p.out_spn) &&
+  a.vec_out = !swapped && vector_ok(p.out, p.out_stride, p.out_sm0, p.out_spn) &&
               (!p.accumulate || vector_ok(p.acc, p.acc_stride, p.acc_sm0, p.acc_spn));
   // 32-bit operand offsets inside a workgroup's panels.
   const int64_t span_m = (int64_t)(TM * 16 / p.M0 + 2) * p.lhs_stride + k_bytes * p.M0;
@@ -187,8 +212,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //   mid   128x128, 4 waves, any K;
 //   small 64x64, 4 waves, any K: for problems with too few 128x128 blocks to
 //         occupy the 256 CUs;
-// `forced` (1 big, 2 mid, 3 small, 4 skinny; 0 = choose) overrides the size
-// heuristic for tests and tuning.
+// `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem;
+// 0 = choose) overrides the size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
 //         streaming the RHS: the barrier-free kernel of mmt4d_mfma_thin.h (16,
 //         32 or 64 rows x 32 columns per workgroup, K split over its 4 waves)
@@ -205,10 +230,12 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced >= 1 && forced <= 4) {
+  if (forced >= 1 && forced <= 5) {
     choice = forced;
   } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
     choice = 4;
+  } else if (RBC >= 8 && (int64_t)p.N1 * p.N0 <= 64) {
+    choice = 5;
   } else if (workgroups(p, 256, 256) >= 192) {
     choice = 1;
   } else if (workgroups(p, 128, 128) >= 192) {
@@ -300,15 +327,32 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     }
     choice = 2;
   }
+  if (choice == 5) {
+    // N-thin (a few columns against many rows, e.g. the last column strip of
+    // a ragged problem): the thin kernel on the transposed problem.
+    if constexpr (RBC >= 8) {
+      const int64_t cols_n = (int64_t)p.N1 * p.N0;
+      int st;
+      if (cols_n <= 16) {
+        st = launch_thin<E, RBC, 1, 2, 4, 4>(p, true, stream);
+      } else if (cols_n <= 32) {
+        st = launch_thin<E, RBC, 2, 2, 4, 4>(p, true, stream);
+      } else {
+        st = launch_thin<E, RBC, 4, 2, 4, 3>(p, true, stream);
+      }
+      if (st >= 0) { *name = "mmt4d_mfma_thin_transposed"; return st; }
+    }
+    choice = 3;
+  }
   if (choice == 4) {
     if constexpr (RBC >= 8) {
       int st;
       if (rows_m <= 16) {
-        st = launch_thin<E, RBC, 1, 2, 4, 4>(p, stream);
+        st = launch_thin<E, RBC, 1, 2, 4, 4>(p, false, stream);
       } else if (rows_m <= 32) {
-        st = launch_thin<E, RBC, 2, 2, 4, 4>(p, stream);
+        st = launch_thin<E, RBC, 2, 2, 4, 4>(p, false, stream);
       } else {
-        st = launch_thin<E, RBC, 4, 2, 4, 3>(p, stream);
+        st = launch_thin<E, RBC, 4, 2, 4, 3>(p, false, stream);
       }
       if (st >= 0) { *name = "mmt4d_mfma_thin"; return st; }
     }

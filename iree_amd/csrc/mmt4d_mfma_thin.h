@@ -13,7 +13,11 @@
 //     adds them in wave order and stores.
 //
 // Operand layout, K-order freedom of the MFMA and the output addressing are
-// those of mmt4d_mfma_kernel.h, whose Args this kernel takes. Row widths of 16
+// those of mmt4d_mfma_kernel.h, whose Args this kernel takes. The launcher may
+// hand the operands over swapped (RHS as LHS) to serve N-thin problems: rows
+// and columns then trade places in Args, four consecutive columns of the
+// kernel are four rows of the caller's matrix (so `vec_out` is 0), and the
+// scales of a dequantizing store are applied column scale first. Row widths of 16
 // bytes and more load one 16-byte piece per operand; 8-byte rows load the two
 // 8-byte halves from two K-tiles (chunk g of a step holds K-tiles g and
 // g + 4). K must be a whole number of steps.
@@ -115,7 +119,7 @@ void mmt4d_thin_kernel(Args a) {
   // ---- output addressing (see for_each_output in mmt4d_mfma_kernel.h) ------
   // Lane (q, r) of block (tm, tn) holds output row r, columns 4q..4q+3.
   auto for_each_output = [&](const char* base, int64_t s_panel, uint32_t s_m0, uint32_t s_pn,
-                             auto f4, auto f1) {
+                             uint32_t s_n0, auto f4, auto f1) {
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
       const int row = (bm * TM + tm) * 16 + (int)r;
@@ -128,13 +132,13 @@ void mmt4d_thin_kernel(Args a) {
         if (a.vec_out) {
           const int pc = col / a.N0, n0 = col - pc * a.N0;
           const int left = a.out_cols - col;
-          char* p = row_base + (int64_t)pc * s_pn + (int64_t)n0 * OB;
+          char* p = row_base + (int64_t)pc * s_pn + (int64_t)n0 * s_n0;
           if (row_ok && pc < a.N1 && left >= 4) {
             f4(tm, tn, p);
           } else if (row_ok && pc < a.N1) {
 #pragma unroll
             for (int e = 0; e < 3; ++e)
-              if (e < left) f1(tm, tn, e, p + e * OB);
+              if (e < left) f1(tm, tn, e, p + e * s_n0);
           }
         } else {
 #pragma unroll
@@ -142,7 +146,7 @@ void mmt4d_thin_kernel(Args a) {
             const int c = col + e;
             const int pc = c / a.N0, n0 = c - pc * a.N0;
             if (row_ok && pc < a.N1 && c < a.out_cols)
-              f1(tm, tn, e, row_base + (int64_t)pc * s_pn + (int64_t)n0 * OB);
+              f1(tm, tn, e, row_base + (int64_t)pc * s_pn + (int64_t)n0 * s_n0);
           }
         }
       }
@@ -171,7 +175,7 @@ void mmt4d_thin_kernel(Args a) {
   for (int tn = 0; tn < TN; ++tn) sn[tn] = v4f{1.0f, 1.0f, 1.0f, 1.0f};
   if (wave == 0) {
     if (a.accumulate) {
-      for_each_output(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn,
+      for_each_output(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn, a.acc_sn0,
                       [&](int tm, int tn, char* p) { acc[tm][tn] = Out::load4(p); },
                       [&](int tm, int tn, int e, char* p) { acc[tm][tn][e] = Out::load1(p); });
     }
@@ -244,20 +248,27 @@ void mmt4d_thin_kernel(Args a) {
     if (a.dequant) {
       typedef v4f v4f_a4 __attribute__((aligned(4)));
       for_each_output(
-          a.out, a.out_stride, a.out_sm0, a.out_spn,
+          a.out, a.out_stride, a.out_sm0, a.out_spn, a.out_sn0,
           [&](int tm, int tn, char* p) {
             v4f v = __builtin_convertvector(acc[tm][tn], v4f);
-            v = v * sm[tm];
-            v = v * sn[tn];
+            if (a.col_scale_first) {
+              v = v * sn[tn];
+              v = v * sm[tm];
+            } else {
+              v = v * sm[tm];
+              v = v * sn[tn];
+            }
             *reinterpret_cast<v4f_a4*>(p) = v;
           },
           [&](int tm, int tn, int e, char* p) {
-            *reinterpret_cast<float*>(p) = (float)acc[tm][tn][e] * sm[tm] * sn[tn][e];
+            const float v = (float)acc[tm][tn][e];
+            *reinterpret_cast<float*>(p) =
+                a.col_scale_first ? v * sn[tn][e] * sm[tm] : v * sm[tm] * sn[tn][e];
           });
       return;
     }
   }
-  for_each_output(a.out, a.out_stride, a.out_sm0, a.out_spn,
+  for_each_output(a.out, a.out_stride, a.out_sm0, a.out_spn, a.out_sn0,
                   [&](int tm, int tn, char* p) { Out::store4(p, acc[tm][tn]); },
                   [&](int tm, int tn, int e, char* p) { Out::store1(p, acc[tm][tn][e]); });
 }

@@ -84,8 +84,9 @@ def _mfma_shapes(M0, N0, K0, bits):
 # 128x128, 64x64 and M-thin workgroup shapes (a forced shape that cannot serve
 # a case falls through to the next one that can; 4 is the barrier-free thin
 # kernel when K is a whole number of 64-byte steps and rows are at least 8
-# bytes wide, else the 32x64 kernel through LDS: the shapes below have both).
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+# bytes wide, else the 32x64 kernel through LDS: the shapes below have both;
+# 5 is the thin kernel on the transposed problem, under the same conditions).
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("n", range(len(MFMA_TILES)))
 def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu
@@ -132,7 +133,7 @@ def test_mmt4d_split_off_remainder_strips(gpu, oracle, shape):
 # single rounding at the end (SKIP_INTERMEDIATE_ROUNDINGS); on the reference
 # tests' small-integer inputs every f32 partial sum is exact, so the result must
 # equal the oracle's bit for bit, final rounding included.
-@pytest.mark.parametrize("variant", [0, 1, 3, 4])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5])
 @pytest.mark.parametrize("tf,M0,N0,K0", [
     (uk.MMT4D_TYPE_F16F16F16, 16, 16, 8), (uk.MMT4D_TYPE_F16F16F16, 16, 16, 1),
     (uk.MMT4D_TYPE_BF16BF16BF16, 16, 16, 8), (uk.MMT4D_TYPE_BF16BF16BF16, 8, 32, 2)])
