@@ -582,8 +582,9 @@ void mmt4d_mfma_kernel(Args a) {
     // order-free for the instruction): in lockstep from step 0 they would all
     // read the same offset of their panels at the same time, and panels are a
     // power-of-two distance apart, which concentrates the requests on a few
-    // memory channels.
-    const int rot = (int)(blockIdx.x % (uint32_t)a.steps);
+    // memory channels. Integer accumulators only: there the order cannot
+    // show in the result, while float sums would differ between workgroups.
+    const int rot = std::is_same<Acc, v4i>::value ? (int)(blockIdx.x % (uint32_t)a.steps) : 0;
     auto load_step = [&](v4i (&dst)[NU][R], int s) {
       int ks = s + rot;
       if (ks >= a.steps) ks -= a.steps;

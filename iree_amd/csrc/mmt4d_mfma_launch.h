@@ -7,7 +7,6 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-#include <cstdlib>
 #include <climits>
 
 #include "mmt4d_mfma_kernel.h"
@@ -212,8 +211,9 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //   mid   128x128, 4 waves, any K;
 //   small 64x64, 4 waves, any K: for problems with too few 128x128 blocks to
 //         occupy the 256 CUs;
-// `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem;
-// 0 = choose) overrides the size heuristic for tests and tuning.
+// `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem,
+// 6 the 64x64 K-split kernel; 0 = choose) overrides the size heuristic for
+// tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
 //         streaming the RHS: the barrier-free kernel of mmt4d_mfma_thin.h (16,
 //         32 or 64 rows x 32 columns per workgroup, K split over its 4 waves)
@@ -230,7 +230,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced >= 1 && forced <= 5) {
+  if (forced >= 1 && forced <= 6) {
     choice = forced;
   } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
     choice = 4;
@@ -240,6 +240,10 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 1;
   } else if (workgroups(p, 128, 128) >= 192) {
     choice = 2;
+  } else if (RBC >= 8 && ((int64_t)p.K1 << p.lrb) >= 8192) {
+    // Measured: with 8 KiB of K per row and more, the 64x64 blocks' operands
+    // outgrow the L2 and the K-split kernel's deeper queue of loads wins.
+    choice = 6;
   } else {
     choice = 3;
   }
@@ -326,6 +330,15 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
       if (st > 0) return st;
     }
     choice = 2;
+  }
+  if (choice == 6) {
+    // Few 64x64 blocks and a long K: the barrier-free kernel with a 64x64
+    // block per workgroup, whose four waves split K.
+    if constexpr (RBC >= 8) {
+      int st = launch_thin<E, RBC, 4, 4, 4, 2>(p, false, stream);
+      if (st >= 0) { *name = "mmt4d_mfma_64x64_ksplit"; return st; }
+    }
+    choice = 3;
   }
   if (choice == 5) {
     // N-thin (a few columns against many rows, e.g. the last column strip of
