@@ -19,6 +19,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 #include <utility>
 
 #include "uk_device_common.h"
@@ -512,11 +513,101 @@ __device__ __forceinline__ typename GBytes<N>::type lds_load_pieces(const char* 
   return *reinterpret_cast<const typename GBytes<N>::type*>(tmp);
 }
 
-template <int G, int VEC, int MV, bool UNPACK, int BLK>
-__global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
+// The same with the piece size known at compile time (P divides N, P >= 4):
+// the hot path of the streaming kernels picks P once per block.
+template <int N> struct Words { uint32_t w[N / 4]; };
+template <int N, int P>
+__device__ __forceinline__ void lds_store_static(char* dst, typename GBytes<N>::type v) {
+  if constexpr (P >= N) {
+    *reinterpret_cast<typename GBytes<N>::type*>(dst) = v;
+  } else {
+    const Words<N> x = __builtin_bit_cast(Words<N>, v);
+#pragma unroll
+    for (int j = 0; j < N / P; ++j) {
+      Words<P> y;
+#pragma unroll
+      for (int k = 0; k < P / 4; ++k) y.w[k] = x.w[j * (P / 4) + k];
+      *reinterpret_cast<typename GBytes<P>::type*>(dst + j * P) =
+          __builtin_bit_cast(typename GBytes<P>::type, y);
+    }
+  }
+}
+template <int N, int P>
+__device__ __forceinline__ typename GBytes<N>::type lds_load_static(const char* src) {
+  if constexpr (P >= N) {
+    return *reinterpret_cast<const typename GBytes<N>::type*>(src);
+  } else {
+    Words<N> x;
+#pragma unroll
+    for (int j = 0; j < N / P; ++j) {
+      const Words<P> y = __builtin_bit_cast(
+          Words<P>, *reinterpret_cast<const typename GBytes<P>::type*>(src + j * P));
+#pragma unroll
+      for (int k = 0; k < P / 4; ++k) x.w[j * (P / 4) + k] = y.w[k];
+    }
+    return __builtin_bit_cast(typename GBytes<N>::type, x);
+  }
+}
+// Four words rotated by a per-lane amount s in 0..3: y[g] = x[(g - s) & 3]
+// (rotate_up) or y[g] = x[(g + s) & 3] (rotate_down), as selects.
+__device__ __forceinline__ void rotate_up4(uint32_t (&x)[4], uint32_t s) {
+  const bool b1 = s & 1, b2 = s & 2;
+  const uint32_t a0 = b1 ? x[3] : x[0], a1 = b1 ? x[0] : x[1], a2 = b1 ? x[1] : x[2],
+                 a3 = b1 ? x[2] : x[3];
+  x[0] = b2 ? a2 : a0; x[1] = b2 ? a3 : a1; x[2] = b2 ? a0 : a2; x[3] = b2 ? a1 : a3;
+}
+__device__ __forceinline__ void rotate_down4(uint32_t (&x)[4], uint32_t s) {
+  rotate_up4(x, (4 - s) & 3);
+}
+
+// A tiled-side vector of VEC bytes from / to its VEC / G granules in LDS.
+// With four 4-byte granules per vector a lane may visit its granules in
+// rotated order (`off` is then the rotated table, access k touching granule
+// (k + rot) & 3) so that the lanes of one LDS instruction spread over the
+// banks; the words are rotated back in registers.
+template <int VEC, int G>
+__device__ __forceinline__ typename GBytes<VEC>::type gather_granules(
+    const char* lbuf, const uint32_t (&off)[VEC / G], uint32_t rot) {
+  Words<VEC> x;
+#pragma unroll
+  for (int k = 0; k < VEC / G; ++k) {
+    const Words<G> y = __builtin_bit_cast(
+        Words<G>, *reinterpret_cast<const typename GBytes<G>::type*>(lbuf + off[k]));
+#pragma unroll
+    for (int j = 0; j < G / 4; ++j) x.w[k * (G / 4) + j] = y.w[j];
+  }
+  if constexpr (VEC == 16 && G == 4) rotate_up4(x.w, rot);
+  return __builtin_bit_cast(typename GBytes<VEC>::type, x);
+}
+template <int VEC, int G>
+__device__ __forceinline__ void scatter_granules(char* lbuf, const uint32_t (&off)[VEC / G],
+                                                 typename GBytes<VEC>::type v, uint32_t rot) {
+  Words<VEC> x = __builtin_bit_cast(Words<VEC>, v);
+  if constexpr (VEC == 16 && G == 4) rotate_down4(x.w, rot);
+#pragma unroll
+  for (int k = 0; k < VEC / G; ++k) {
+    Words<G> y;
+#pragma unroll
+    for (int j = 0; j < G / 4; ++j) y.w[j] = x.w[k * (G / 4) + j];
+    *reinterpret_cast<typename GBytes<G>::type*>(lbuf + off[k]) =
+        __builtin_bit_cast(typename GBytes<G>::type, y);
+  }
+}
+// Calls f with the piece size as a compile-time constant (4, 8 or 16, capped
+// at N); false when `piece` is none of them.
+template <int N, typename F>
+__device__ __forceinline__ bool with_static_piece(uint32_t piece, F f) {
+  if (piece >= N) { f(std::integral_constant<int, N>{}); return true; }
+  if (N > 8 && piece == 8) { f(std::integral_constant<int, (N > 8 ? 8 : N)>{}); return true; }
+  if (N > 4 && piece == 4) { f(std::integral_constant<int, 4>{}); return true; }
+  return false;
+}
+
+template <int G, int VEC, int MV, bool UNPACK, int BLK, int NT = kThreads, int DEPTH = 2>
+__global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  constexpr int N1 = BLK / MV / kThreads;   // 2-D side items per thread
-  constexpr int N2 = BLK / VEC / kThreads;  // tiled side items per thread
+  constexpr int N1 = BLK / MV / NT;   // 2-D side items per thread
+  constexpr int N2 = BLK / VEC / NT;  // tiled side items per thread
   constexpr int NG = VEC / G;                             // granules per tiled vector
   using MatVec = typename GBytes<MV>::type;
   using TileVec = typename GBytes<VEC>::type;
@@ -534,7 +625,7 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
 #pragma unroll
   for (int i = 0; i < N1; ++i) {
     uint32_t r, cb;
-    mat_item<MV>(a, tid + i * kThreads, &r, &cb);
+    mat_item<MV>(a, tid + i * NT, &r, &cb);
     g1off[i] = r * a.mat_stride0_bytes32 + cb;
     l1off[i] = r * a.lds_pitch + cb;
   }
@@ -542,12 +633,37 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
 #pragma unroll
   for (int i = 0; i < N2; ++i) {
     uint32_t run, t, in_tile, tl0, tl1;
-    tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+    tiled_item<VEC>(a, tid + i * NT, &run, &t, &in_tile, &tl0, &tl1);
     g2off[i] = tl0 * a.sl0_bytes32 + tl1 * a.sl1_bytes32 + in_tile;
     for_each_granule<G, VEC>(a, run, t, in_tile, [&](int k, uint32_t off) { l2off[i][k] = off; });
   }
+  // Granule rotation (see gather_granules). With 4-byte granules, granule k of
+  // a vector lies k LDS rows below granule 0 and the 32 lanes of a half wave
+  // that walk one run sit 4 rows apart: unrotated, one LDS instruction would
+  // reach only 8 of the 32 banks. Lane groups of 8 take rotations 0..3. The
+  // position of a thread's vectors inside their run is the same for all of
+  // its items when the run length divides the workgroup size.
+  uint32_t rot = 0;
+  if constexpr (NG == 4 && G == 4) {
+    if ((a.run_vecs % 32 == 0 || a.run_vecs == 16) && NT % a.run_vecs == 0) {
+      // Runs of 16 vectors put two runs (neighbouring LDS columns, one bank
+      // apart) in a half wave: their lane groups take rotations 0 and 2.
+      const uint32_t v = tid % a.run_vecs;
+      rot = a.run_vecs == 16 ? ((v >> 3) & 1) * 2 : (v >> 3) & 3;
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        // table[k] = original[(k + rot) & 3]
+        rotate_down4(l2off[i], rot);
+      }
+    }
+  }
 
   const uint32_t nblocks = a.nblk0 * a.nblk1;
+  // Every thread has all of its N1 and N2 items and the LDS piece size is one
+  // of the compile-time cases: interior blocks then run without per-item
+  // bounds checks and with the piece size resolved once per block.
+  const bool full = total1 == (uint32_t)N1 * NT && total2 == (uint32_t)N2 * NT &&
+                    (piece >= MV || piece == 8 || piece == 4);
 
   // Block coordinates, base pointers and whether the whole block lies inside
   // the matrix and the tile grid ("interior").
@@ -572,20 +688,34 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
     return b;
   };
 
-  // The global loads of an interior block are issued one block ahead, before
-  // the barrier and the store phase of the current block, so that a workgroup
-  // keeps loads and stores in flight together. Edge blocks load in place.
-  MatVec pre1[UNPACK ? 1 : N1];
-  TileVec pre2[UNPACK ? N2 : 1];
-  auto prefetch = [&](const Block& b) {
+  // The global loads of an interior block are issued DEPTH (1 or 2) blocks
+  // ahead, into one of DEPTH register sets (with two: the parity of the
+  // block's turn), right after the set's previous contents have gone to LDS,
+  // so that a workgroup keeps DEPTH blocks of loads and a block of stores in
+  // flight. Edge blocks load in place.
+  static_assert(DEPTH == 1 || DEPTH == 2, "one or two register sets");
+  MatVec pre1[DEPTH][UNPACK ? 1 : N1];
+  TileVec pre2[DEPTH][UNPACK ? N2 : 1];
+  auto prefetch = [&](const Block& b, auto slot_c) {
+    constexpr int S = decltype(slot_c)::value % DEPTH;
+    if (full) {
+      if constexpr (!UNPACK) {
+#pragma unroll
+        for (int i = 0; i < N1; ++i) pre1[S][i] = gload<MV>(b.mat_c + g1off[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < N2; ++i) pre2[S][i] = gload<VEC>(b.tiled_c + g2off[i]);
+      }
+      return;
+    }
     if constexpr (!UNPACK) {
 #pragma unroll
       for (int i = 0; i < N1; ++i)
-        if (tid + i * kThreads < total1) pre1[i] = gload<MV>(b.mat_c + g1off[i]);
+        if (tid + i * NT < total1) pre1[S][i] = gload<MV>(b.mat_c + g1off[i]);
     } else {
 #pragma unroll
       for (int i = 0; i < N2; ++i)
-        if (tid + i * kThreads < total2) pre2[i] = gload<VEC>(b.tiled_c + g2off[i]);
+        if (tid + i * NT < total2) pre2[S][i] = gload<VEC>(b.tiled_c + g2off[i]);
     }
   };
 
@@ -596,27 +726,33 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
   // both halves of such a line at about the same time.
   const uint32_t first_blk = (gridDim.x & 7) ? blockIdx.x
                                              : (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  uint32_t buf = 0;
-  bool have_pre = false;
-  for (uint32_t blk = first_blk; blk < nblocks; blk += gridDim.x) {
+  bool have_pre[2] = {false, false};
+  auto process = [&](uint32_t blk, auto slot_c) {
+    constexpr int L = decltype(slot_c)::value;  // LDS buffer: parity of the turn
+    constexpr int S = L % DEPTH;                // register set
     const Block b = block_at(blk);
     const uint32_t blk0 = b.blk0, blk1 = b.blk1, row_base = b.row_base,
                    col_base_bytes = b.col_base_bytes;
     const char* mat_c = b.mat_c;
     const char* tiled_c = b.tiled_c;
     const bool interior = b.interior;
-    char* lbuf = lds + buf * a.lds_buf_bytes;
-    buf ^= 1;
-    if (interior && !have_pre) prefetch(b);
+    char* lbuf = lds + L * a.lds_buf_bytes;
+    if (interior && !have_pre[S]) prefetch(b, slot_c);
 
     if constexpr (!UNPACK) {
       // ---- pack phase 1: 2-D rows -> LDS ----
-      if (interior) {
+      if (interior && full) {
+        with_static_piece<MV>(piece, [&](auto pc) {
+          constexpr int P = decltype(pc)::value;
+#pragma unroll
+          for (int i = 0; i < N1; ++i) lds_store_static<MV, P>(lbuf + l1off[i], pre1[S][i]);
+        });
+      } else if (interior) {
 #pragma unroll
         for (int i = 0; i < N1; ++i)
-          if (tid + i * kThreads < total1) lds_store_pieces<MV>(lbuf + l1off[i], pre1[i], piece);
+          if (tid + i * NT < total1) lds_store_pieces<MV>(lbuf + l1off[i], pre1[S][i], piece);
       } else {
-        for (uint32_t idx = tid; idx < total1; idx += kThreads) {
+        for (uint32_t idx = tid; idx < total1; idx += NT) {
           uint32_t r, cb;
           mat_item<MV>(a, idx, &r, &cb);
           __attribute__((aligned(16))) char reg[MV];
@@ -653,39 +789,37 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
       }
     } else {
       // ---- unpack phase 1: tiled runs -> LDS (scatter by granules) ----
+      if (interior && full) {
+#pragma unroll
+        for (int i = 0; i < N2; ++i) scatter_granules<VEC, G>(lbuf, l2off[i], pre2[S][i], rot);
+      } else {
       bool ok[N2];
 #pragma unroll
       for (int i = 0; i < N2; ++i) {
-        ok[i] = tid + i * kThreads < total2;
+        ok[i] = tid + i * NT < total2;
         if (!interior) {
           if (ok[i]) {
             uint32_t run, t, in_tile, tl0, tl1;
-            tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+            tiled_item<VEC>(a, tid + i * NT, &run, &t, &in_tile, &tl0, &tl1);
             ok[i] = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
           }
-          if (ok[i]) pre2[i] = gload<VEC>(tiled_c + g2off[i]);
+          if (ok[i]) pre2[S][i] = gload<VEC>(tiled_c + g2off[i]);
         }
       }
 #pragma unroll
       for (int i = 0; i < N2; ++i) {
-        if (ok[i]) {
-          __attribute__((aligned(16))) char tmp[VEC];
-          *reinterpret_cast<TileVec*>(tmp) = pre2[i];
-#pragma unroll
-          for (int k = 0; k < NG; ++k)
-            *reinterpret_cast<Gran*>(lbuf + l2off[i][k]) =
-                *reinterpret_cast<const Gran*>(tmp + k * G);
-        }
+        if (ok[i]) scatter_granules<VEC, G>(lbuf, l2off[i], pre2[S][i], rot);
+      }
       }
     }
 
-    // Next block's loads (interior blocks only).
-    have_pre = false;
-    if (blk + gridDim.x < nblocks) {
-      const Block nb = block_at(blk + gridDim.x);
+    // This register set's next block, DEPTH turns on (interior blocks only).
+    have_pre[S] = false;
+    if (blk + DEPTH * gridDim.x < nblocks) {
+      const Block nb = block_at(blk + DEPTH * gridDim.x);
       if (nb.interior) {
-        prefetch(nb);
-        have_pre = true;
+        prefetch(nb, slot_c);
+        have_pre[S] = true;
       }
     }
     __syncthreads();
@@ -693,24 +827,24 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
     if constexpr (!UNPACK) {
       // ---- pack phase 2: LDS -> tiled runs ----
       TileVec reg[N2];
+      if (interior && full) {
 #pragma unroll
-      for (int i = 0; i < N2; ++i) {
-        if (tid + i * kThreads < total2) {
-          __attribute__((aligned(16))) char tmp[VEC];
+        for (int i = 0; i < N2; ++i) reg[i] = gather_granules<VEC, G>(lbuf, l2off[i], rot);
 #pragma unroll
-          for (int k = 0; k < NG; ++k)
-            *reinterpret_cast<Gran*>(tmp + k * G) =
-                *reinterpret_cast<const Gran*>(lbuf + l2off[i][k]);
-          reg[i] = *reinterpret_cast<const TileVec*>(tmp);
-        }
+        for (int i = 0; i < N2; ++i) gstore<VEC>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
+        return;
       }
 #pragma unroll
       for (int i = 0; i < N2; ++i) {
-        if (tid + i * kThreads < total2) {
+        if (tid + i * NT < total2) reg[i] = gather_granules<VEC, G>(lbuf, l2off[i], rot);
+      }
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        if (tid + i * NT < total2) {
           bool ok = true;
           if (!interior) {
             uint32_t run, t, in_tile, tl0, tl1;
-            tiled_item<VEC>(a, tid + i * kThreads, &run, &t, &in_tile, &tl0, &tl1);
+            tiled_item<VEC>(a, tid + i * NT, &run, &t, &in_tile, &tl0, &tl1);
             ok = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
           }
           if (ok) gstore<VEC>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
@@ -718,17 +852,26 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
       }
     } else {
       // ---- unpack phase 2: LDS rows -> 2-D rows ----
-      if (interior) {
+      if (interior && full) {
+        MatVec reg[N1];
+        with_static_piece<MV>(piece, [&](auto pc) {
+          constexpr int P = decltype(pc)::value;
+#pragma unroll
+          for (int i = 0; i < N1; ++i) reg[i] = lds_load_static<MV, P>(lbuf + l1off[i]);
+        });
+#pragma unroll
+        for (int i = 0; i < N1; ++i) gstore<MV>(const_cast<char*>(mat_c) + g1off[i], reg[i]);
+      } else if (interior) {
         MatVec reg[N1];
 #pragma unroll
         for (int i = 0; i < N1; ++i)
-          if (tid + i * kThreads < total1) reg[i] = lds_load_pieces<MV>(lbuf + l1off[i], piece);
+          if (tid + i * NT < total1) reg[i] = lds_load_pieces<MV>(lbuf + l1off[i], piece);
 #pragma unroll
         for (int i = 0; i < N1; ++i)
-          if (tid + i * kThreads < total1) gstore<MV>(const_cast<char*>(mat_c) + g1off[i], reg[i]);
+          if (tid + i * NT < total1) gstore<MV>(const_cast<char*>(mat_c) + g1off[i], reg[i]);
       } else {
         const uint32_t es = a.elem_bytes;
-        for (uint32_t idx = tid; idx < total1; idx += kThreads) {
+        for (uint32_t idx = tid; idx < total1; idx += NT) {
           uint32_t r, cb;
           mat_item<MV>(a, idx, &r, &cb);
           if (row_base + r >= a.mat_size0) continue;
@@ -749,6 +892,25 @@ __global__ __launch_bounds__(kThreads) void stream_tiled_kernel(TiledArgs a) {
     }
     // No second barrier: the next block uses the other LDS buffer, and its
     // barrier orders this block's LDS reads before the buffer is reused.
+  };
+  // Start the pipeline: the first two blocks of this workgroup.
+  if (first_blk < nblocks) {
+    const Block b0 = block_at(first_blk);
+    if (b0.interior) {
+      prefetch(b0, std::integral_constant<int, 0>{});
+      have_pre[0] = true;
+    }
+    if (DEPTH == 2 && first_blk + gridDim.x < nblocks) {
+      const Block b1 = block_at(first_blk + gridDim.x);
+      if (b1.interior) {
+        prefetch(b1, std::integral_constant<int, 1>{});
+        have_pre[1] = true;
+      }
+    }
+  }
+  for (uint32_t blk = first_blk; blk < nblocks; blk += 2 * gridDim.x) {
+    process(blk, std::integral_constant<int, 0>{});
+    if (blk + gridDim.x < nblocks) process(blk + gridDim.x, std::integral_constant<int, 1>{});
   }
 }
 
@@ -958,12 +1120,13 @@ bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
   if (plan.big) {
     // One workgroup per CU: two 66 KB buffers fill its LDS.
     if (!(plan.G == 4 && plan.VEC == 16 && plan.MV == 16)) return false;
-    auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes>;
+    constexpr int kBigThreads = 1024;
+    auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes, kBigThreads, 1>;
     static hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
         160 * 1024);
     if (attr != hipSuccess || lds > 160 * 1024) return false;
-    uk::launch(UNPACK ? 1 : 0, kernel, dim3(nblocks < 256 ? nblocks : 256), dim3(kThreads), lds,
+    uk::launch(UNPACK ? 1 : 0, kernel, dim3(nblocks < 256 ? nblocks : 256), dim3(kBigThreads), lds,
                stream, plan.args);
     return true;
   }
