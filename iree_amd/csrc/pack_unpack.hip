@@ -692,12 +692,41 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
   // ahead, into one of DEPTH register sets (with two: the parity of the
   // block's turn), right after the set's previous contents have gone to LDS,
   // so that a workgroup keeps DEPTH blocks of loads and a block of stores in
-  // flight. Edge blocks load in place.
+  // flight.
   static_assert(DEPTH == 1 || DEPTH == 2, "one or two register sets");
   MatVec pre1[DEPTH][UNPACK ? 1 : N1];
   TileVec pre2[DEPTH][UNPACK ? N2 : 1];
   auto prefetch = [&](const Block& b, auto slot_c) {
     constexpr int S = decltype(slot_c)::value % DEPTH;
+    if (!b.interior) {
+      // Edge block: only what exists is loaded (2-D side: vectors that lie
+      // wholly inside the matrix; tiled side: vectors of tiles that exist);
+      // phase 1 applies the same predicate before it uses a register.
+      if constexpr (!UNPACK) {
+#pragma unroll
+        for (int i = 0; i < N1; ++i) {
+          const uint32_t idx = tid + i * NT;
+          if (idx < total1) {
+            uint32_t r, cb;
+            mat_item<MV>(a, idx, &r, &cb);
+            if (b.row_base + r < a.mat_size0 && b.col_base_bytes + cb + MV <= size1_bytes)
+              pre1[S][i] = gload<MV>(b.mat_c + g1off[i]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < N2; ++i) {
+          const uint32_t idx = tid + i * NT;
+          if (idx < total2) {
+            uint32_t run, t, in_tile, tl0, tl1;
+            tiled_item<VEC>(a, idx, &run, &t, &in_tile, &tl0, &tl1);
+            if (b.blk0 * a.G0 + tl0 < a.outer0 && b.blk1 * a.G1 + tl1 < a.outer1)
+              pre2[S][i] = gload<VEC>(b.tiled_c + g2off[i]);
+          }
+        }
+      }
+      return;
+    }
     if (full) {
       if constexpr (!UNPACK) {
 #pragma unroll
@@ -737,7 +766,7 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
     const char* tiled_c = b.tiled_c;
     const bool interior = b.interior;
     char* lbuf = lds + L * a.lds_buf_bytes;
-    if (interior && !have_pre[S]) prefetch(b, slot_c);
+    if (!have_pre[S]) prefetch(b, slot_c);
 
     if constexpr (!UNPACK) {
       // ---- pack phase 1: 2-D rows -> LDS ----
@@ -752,16 +781,20 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
         for (int i = 0; i < N1; ++i)
           if (tid + i * NT < total1) lds_store_pieces<MV>(lbuf + l1off[i], pre1[S][i], piece);
       } else {
-        for (uint32_t idx = tid; idx < total1; idx += NT) {
+#pragma unroll
+        for (int i = 0; i < N1; ++i) {
+          const uint32_t idx = tid + i * NT;
+          if (idx >= total1) continue;
           uint32_t r, cb;
           mat_item<MV>(a, idx, &r, &cb);
           __attribute__((aligned(16))) char reg[MV];
           const bool row_ok = row_base + r < a.mat_size0;
           const char* gp = mat_c + (r * a.mat_stride0_bytes32 + cb);
           const uint32_t es = a.elem_bytes;
-          // Whole vector inside the matrix, or whole vector padding: one access.
+          // Whole vector inside the matrix (already loaded), or whole vector
+          // padding: one access.
           if (row_ok && col_base_bytes + cb + MV <= size1_bytes) {
-            lds_store_pieces<MV>(lbuf + r * a.lds_pitch + cb, gload<MV>(gp), piece);
+            lds_store_pieces<MV>(lbuf + l1off[i], pre1[S][i], piece);
             continue;
           }
           if (!row_ok || col_base_bytes + cb >= size1_bytes) {
@@ -803,7 +836,6 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
             tiled_item<VEC>(a, tid + i * NT, &run, &t, &in_tile, &tl0, &tl1);
             ok[i] = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
           }
-          if (ok[i]) pre2[S][i] = gload<VEC>(tiled_c + g2off[i]);
         }
       }
 #pragma unroll
@@ -813,14 +845,11 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
       }
     }
 
-    // This register set's next block, DEPTH turns on (interior blocks only).
+    // This register set's next block, DEPTH turns on.
     have_pre[S] = false;
     if (blk + DEPTH * gridDim.x < nblocks) {
-      const Block nb = block_at(blk + DEPTH * gridDim.x);
-      if (nb.interior) {
-        prefetch(nb, slot_c);
-        have_pre[S] = true;
-      }
+      prefetch(block_at(blk + DEPTH * gridDim.x), slot_c);
+      have_pre[S] = true;
     }
     __syncthreads();
 
@@ -895,17 +924,11 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
   };
   // Start the pipeline: the first two blocks of this workgroup.
   if (first_blk < nblocks) {
-    const Block b0 = block_at(first_blk);
-    if (b0.interior) {
-      prefetch(b0, std::integral_constant<int, 0>{});
-      have_pre[0] = true;
-    }
+    prefetch(block_at(first_blk), std::integral_constant<int, 0>{});
+    have_pre[0] = true;
     if (DEPTH == 2 && first_blk + gridDim.x < nblocks) {
-      const Block b1 = block_at(first_blk + gridDim.x);
-      if (b1.interior) {
-        prefetch(b1, std::integral_constant<int, 1>{});
-        have_pre[1] = true;
-      }
+      prefetch(block_at(first_blk + gridDim.x), std::integral_constant<int, 1>{});
+      have_pre[1] = true;
     }
   }
   for (uint32_t blk = first_blk; blk < nblocks; blk += 2 * gridDim.x) {
