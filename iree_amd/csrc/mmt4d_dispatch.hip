@@ -23,8 +23,11 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
                                             const iree_uk_amd_rowmajor_out_t* rowmajor,
                                             void* stream, int kernel_mode,
                                             const char** kernel_name) {
+  // s8 x s4 -> s32 has an MFMA kernel for some shapes only; the launcher says
+  // "not served" (negative) for the rest.
+  const bool maybe = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32;
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC &&
-      iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) {
+      (maybe || iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags))) {
     const int forced = kernel_mode >= IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
                            ? kernel_mode - IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
                            : 0;

@@ -13,6 +13,7 @@ int launch_f8(const Problem& p, int forced, hipStream_t stream, const char** nam
 int launch_f32(const Problem& p, int forced, hipStream_t stream, const char** name);
 int launch_f16f16(const Problem& p, int forced, hipStream_t stream, const char** name);
 int launch_bf16bf16(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_s8s4(const Problem& p, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 
 namespace {
@@ -73,16 +74,30 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
                                                  const char** kernel_name) {
   Elem e;
   int eb, ob;
-  if (!elem_of(p->flags, &e, &eb, &ob)) return -1;
-  if (!iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) return -1;
+  // s8 x s4 -> s32 has a kernel for some shapes only (K0 a power of two in
+  // [16, 64], K in whole 64-element steps): it does not count as "supported"
+  // for iree_uk_mmt4d_info, but is tried before the generic kernel.
+  const bool s8s4 = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32;
+  if (s8s4) {
+    e = Elem::kS8S4;
+    eb = 1;
+    ob = 4;
+    if (p->K0 != 16 && p->K0 != 32 && p->K0 != 64) return -1;
+    if (p->M0 < 1 || p->N0 < 1 || p->M0 > 64 || p->N0 > 64) return -1;
+    if (forced_variant != 0 && forced_variant != 4) return -1;
+  } else {
+    if (!elem_of(p->flags, &e, &eb, &ob)) return -1;
+    if (!iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) return -1;
+  }
   if (p->K == 0) return -1;  // zero fill only: the generic kernel does it
   hipStream_t stream = (hipStream_t)stream_v;
   uk_mfma::Problem pr;
   pr.lhs = (const char*)p->lhs_buffer + p->lhs_offset * eb;
-  pr.rhs = (const char*)p->rhs_buffer + p->rhs_offset * eb;
+  // 4-bit elements: offsets and strides land on byte boundaries (validated).
+  pr.rhs = (const char*)p->rhs_buffer + (s8s4 ? p->rhs_offset / 2 : p->rhs_offset * eb);
   pr.out = (char*)p->out_buffer + p->out_offset * ob;
   pr.lhs_stride = p->lhs_stride0 * eb;
-  pr.rhs_stride = p->rhs_stride0 * eb;
+  pr.rhs_stride = s8s4 ? p->rhs_stride0 / 2 : p->rhs_stride0 * eb;
   if (rowmajor) {
     // Row m of panel pl is matrix row pl * M0 + m; column panels follow each
     // other inside a row.
@@ -117,11 +132,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
       if ((uintptr_t)pr.acc & 3) return -1;
     }
   }
-  // 16-byte vector loads need 16-byte aligned panels.
-  if (((uintptr_t)pr.lhs | (uintptr_t)pr.rhs | (uint64_t)pr.lhs_stride |
-       (uint64_t)pr.rhs_stride) & 15) {
-    return -1;
-  }
+  // 16-byte vector loads need 16-byte aligned panels (8-byte loads of 4-bit
+  // rows: 8-byte aligned).
+  if (((uintptr_t)pr.lhs | (uint64_t)pr.lhs_stride) & 15) return -1;
+  if (((uintptr_t)pr.rhs | (uint64_t)pr.rhs_stride) & (s8s4 ? 7 : 15)) return -1;
   if ((uintptr_t)pr.out & (uintptr_t)(ob - 1)) return -1;
   pr.M1 = (int32_t)p->M;
   pr.N1 = (int32_t)p->N;
@@ -133,6 +147,7 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
   while ((1 << pr.lrb) < pr.rb) ++pr.lrb;
   pr.accumulate = (p->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   switch (e) {
+    case Elem::kS8S4: return uk_mfma::launch_s8s4(pr, stream, kernel_name);
     case Elem::kS8: return uk_mfma::launch_s8(pr, forced_variant, stream, kernel_name);
     case Elem::kF16: return uk_mfma::launch_f16(pr, forced_variant, stream, kernel_name);
     case Elem::kBF16: return uk_mfma::launch_bf16(pr, forced_variant, stream, kernel_name);

@@ -61,7 +61,10 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 // kF16F16 / kBF16BF16: 16-bit float output, accumulated in f32 over all of K
 // and rounded once at the end (IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS,
 // runtime/src/iree/builtins/ukernel/mmt4d_tile_generic.c:258-286,348-376).
-enum class Elem { kS8, kF16, kBF16, kF8, kF32, kF16F16, kBF16BF16 };
+// kS8S4: s8 x s4 -> s32 (two 4-bit RHS values per byte, low nibble first,
+// runtime/src/iree/builtins/ukernel/mmt4d_tile_generic.c:11-51); served by
+// the thin kernel only (mmt4d_mfma_thin.h).
+enum class Elem { kS8, kF16, kBF16, kF8, kF32, kF16F16, kBF16BF16, kS8S4 };
 
 typedef uint16_t v4u16 __attribute__((ext_vector_type(4)));
 
@@ -108,6 +111,7 @@ template <> struct ElemTraits<Elem::kS8> {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b[0], c, 0, 0, 0);
   }
 };
+template <> struct ElemTraits<Elem::kS8S4> : ElemTraits<Elem::kS8> {};
 template <> struct ElemTraits<Elem::kF16> {
   using Acc = v4f;
   using Out = Out32<v4f, float>;

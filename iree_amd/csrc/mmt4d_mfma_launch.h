@@ -151,9 +151,13 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream) {
   }
   constexpr int KS = 64 * ElemTraits<E>::kHalves;
   constexpr int OB = OBYTES;
-  if (p.rb > KS || p.rb < 8) return -1;
+  constexpr bool S4 = E == Elem::kS8S4;  // rb, lrb describe the LHS; RHS rows are half as wide
+  if (p.rb > KS || p.rb < (S4 ? 16 : 8)) return -1;
   const int64_t k_bytes = (int64_t)p.K1 << p.lrb;
   if (k_bytes == 0 || k_bytes % KS) return -1;
+  // 4-bit RHS: the accumulators hold 16 * sum; |sum| <= K * 128 * 8 must stay
+  // below 2^27 for that to be exact.
+  if (S4 && k_bytes >= 131072) return -1;
   if (p.out_rows <= 0 || p.out_cols <= 0) return 0;
   Args a{};
   a.lhs = p.lhs; a.rhs = p.rhs; a.out = p.out;
@@ -190,7 +194,8 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream) {
               (!p.accumulate || vector_ok(p.acc, p.acc_stride, p.acc_sm0, p.acc_spn));
   // 32-bit operand offsets inside a workgroup's panels.
   const int64_t span_m = (int64_t)(TM * 16 / p.M0 + 2) * p.lhs_stride + k_bytes * p.M0;
-  const int64_t span_n = (int64_t)(TN * 16 / p.N0 + 2) * p.rhs_stride + k_bytes * p.N0;
+  const int64_t span_n =
+      (int64_t)(TN * 16 / p.N0 + 2) * p.rhs_stride + k_bytes * p.N0 / (S4 ? 2 : 1);
   if (span_m >= (1ll << 31) || span_n >= (1ll << 31)) return -1;
   uk::launch(2, mmt4d_thin_kernel<E, RBC, TM, TN, KSPLIT, D>, dim3((uint32_t)(grid_m * grid_n)),
              dim3(KSPLIT * 64), 0, stream, a);

@@ -21,6 +21,16 @@
 // bytes and more load one 16-byte piece per operand; 8-byte rows load the two
 // 8-byte halves from two K-tiles (chunk g of a step holds K-tiles g and
 // g + 4). K must be a whole number of steps.
+//
+// s8 x s4 -> s32 (Elem::kS8S4) runs here too. A lane loads 8 RHS bytes (16
+// nibbles, the same 16 K elements as its 16 LHS bytes) and turns them into two
+// groups of eight signed bytes without unpacking to true values: (x << 4) &
+// 0xF0F0F0F0 holds 16 * (low nibble as s4) in every byte and x & 0xF0F0F0F0
+// holds 16 * (high nibble as s4), i.e. the even and the odd K elements; the
+// LHS bytes are split into even and odd positions to match (v_perm_b32). The
+// MFMA then accumulates 16 times the true sum, exactly (the launcher bounds K
+// so that this cannot wrap), and the store path shifts it back before it adds
+// the ACCUMULATE input.
 #ifndef IREE_UK_AMD_MMT4D_MFMA_THIN_H_
 #define IREE_UK_AMD_MMT4D_MFMA_THIN_H_
 
@@ -41,7 +51,9 @@ void mmt4d_thin_kernel(Args a) {
   constexpr int NCH = 4 * HALVES;             // 16-byte chunks per row per step
   constexpr int KS = NCH * 16;                // bytes of K per row per step
   constexpr int PIECES = RBC >= 16 ? 1 : 2;   // loads per 16-byte operand
+  constexpr bool S4 = E == Elem::kS8S4;       // 4-bit RHS: half the bytes per row
   static_assert(RBC >= 8, "rows narrower than 8 bytes take the LDS kernels");
+  static_assert(!S4 || RBC >= 16, "4-bit RHS: LHS rows of at least 16 bytes");
 
   __shared__ v4i partial[KSPLIT > 1 ? KSPLIT - 1 : 1][TM * TN][64];
 
@@ -51,7 +63,8 @@ void mmt4d_thin_kernel(Args a) {
   const int bm = (int)(blockIdx.x / (uint32_t)a.grid_n);
   const int bn = (int)(blockIdx.x - (uint32_t)bm * a.grid_n);
   const int lrb = a.lrb;
-  const uint32_t kt_m = (uint32_t)a.M0 << lrb, kt_n = (uint32_t)a.N0 << lrb;
+  const int lrb_b = S4 ? lrb - 1 : lrb;       // log2 of the RHS row bytes
+  const uint32_t kt_m = (uint32_t)a.M0 << lrb, kt_n = (uint32_t)a.N0 << lrb_b;
   const uint32_t kts_per_step = KS >> lrb;
   const uint32_t sstep_a = kts_per_step * kt_m, sstep_b = kts_per_step * kt_n;
 
@@ -63,7 +76,7 @@ void mmt4d_thin_kernel(Args a) {
   const char* base_a = a.lhs + (int64_t)pa0 * a.lhs_stride;
   const char* base_b = a.rhs + (int64_t)pb0 * a.rhs_stride;
   auto operand_offsets = [&](uint32_t (&off)[HALVES][PIECES], int x, int X0, int X1, int p0,
-                             int64_t stride, uint32_t kt_bytes) {
+                             int64_t stride, uint32_t kt_bytes, int lrb, uint32_t piece_bytes) {
     const uint32_t row = (uint32_t)x * 16 + r;
     const uint32_t pabs = row / (uint32_t)X0;
     const uint32_t x0 = row - pabs * X0;
@@ -76,7 +89,7 @@ void mmt4d_thin_kernel(Args a) {
       for (int t = 0; t < PIECES; ++t) {
         uint32_t o;
         if constexpr (RBC >= 16) {
-          const uint32_t kb = g * 16;
+          const uint32_t kb = g * piece_bytes;
           o = (kb >> lrb) * kt_bytes + (x0 << lrb) + (kb & ((1u << lrb) - 1));
         } else {
           o = (g + (uint32_t)t * NCH) * kt_bytes + x0 * 8;
@@ -88,10 +101,11 @@ void mmt4d_thin_kernel(Args a) {
   uint32_t offa[TM][HALVES][PIECES], offb[TN][HALVES][PIECES];
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm)
-    operand_offsets(offa[tm], bm * TM + tm, a.M0, a.M1, pa0, a.lhs_stride, kt_m);
+    operand_offsets(offa[tm], bm * TM + tm, a.M0, a.M1, pa0, a.lhs_stride, kt_m, lrb, 16);
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn)
-    operand_offsets(offb[tn], bn * TN + tn, a.N0, a.N1, pb0, a.rhs_stride, kt_n);
+    operand_offsets(offb[tn], bn * TN + tn, a.N0, a.N1, pb0, a.rhs_stride, kt_n, lrb_b,
+                    S4 ? 8 : 16);
 
   auto load_operand = [&](const char* base, const uint32_t (&off)[PIECES], uint32_t adv) {
     if constexpr (RBC >= 16) {
@@ -102,14 +116,22 @@ void mmt4d_thin_kernel(Args a) {
       return v4i{lo[0], lo[1], hi[0], hi[1]};
     }
   };
-  v4i fa[D][TM][HALVES], fb[D][TN][HALVES];
+  using BFrag = typename std::conditional<S4, v2i, v4i>::type;
+  v4i fa[D][TM][HALVES];
+  BFrag fb[D][TN][HALVES];
   // Local step i of this wave is K step wave + i * KSPLIT.
   auto load_step = [&](int d, int i) {
     const uint32_t s = (uint32_t)(wave + i * KSPLIT);
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-      for (int h = 0; h < HALVES; ++h) fb[d][tn][h] = load_operand(base_b, offb[tn][h], s * sstep_b);
+      for (int h = 0; h < HALVES; ++h) {
+        if constexpr (S4) {
+          fb[d][tn][h] = *reinterpret_cast<const v2i*>(base_b + (offb[tn][h][0] + s * sstep_b));
+        } else {
+          fb[d][tn][h] = load_operand(base_b, offb[tn][h], s * sstep_b);
+        }
+      }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
@@ -173,11 +195,26 @@ void mmt4d_thin_kernel(Args a) {
   for (int tm = 0; tm < TM; ++tm) sm[tm] = 1.0f;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) sn[tn] = v4f{1.0f, 1.0f, 1.0f, 1.0f};
+  // With the 4-bit RHS the accumulators hold 16 times the sum, so the
+  // ACCUMULATE input waits in registers of its own.
+  Acc cin[S4 ? TM : 1][S4 ? TN : 1];
+  if constexpr (S4) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) cin[tm][tn] = Acc{0, 0, 0, 0};
+  }
   if (wave == 0) {
     if (a.accumulate) {
       for_each_output(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn, a.acc_sn0,
-                      [&](int tm, int tn, char* p) { acc[tm][tn] = Out::load4(p); },
-                      [&](int tm, int tn, int e, char* p) { acc[tm][tn][e] = Out::load1(p); });
+                      [&](int tm, int tn, char* p) {
+                        if constexpr (S4) cin[tm][tn] = Out::load4(p);
+                        else acc[tm][tn] = Out::load4(p);
+                      },
+                      [&](int tm, int tn, int e, char* p) {
+                        if constexpr (S4) cin[tm][tn][e] = Out::load1(p);
+                        else acc[tm][tn][e] = Out::load1(p);
+                      });
     }
     if (OB == 4 && a.dequant) {
       if (a.row_scale) {
@@ -196,10 +233,33 @@ void mmt4d_thin_kernel(Args a) {
     }
   }
   auto compute = [&](int d) {
+    if constexpr (S4) {
+      // LHS: even K bytes, then odd K bytes; RHS: low nibbles, then high ones.
+      v4i ea[TM], eb[TN];
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
+      for (int tm = 0; tm < TM; ++tm) {
+        const v4i x = fa[d][tm][0];
+        ea[tm] = v4i{(int)__builtin_amdgcn_perm((uint32_t)x[1], (uint32_t)x[0], 0x06040200u),
+                     (int)__builtin_amdgcn_perm((uint32_t)x[3], (uint32_t)x[2], 0x06040200u),
+                     (int)__builtin_amdgcn_perm((uint32_t)x[1], (uint32_t)x[0], 0x07050301u),
+                     (int)__builtin_amdgcn_perm((uint32_t)x[3], (uint32_t)x[2], 0x07050301u)};
+      }
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fb[d][tn], fa[d][tm], acc[tm][tn]);
+      for (int tn = 0; tn < TN; ++tn) {
+        const uint32_t x0 = (uint32_t)fb[d][tn][0][0], x1 = (uint32_t)fb[d][tn][0][1];
+        eb[tn] = v4i{(int)((x0 << 4) & 0xF0F0F0F0u), (int)((x1 << 4) & 0xF0F0F0F0u),
+                     (int)(x0 & 0xF0F0F0F0u), (int)(x1 & 0xF0F0F0F0u)};
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(&eb[tn], &ea[tm], acc[tm][tn]);
+    } else {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fb[d][tn], fa[d][tm], acc[tm][tn]);
+    }
   };
   int i = 0;
   // Steady state: every step computed is followed by the load of the step D
@@ -241,6 +301,13 @@ void mmt4d_thin_kernel(Args a) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
           acc[tm][tn] += __builtin_bit_cast(Acc, partial[w][tm * TN + tn][lane]);
+  }
+
+  if constexpr (S4) {
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = (acc[tm][tn] >> 4) + cin[tm][tn];
   }
 
   // ---- store --------------------------------------------------------------------
