@@ -430,11 +430,14 @@ __global__ __launch_bounds__(kThreads) void unpack_tiled_kernel(TiledArgs a) {
 //   * a workgroup walks many blocks; everything that depends only on the
 //     thread and the block shape (global offsets inside a block, LDS offsets
 //     of every granule) is computed once, before the walk;
-//   * all loads of a phase are issued before any of their data is used;
+//   * all loads of a phase are issued before any of their data is used, one
+//     or two blocks ahead of their use;
 //   * LDS is double-buffered, one barrier per block, so the stores of block b
-//     and the loads of block b+1 are in flight together;
-//   * global accesses are non-temporal (every byte is touched once).
-// Blocks on the ragged edge of the matrix take a slower, bounds-checked path.
+//     and the loads of the following blocks are in flight together;
+//   * interior blocks in which every thread has all of its items run without
+//     per-item bounds checks.
+// Blocks on the ragged edge of the matrix take a slower, bounds-checked path
+// (their loads are issued ahead all the same, predicated).
 //===----------------------------------------------------------------------===//
 
 typedef uint32_t v2u __attribute__((ext_vector_type(2)));
@@ -611,7 +614,6 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
   constexpr int NG = VEC / G;                             // granules per tiled vector
   using MatVec = typename GBytes<MV>::type;
   using TileVec = typename GBytes<VEC>::type;
-  using Gran = typename GBytes<G < 4 ? 4 : G>::type;  // G >= 4 here (see planner)
   static_assert(G >= 4, "streaming kernels move granules of at least 4 bytes");
 
   const uint32_t tid = threadIdx.x;
