@@ -202,3 +202,31 @@ def test_dequant_unpack_contract(lib):
         call(uk.MMT4D_TYPE_S8S8S32, rows=0, M=0)
     finally:
         lib.raise_on_violation(False)
+
+
+@pytest.mark.gpu
+def test_decode_without_pack_row_major_activations_are_m0_1_tiles(gpu):
+    """A row-major [M, K] activation matrix is the mmt4d LHS layout with
+    M0 = 1, so a decode step needs neither pack nor unpack on the activation
+    side: mmt4d_dequant_unpack on M0 = 1 tiles against the exact product."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    M, N, K, N0, K0 = 16, 2048, 4096, 16, 16
+    g = torch.Generator(device="cuda"); g.manual_seed(9)
+    act = torch.randint(-128, 128, (M, K), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8)
+    rs = torch.rand(M, generator=g, device="cuda") * 0.02 + 0.001
+    cs = torch.rand(N, generator=g, device="cuda") * 0.02 + 0.001
+    N1, K1 = N // N0, K // K0
+    rhs4 = torch.empty(N1 * K1 * N0 * K0, device="cuda", dtype=torch.int8)
+    lib.pack(w.data_ptr(), 0, K, 1, rhs4.data_ptr(), 0, K1 * N0 * K0, N0 * K0, N, K, N1, K1, N0, K0, 0,
+             uk.PACK_TYPE_I8I8)                       # weights: packed once
+    y = torch.empty(M, N, device="cuda")
+    lib.mmt4d_dequant_unpack(act.data_ptr(), 0, K, rhs4.data_ptr(), 0, K1 * N0 * K0, None, 0, 0,
+                             y.data_ptr(), 0, N, M, N, rs.data_ptr(), cs.data_ptr(),
+                             M, N1, K1, 1, N0, K0, uk.MMT4D_TYPE_S8S8S32)
+    lib.synchronize()
+    assert lib.last_kernel_name() == "mmt4d_mfma_thin"
+    prod = (act.cpu().to(torch.int64) @ w.cpu().to(torch.int64).T).to(torch.int32)
+    want = (prod.float() * rs.cpu()[:, None]) * cs.cpu()[None, :]
+    assert torch.equal(y.cpu(), want)
