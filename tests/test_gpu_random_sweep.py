@@ -161,6 +161,58 @@ def test_mmt4d_random_sweep_larger_shapes_and_forced_variants(gpu, oracle):
     assert done >= 120, done
 
 
+def test_mmt4d_random_sweep_thin_kernels(gpu, oracle):
+    """The barrier-free kernels (M-thin, N-thin on the transposed problem, the
+    64x64 K split, the 4-bit RHS): K in whole 64- or 128-byte steps, few rows
+    or few columns or few blocks, random tiles incl. heights that straddle the
+    16-row MFMA blocks, loose strides, ACCUMULATE, each forced shape."""
+    lib, torch = gpu
+    rng = np.random.default_rng(2029)
+    types = [uk.MMT4D_TYPE_S8S8S32, uk.MMT4D_TYPE_F16F16F32, uk.MMT4D_TYPE_BF16BF16F32,
+             uk.MMT4D_TYPE_F32F32F32, uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, uk.MMT4D_TYPE_S8S4S32,
+             uk.MMT4D_TYPE_F16F16F16 | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS]
+    names = set()
+    done = 0
+    for ci in range(420):
+        tf = types[ci % len(types)]
+        s8s4 = (tf & 0xFF) == uk.MMT4D_TYPE_S8S4S32
+        bits = uk.MMT4D_TYPE_BITS[tf & 0xFF][0]
+        M0, N0 = int(rng.choice([1, 2, 5, 8, 12, 16, 24, 32, 64])), int(rng.choice([1, 4, 8, 16, 20, 32, 64]))
+        K0 = int(rng.choice([16, 32, 64] if s8s4 else [1, 2, 4, 8, 16, 32, 64]))
+        rb = K0 * bits // 8
+        if rb < 8 or rb > 128 or (not s8s4 and not lib.mmt4d_info(M0, N0, K0, tf)):
+            continue
+        step = 128 if (tf & 0xFF) == uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32 else 64
+        if rb > step:
+            continue
+        K = (step // rb) * int(rng.integers(1, 9))             # whole steps
+        shape_kind = ci % 3
+        if shape_kind == 0:      # few rows
+            M, N = max(1, int(rng.integers(1, 70)) // M0), int(rng.integers(1, 30))
+        elif shape_kind == 1:    # few columns
+            M, N = int(rng.integers(1, 30)), max(1, int(rng.integers(1, 70)) // N0)
+        else:                    # a few blocks each way
+            M, N = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+        acc = uk.MMT4D_ACCUMULATE if rng.integers(0, 2) else 0
+        c = T.Mmt4dCase(tf | acc, M, N, K, M0, N0, K0, K * M0 * K0 + 32, K * N0 * K0 + 32,
+                        N * M0 * N0 + 16, 32, 32, 16)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        variant = 0 if s8s4 else int(rng.choice([0, 4, 5, 6]))
+        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert np.array_equal(got, want), (ci, c, variant, lib.last_kernel_name())
+        assert lib.last_kernel_name().startswith("mmt4d_mfma"), (ci, c, variant, lib.last_kernel_name())
+        names.add(lib.last_kernel_name())
+        done += 1
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    assert done >= 150, done
+    for want_name in ("mmt4d_mfma_thin", "mmt4d_mfma_thin_transposed", "mmt4d_mfma_64x64_ksplit",
+                      "mmt4d_mfma_thin_s8s4"):
+        assert want_name in names, names
+
+
 def test_pack_unpack_random_round_trips_multi_block(gpu):
     """Sizes of several blocks per dimension: pack must equal numpy's
     pad + reshape + transpose and unpack must invert it, for random tiles,
