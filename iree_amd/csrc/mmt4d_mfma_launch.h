@@ -217,8 +217,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //   small 64x64, 4 waves, any K: for problems with too few 128x128 blocks to
 //         occupy the 256 CUs;
 // `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem,
-// 6 the 64x64 K-split kernel; 0 = choose) overrides the size heuristic for
-// tests and tuning.
+// 6 the 64x64 K-split kernel, 7 the 256x128 shape; 0 = choose) overrides the
+// size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
 //         streaming the RHS: the barrier-free kernel of mmt4d_mfma_thin.h (16,
 //         32 or 64 rows x 32 columns per workgroup, K split over its 4 waves)
@@ -235,7 +235,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced >= 1 && forced <= 6) {
+  if (forced >= 1 && forced <= 7) {
     choice = forced;
   } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
     choice = 4;
@@ -243,6 +243,10 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 5;
   } else if (workgroups(p, 256, 256) >= 192) {
     choice = 1;
+  } else if (RBC >= 16 && ElemTraits<E>::kHalves == 1 && workgroups(p, 256, 128) >= 192 &&
+             workgroups(p, 256, 128) <= 256) {
+    // One round of 256x128 blocks (measured 5-7 % ahead of 128x128 there).
+    choice = 7;
   } else if (workgroups(p, 128, 128) >= 192) {
     choice = 2;
   } else if (RBC >= 8 && ((int64_t)p.K1 << p.lrb) >= 8192) {
@@ -333,6 +337,23 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
       }
       if (st > 0) return st;
+    }
+    choice = 2;
+  }
+  if (choice == 7) {
+    // 256 rows x 128 columns, 8 waves of 128x32: for problems with too few
+    // 256x256 blocks to fill the CUs; moves fewer L1 bytes per MFMA than the
+    // 128x128 shape.
+    if constexpr (RBC >= 16 && ElemTraits<E>::kHalves == 1) {
+      if (kt_main > 0) {
+        int st = launch_variant<E, RBC, 8, 2, 2, 4, 1, 3>(p, 0, kt_main, p.accumulate, stream);
+        if (st == 0) {
+          *name = "mmt4d_mfma_256x128_rhs_direct";
+          if (kt_main == p.K1) return 0;
+          return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+        }
+        if (st > 0) return st;
+      }
     }
     choice = 2;
   }

@@ -86,8 +86,8 @@ def _mfma_shapes(M0, N0, K0, bits):
 # kernel when K is a whole number of 64-byte steps and rows are at least 8
 # bytes wide, else the 32x64 kernel through LDS: the shapes below have both;
 # 5 is the thin kernel on the transposed problem and 6 the same kernel with
-# 64x64 blocks, under the same conditions).
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+# 64x64 blocks, under the same conditions; 7 is the 256x128 shape).
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("n", range(len(MFMA_TILES)))
 def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu
