@@ -243,8 +243,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 5;
   } else if (workgroups(p, 256, 256) >= 192) {
     choice = 1;
-  } else if (RBC >= 16 && ElemTraits<E>::kHalves == 1 && workgroups(p, 256, 128) >= 192 &&
-             workgroups(p, 256, 128) <= 256) {
+  } else if (RBC >= 16 && workgroups(p, 256, 128) >= 192 && workgroups(p, 256, 128) <= 256) {
     // One round of 256x128 blocks (measured 5-7 % ahead of 128x128 there).
     choice = 7;
   } else if (workgroups(p, 128, 128) >= 192) {
@@ -344,7 +343,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     // 256 rows x 128 columns, 8 waves of 128x32: for problems with too few
     // 256x256 blocks to fill the CUs; moves fewer L1 bytes per MFMA than the
     // 128x128 shape.
-    if constexpr (RBC >= 16 && ElemTraits<E>::kHalves == 1) {
+    if constexpr (RBC >= 16) {
       if (kt_main > 0) {
         int st = launch_variant<E, RBC, 8, 2, 2, 4, 1, 3>(p, 0, kt_main, p.accumulate, stream);
         if (st == 0) {

@@ -229,6 +229,21 @@ class Runner:
                             op.flops, op.bytes, "bf16",
                             dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
                                  M0=M0, N0=N0, K0=K0))
+        if name.startswith("f8_mmt4d_"):
+            _, _, size, k0 = name.split("_")
+            S, K0 = int(size), int(k0[1:])
+            M0 = N0 = 16
+            M1 = N1 = S // 16
+            K1 = S // K0
+            lhs4 = self.normal_f8((M1 * K1 * M0 * K0,), 17)
+            rhs4 = self.normal_f8((N1 * K1 * N0 * K0,), 18)
+            out4 = self.empty(M1 * N1 * M0 * N0, torch.float32)
+            op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, "f8", 1)
+            return Workload(name, f"mmt4d f8E4M3FN->f32 {S}^3 tiles 16x16x{K0}", [op],
+                            op.flops, op.bytes, "f8",
+                            dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
+                                 M0=M0, N0=N0, K0=K0))
         if name.startswith("f32_mmt4d_"):
             _, _, size, k0 = name.split("_")
             S, K0 = int(size), int(k0[1:])
