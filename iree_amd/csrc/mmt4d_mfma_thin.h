@@ -3,9 +3,9 @@
 // bound by memory, so the kernel is built around keeping loads in flight:
 //
 //   * no LDS staging and no barrier in the K loop. A workgroup owns TM x TN
-//     output blocks of 16x16; its KSPLIT waves take the 64-byte K steps round
-//     robin (wave w: steps w, w + KSPLIT, ...), so together they read the
-//     workgroup's RHS panels front to back;
+//     output blocks of 16x16; its KSPLIT waves take the K steps (64 bytes of K
+//     per row, 128 for f8) round robin (wave w: steps w, w + KSPLIT, ...), so
+//     together they read the workgroup's RHS panels front to back;
 //   * each lane loads its MFMA operands straight from global memory, the RHS
 //     from HBM and the (small, shared) LHS from L2, D steps ahead of the MFMAs
 //     through D register buffers;
@@ -13,7 +13,9 @@
 //     adds them in wave order and stores.
 //
 // Operand layout, K-order freedom of the MFMA and the output addressing are
-// those of mmt4d_mfma_kernel.h, whose Args this kernel takes. The launcher may
+// those of mmt4d_mfma_kernel.h, whose Args this kernel takes. With TM = TN = 4
+// the same kernel serves problems of few 64x64 blocks and a long K, where the
+// split of K over the waves matters more than operand reuse. The launcher may
 // hand the operands over swapped (RHS as LHS) to serve N-thin problems: rows
 // and columns then trade places in Args, four consecutive columns of the
 // kernel are four rows of the caller's matrix (so `vec_out` is 0), and the
