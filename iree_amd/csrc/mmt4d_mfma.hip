@@ -132,6 +132,11 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
       if ((uintptr_t)pr.acc & 3) return -1;
     }
   }
+  // The kernels add unsigned 32-bit offsets to panel bases: no negative strides.
+  if (pr.lhs_stride < 0 || pr.rhs_stride < 0 || pr.out_stride < 0 || pr.out_sm0 < 0 ||
+      pr.acc_stride < 0) {
+    return -1;
+  }
   // 16-byte vector loads need 16-byte aligned panels (8-byte loads of 4-bit
   // rows: 8-byte aligned).
   if (((uintptr_t)pr.lhs | (uint64_t)pr.lhs_stride) & 15) return -1;

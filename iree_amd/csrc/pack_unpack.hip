@@ -1082,7 +1082,9 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   a.lds_buf_bytes = (uint32_t)((lds_bytes + 255) / 256 * 256);
   // Streaming kernels: 32-bit offsets inside one block on both sides, granules
   // of at least 4 bytes, at most 4 granules per vector, block within budget.
-  plan.stream = mat_vec >= 4 && G >= 4 && VEC / G <= 4 &&
+  // (and non-negative strides: the 32-bit offsets are unsigned)
+  plan.stream = mat_vec >= 4 && G >= 4 && VEC / G <= 4 && mat_stride0 >= 0 && v.sl0 >= 0 &&
+                v.sl1 >= 0 &&
                 block_rows * block_row_bytes <= stream_block &&
                 lds_bytes <= (big ? 80 * 1024 : 2 * stream_block) &&
                 block_rows * std::abs(mat_stride0) * es < (1ll << 31) &&

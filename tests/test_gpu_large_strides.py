@@ -64,3 +64,26 @@ def test_pack_and_unpack_row_pitch_whose_block_span_exceeds_2gib(gpu):
     want4 = tiled.permute(0, 2, 1, 3).reshape(32, 32)[:rows4, :cols4].cpu()
     got4 = torch.stack([dst[r * pitch4:r * pitch4 + cols4] for r in range(rows4)]).cpu()
     assert torch.equal(got4, want4)
+
+
+def test_mmt4d_negative_panel_stride_takes_the_signed_64_bit_kernel(gpu):
+    """A negative outer stride walks the panels backwards (mmt4d.c:70-100 does
+    signed index arithmetic and, unlike pack.c:69-71, asserts no sign): equal
+    to the forward call with the row panels reversed."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    M1, N1, K1, M0, N0, K0 = 5, 3, 8, 16, 16, 16
+    panel = K1 * M0 * K0
+    g = torch.Generator(device="cuda"); g.manual_seed(33)
+    lhs = torch.randint(-128, 128, (M1, panel), generator=g, device="cuda", dtype=torch.int8)
+    rhs = torch.randint(-128, 128, (N1, K1 * N0 * K0), generator=g, device="cuda", dtype=torch.int8)
+    fwd = torch.zeros(M1, N1 * M0 * N0, device="cuda", dtype=torch.int32)
+    lib.mmt4d(lhs.data_ptr(), 0, panel, rhs.data_ptr(), 0, K1 * N0 * K0, fwd.data_ptr(), 0, N1 * M0 * N0,
+              M1, N1, K1, M0, N0, K0, uk.MMT4D_TYPE_S8S8S32 | 0x200)
+    assert lib.last_kernel_name().startswith("mmt4d_mfma")
+    bwd = torch.zeros_like(fwd)
+    lib.mmt4d(lhs.data_ptr(), (M1 - 1) * panel, -panel, rhs.data_ptr(), 0, K1 * N0 * K0, bwd.data_ptr(), 0,
+              N1 * M0 * N0, M1, N1, K1, M0, N0, K0, uk.MMT4D_TYPE_S8S8S32 | 0x200)
+    lib.synchronize()
+    assert lib.last_kernel_name() == "mmt4d_generic"
+    assert torch.equal(bwd, fwd.flip(0))
