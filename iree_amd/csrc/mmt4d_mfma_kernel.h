@@ -799,12 +799,14 @@ void mmt4d_mfma_kernel(Args a) {
     //   issues the LHS global loads of step s+4 into register set (P+1)%3,
     //   stores register set (P+2)%3 (step s+2, loaded in iteration s-2) to
     //   LDS stage (P+2)%3, and loads the RHS fragments of step s+2 into
-    //   buffer (P+2)%3. LHS fragments are fetched one row ahead.
+    //   buffer (P+2)%3. LHS fragments are fetched two rows ahead through a
+    //   ring of three (an LDS read then has eight MFMAs to arrive in, not four).
     static_assert(RBC >= 16, "register-direct RHS needs row bytes >= 16");
     static_assert(NKK == 1 && TM % 2 == 0, "see PIPE 1");
     constexpr int NP = NU;
+    constexpr int FR = 3;  // LHS fragment ring: row tm of phase P sits in slot (P * TM + tm) % 3
     v4i regs[3][NU][R];
-    v4i fa[2][HALVES], fb[3][TN][HALVES];
+    v4i fa[FR][HALVES], fb[3][TN][HALVES];
     const char* sbase_b = a.rhs + (int64_t)pn0 * a.rhs_stride;
     const uint32_t kt_bytes_b = (uint32_t)a.N0 << lrb;
     const uint32_t sstep_b = (uint32_t)kts_per_step * kt_bytes_b;
@@ -847,6 +849,7 @@ void mmt4d_mfma_kernel(Args a) {
     }
     __syncthreads();
     read_a(fa[0], 0, 0);
+    read_a(fa[1], 0, 1);
     auto iteration = [&](int s, auto phase) {
       constexpr int P = decltype(phase)::value;
       constexpr uint32_t st_cur = P * STAGE, st_next = ((P + 1) % 3) * STAGE,
@@ -863,11 +866,11 @@ void mmt4d_mfma_kernel(Args a) {
           *reinterpret_cast<v4i*>(lds + st_write + loff[k]) = regs[(P + 2) % 3][k][0];
           regs[(P + 1) % 3][k][0] = load_piece(k, voff[k] + (uint32_t)ld_step * sstep[k]);
         }
-        if (tm + 1 < TM) read_a(fa[(tm + 1) & 1], st_cur, tm + 1);
-        else read_a(fa[0], st_next, 0);
+        if (tm + 2 < TM) read_a(fa[(P * TM + tm + 2) % FR], st_cur, tm + 2);
+        else read_a(fa[(P * TM + tm + 2) % FR], st_next, tm + 2 - TM);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
-          acc[tm][tn] = TT::mfma(fb[P][tn], fa[tm & 1], acc[tm][tn]);
+          acc[tm][tn] = TT::mfma(fb[P][tn], fa[(P * TM + tm) % FR], acc[tm][tn]);
         __builtin_amdgcn_sched_barrier(0);
       }
       __syncthreads();
