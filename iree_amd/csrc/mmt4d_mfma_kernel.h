@@ -749,9 +749,17 @@ void mmt4d_mfma_kernel(Args a) {
     store_lds(regs[0], 0);
     load_global(regs[0], min(1, last), false);
     store_lds(regs[0], STAGE);
-    load_global(regs[1], min(2, last), false);
+    // What iteration -1 would have left in flight, in the loop's own issue
+    // order (see PIPE 3 below for why the order matters).
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) load_b(fb[0][tn], tn, 0);
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+      for (int tn = tm * TN / TM; tn < (tm + 1) * TN / TM; ++tn) load_b(fb[0][tn], tn, 0);
+#pragma unroll
+      for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k)
+        regs[1][k][0] = load_piece(k, voff[k] + (uint32_t)min(2, last) * sstep[k]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
     read_a(fa[0], 0, 0);
     uint32_t st_cur = 0, st_next = STAGE, st_write = 2 * STAGE;
@@ -837,16 +845,32 @@ void mmt4d_mfma_kernel(Args a) {
                                                (tm * NCHB + h) * 1024 + rd_slot[h]);
     };
     load_global(regs[0], 0, false);
-    store_lds(regs[0], 0);
     load_global(regs[1], min(1, last), false);
+    store_lds(regs[0], 0);
     store_lds(regs[1], STAGE);
-    load_global(regs[2], min(2, last), false);
-    load_global(regs[0], min(3, last), false);
+    // What iterations -2 and -1 would have left in flight, issued in the order
+    // in which the loop issues it (RHS fragments and LHS pieces interleaved
+    // row by row). The order matters: the wait counters are in-order, and the
+    // waits the compiler places in the loop must hold on entry from here as
+    // well as around the back edge. Were the fragments of steps 0 and 1 the
+    // newest loads here, the first phase of the loop would wait for nearly
+    // everything in flight, every third step.
+    auto issue_like_iteration = [&](auto bbuf, int b_step, auto aset, int a_step) {
+      constexpr int BB = decltype(bbuf)::value, AS = decltype(aset)::value;
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-      load_b(fb[0][tn], tn, 0);
-      load_b(fb[1][tn], tn, min(1, last));
-    }
+      for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int tn = tm * TN / TM; tn < (tm + 1) * TN / TM; ++tn) load_b(fb[BB][tn], tn, b_step);
+#pragma unroll
+        for (int k = tm * NP / TM; k < (tm + 1) * NP / TM; ++k)
+          regs[AS][k][0] = load_piece(k, voff[k] + (uint32_t)a_step * sstep[k]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    issue_like_iteration(std::integral_constant<int, 0>{}, 0, std::integral_constant<int, 2>{},
+                         min(2, last));
+    issue_like_iteration(std::integral_constant<int, 1>{}, min(1, last),
+                         std::integral_constant<int, 0>{}, min(3, last));
     __syncthreads();
     read_a(fa[0], 0, 0);
     read_a(fa[1], 0, 1);
