@@ -24,7 +24,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 EXTRA_WORKLOADS = [
-    "s8_mmt4d_8192_k2", "s8_mmt4d_8192_k16", "s8_mmt4d_8192_k64", "s8_mmt4d_1024_k2",
+    "s8_mmt4d_8192_k2", "s8_mmt4d_8192_k16", "s8_mmt4d_8192_k16_zeros", "s8_mmt4d_8192_k64",
+    "s8_mmt4d_1024_k2",
     "c2_f16_chain_ragged", "c2_f16_fused_4096", "c2_f16_fused_ragged", "c3_s8_decode",
     "c3_s8_decode_fused", "c4_f8_prefill",
     "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "f32_mmt4d_4096_k1",
@@ -315,7 +316,7 @@ def main() -> int:
             if w.flops:
                 # sum of the kernels' device times (no launch gaps)
                 entry["chain_TFLOPs"] = round(w.flops / (total_us * 1e-6) / 1e12, 3)
-            if not args.no_cpu:
+            if not args.no_cpu and not name.endswith("_zeros"):
                 try:
                     entry["cpu_baseline"] = cpu_baseline_extra(w)
                 except Exception as e:  # the baseline is a reported aside, never fatal

@@ -200,18 +200,31 @@ class Runner:
                             "f16", dict(a=a, bt=bt, lhs4=lhs4, rhs4=rhs4, out=out, M=M, N=N, K=K,
                                         M0=M0, N0=N0, K0=K0))
         if name.startswith("s8_mmt4d_"):
-            # s8_mmt4d_<size>_k<K0>, tiles 16x16xK0, packed operands filled directly.
-            _, _, size, k0 = name.split("_")
+            # s8_mmt4d_<size>_k<K0>[_zeros], tiles 16x16xK0, packed operands
+            # filled directly. `_zeros` is a power probe: the same launch on
+            # all-zero operands, i.e. the same instructions and memory traffic
+            # with next to no switching in the multipliers. What it gains over
+            # the uniform-random case is clock the part gives up under load,
+            # not kernel structure.
+            parts = name.split("_")
+            zeros = len(parts) == 5 and parts[4] == "zeros"
+            if len(parts) != 4 and not zeros:
+                raise ValueError(f"unknown workload {name!r}")
+            size, k0 = parts[2], parts[3]
             S, K0 = int(size), int(k0[1:])
             M0 = N0 = 16
             M1 = N1 = S // 16
             K1 = S // K0
             lhs4 = self.uniform_s8((M1 * K1 * M0 * K0,), 3)
             rhs4 = self.uniform_s8((N1 * K1 * N0 * K0,), 4)
+            if zeros:
+                lhs4.zero_()
+                rhs4.zero_()
             out4 = self.empty(M1 * N1 * M0 * N0, torch.int32)
             op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
                                 uk.MMT4D_TYPE_S8S8S32, "s8", 1)
-            return Workload(name, f"mmt4d s8xs8->s32 {S}^3 tiles 16x16x{K0}", [op], op.flops,
+            return Workload(name, f"mmt4d s8xs8->s32 {S}^3 tiles 16x16x{K0}" +
+                            (" on all-zero operands (power probe)" if zeros else ""), [op], op.flops,
                             op.bytes, "s8", dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1,
                                                  N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
         if name.startswith("bf16_mmt4d_"):
