@@ -352,9 +352,13 @@ IREE_UK_AMD_EXPORT const char* iree_uk_amd_version(void);
 
 /* The convolution ukernel of the same reference library
  * (runtime/src/iree/builtins/ukernel/conv_nchwc.h:14-31), kept so that the
- * library stands in for all of iree/builtins/ukernel/api.h. It is served by a
- * scalar kernel (one thread per output element, the reference's accumulation
- * order): correct for every shape, not tuned.
+ * library stands in for all of iree/builtins/ukernel/api.h. Tile shapes
+ * k0 = 16, c0 a multiple of 16 (the reference's own tuned shape is 16x16,
+ * arch/x86_64/conv_nchwc_x86_64_avx512_base.c:17-28) run on the matrix cores
+ * (v_mfma_f32_16x16x4_f32; sums in MFMA order, equal to the reference's to f32
+ * rounding and exactly where the partial sums are exact); every other shape on
+ * a scalar kernel (one thread per output element, the reference's generic
+ * accumulation order, bit-identical to it).
  *
  * input [N][IC_outer][IH][IW][c0], filter [OC_outer][IC_outer][FH][FW][c0][k0],
  * output [N][OC_outer][OH][OW][k0]; the named strides are in elements.
@@ -421,8 +425,9 @@ IREE_UK_AMD_EXPORT void iree_uk_conv_nchwc(
 /* Replaces iree_uk_conv_nchwc_p (conv_nchwc_internal.h:48, conv_nchwc.c:132-155). */
 IREE_UK_AMD_EXPORT void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params);
 /* Replace iree_uk_conv_nchwc_info (conv_nchwc.h:29-31, conv_nchwc.c:210-218) and
- * iree_uk_conv_nchwc_info_p (conv_nchwc.c:200-208): 0, there is no tuned
- * kernel, so callers must pass ALLOW_GENERIC_FALLBACK_TILE_FUNCTION. */
+ * iree_uk_conv_nchwc_info_p (conv_nchwc.c:200-208):
+ * HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION for k0 = 16 with c0 a multiple of
+ * 16, else 0 and callers must pass ALLOW_GENERIC_FALLBACK_TILE_FUNCTION. */
 IREE_UK_AMD_EXPORT uint32_t iree_uk_conv_nchwc_info(int32_t k0, int32_t c0, uint32_t flags,
                                                     const uint64_t* cpu_data);
 IREE_UK_AMD_EXPORT uint32_t iree_uk_conv_nchwc_info_p(

@@ -52,7 +52,11 @@ int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* params,
                                  const char** kernel_name);
 
 int iree_uk_amd_hip_launch_conv_nchwc(const iree_uk_conv_nchwc_params_t* params,
-                                      void* stream, const char** kernel_name);
+                                      void* stream, int kernel_mode,
+                                      const char** kernel_name);
+/* 1 when the MFMA kernel serves (k0, c0, type) for every problem size. */
+int iree_uk_amd_hip_conv_nchwc_has_mfma_kernel(int32_t k0, int32_t c0,
+                                               uint32_t flags);
 
 /* 1 when an MFMA kernel serves (M0,N0,K0,type) regardless of M,N,K. */
 int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0, int32_t K0,

@@ -714,15 +714,21 @@ static int conv_nchwc_validate(const iree_uk_conv_nchwc_params_t* p) {
   return 1;
 }
 
+/* conv_nchwc.c:200-218: the bit says that a tuned (here: MFMA) kernel serves
+ * the tile shape, in which case the fallback flag is not needed. */
 uint32_t iree_uk_conv_nchwc_info_p(const iree_uk_conv_nchwc_params_t* params) {
-  (void)params;
-  return 0; /* served by the scalar kernel only */
+  return iree_uk_amd_hip_conv_nchwc_has_mfma_kernel(params->k0, params->c0,
+                                                    params->flags)
+             ? IREE_UK_FLAG_CONV_NCHWC_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
+             : 0;
 }
 
 uint32_t iree_uk_conv_nchwc_info(int32_t k0, int32_t c0, uint32_t flags,
                                  const uint64_t* cpu_data) {
-  (void)k0; (void)c0; (void)flags; (void)cpu_data;
-  return 0;
+  (void)cpu_data;
+  return iree_uk_amd_hip_conv_nchwc_has_mfma_kernel(k0, c0, flags)
+             ? IREE_UK_FLAG_CONV_NCHWC_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
+             : 0;
 }
 
 void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params) {
@@ -738,7 +744,8 @@ void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params) {
       params->IC_outer == 0 || params->FH == 0 || params->FW == 0;
   if (no_taps && (params->flags & IREE_UK_FLAG_CONV_NCHWC_ACCUMULATE)) return;
   /* conv_nchwc.c:139-152 */
-  if (!(params->flags &
+  if (!iree_uk_conv_nchwc_info_p(params) &&
+      !(params->flags &
         IREE_UK_FLAG_CONV_NCHWC_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)) {
     assert_fail(__FILE__, __LINE__, __func__,
                 "no target-specific tile function, and fallback not enabled.");
@@ -776,7 +783,8 @@ void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params) {
     if (in.device) { p.input_buffer = in.device; p.input_offset = 0; }
     if (flt.device) { p.filter_buffer = flt.device; p.filter_offset = 0; }
     if (out.device) { p.output_buffer = out.device; p.output_offset = 0; }
-    st = iree_uk_amd_hip_launch_conv_nchwc(&p, tls_stream, &tls_kernel_name);
+    st = iree_uk_amd_hip_launch_conv_nchwc(&p, tls_stream, tls_kernel_mode,
+                                           &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
   if (in.device || flt.device || out.device) {

@@ -64,10 +64,16 @@ class ConvCase:
                   self.k0, self.c0, self.stride_h, self.stride_w, self.flags))
 
 
-def cases(seed: int):
+# Larger than anything in the reference's grid: several 16-pixel panels per
+# row, an odd number of output-channel blocks, strides in both directions.
+WIDE_SHAPES = [(2, 3, 4, 40, 2, 3, 3, 1, 1), (1, 3, 2, 35, 1, 2, 2, 2, 1), (1, 5, 3, 64, 3, 1, 1, 1, 2),
+               (1, 2, 2, 17, 1, 3, 3, 2, 2)]
+
+
+def cases(seed: int, tiles=None, shapes=None):
     rng = np.random.default_rng(seed)
-    for (k0, c0) in TILES:
-        for shape in SHAPES:
+    for (k0, c0) in (tiles or TILES):
+        for shape in (shapes or SHAPES):
             for acc in (0, 1):
                 N, OC, OH, OW, IC, FH, FW, sh, sw = shape
                 H = (OH - 1) * sh + FH if OH else FH
