@@ -4,11 +4,12 @@
 //     tuned tile shape is 16 x 16 x 16,
 //     runtime/src/iree/builtins/ukernel/arch/x86_64/conv_nchwc_x86_64_avx512_base.c:17-28):
 //     an output panel of 16 pixels x 16 channels is a 16x16 MFMA block whose K
-//     runs over (ic_outer, fh, fw, ci). A wave owns TW panels along OW times
-//     TO along OC_outer and feeds v_mfma_f32_16x16x4_f32 straight from global
-//     memory: a lane's 16-byte piece of one input pixel (four ci) is the
-//     operand of four instructions, one per word, against four filter words
-//     of the same four ci. Sums are in MFMA order, so results equal the
+//     runs over (ic_outer, fh, fw, ci). A wave owns TW panels of consecutive
+//     output pixels times TO blocks of OC_outer and feeds
+//     v_mfma_f32_16x16x4_f32: a lane's 16-byte piece of one input pixel (four
+//     ci, straight from global memory) is the operand of four instructions,
+//     one per word, against four filter words of the same four ci (staged
+//     through LDS by the workgroup). Sums are in MFMA order, so results equal the
 //     reference's to rounding, and exactly where every partial sum is exact
 //     (the reference's own test data, tools/conv_nchwc_test.c:174-178).
 //   * conv_nchwc_generic, for every other shape: one thread per output
@@ -17,6 +18,8 @@
 //     a separate multiply and add, so that results equal the reference's
 //     generic path bit for bit.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
@@ -70,50 +73,72 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_generic_kernel(ConvArgs a
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef v4f v4f_a4 __attribute__((aligned(4)));  // dword-aligned wide accesses are legal here
 
-// One wave per work item (n, group of TO output-channel blocks, oh, group of
-// TW panels of 16 output pixels); no LDS, no barrier. Lane (q, r) = (lane / 16,
-// lane % 16) supplies input pixel r, channels 4q..4q+3 of the current 16, and
-// filter words [ci = 4q + w][ko = r]; with the filter as the first MFMA operand
-// it ends up holding output pixel r, channels 4q..4q+3: one 16-byte store.
-// Pixels and channel blocks past the end read the last valid one instead
-// (their accumulators are not stored).
+// A workgroup of four waves owns (n, TO output-channel blocks, 4 x TW panels of
+// 16 output pixels); each wave computes TW panels against all TO blocks.
+// Pixels are counted through (oh, ow) together, so rows shorter than a panel
+// waste nothing. A step is one (ic_outer, fh, fw, 16 channels): 16 input
+// floats per pixel against a [16 ci][16 ko] filter tile per channel block.
+//
+// Lane (q, r) = (lane / 16, lane % 16) supplies input pixel r, channels
+// 4q..4q+3 of the step's 16 (one 16-byte global load, a step ahead, two
+// register buffers) and filter words [ci = 4q + w][ko = r], w = 0..3. Those
+// four words are 64 bytes apart in memory, so the filter tiles go through LDS:
+// the first TO waves copy a step's tiles with one 16-byte load per lane
+// (global memory a step ahead, LDS double-buffered, rows padded to 20 floats so
+// that the 64 lanes of a read hit 64 different banks), one barrier per step.
+// With the filter as the first MFMA operand a lane ends up holding output
+// pixel r, channels 4q..4q+3: one 16-byte store. Pixels, panels and channel
+// blocks past the end read the last valid one instead and are not stored; a
+// prefetch past the last step reloads the last step.
+constexpr int kFilterRow = 20;                 // floats per padded ci row in LDS
+constexpr int kFilterTile = 16 * kFilterRow;   // floats per [16][16] tile in LDS
+
 template <int TW, int TO>
-__global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, int64_t items,
-                                                                   int64_t ow_chunks,
+__global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, int64_t px_chunks,
+                                                                   int64_t px_groups,
                                                                    int64_t oc_chunks) {
+  static_assert(TO * 64 <= kThreads, "one loader lane per 16 bytes of the step's filter tiles");
+  __shared__ __attribute__((aligned(16))) float filt[2][TO * kFilterTile];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t item = (int64_t)blockIdx.x * (kThreads / 64) + wave;
-  if (item >= items) return;
-  int64_t t = item;
-  const int64_t owc = t % ow_chunks; t /= ow_chunks;
-  const int64_t oh = t % a.OH; t /= a.OH;
+  // Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own
+  // L2. Give every XCD a contiguous range of the work instead, so that one L2
+  // sees one image and one filter slice at a time, not a slice of all.
+  const uint32_t nb = gridDim.x, xcd = blockIdx.x & 7u;
+  int64_t t = (int64_t)(xcd * (nb / 8u) + min(xcd, nb % 8u) + (blockIdx.x >> 3));
+  const int64_t pxg = t % px_groups; t /= px_groups;
   const int64_t occ = t % oc_chunks;
   const int64_t n = t / oc_chunks;
+  const int64_t pxc_raw = pxg * 4 + wave;
+  const bool wave_ok = pxc_raw < px_chunks;
+  const int64_t pxc = wave_ok ? pxc_raw : px_chunks - 1;
   const int r = lane & 15, q = lane >> 4;
+  const int64_t pixels = a.OH * a.OW;
 
   const float* pa[TW];
-  const float* pb[TO];
   float* po[TW][TO];
   bool ok[TW][TO];
 #pragma unroll
   for (int tw = 0; tw < TW; ++tw) {
-    const int64_t ow = owc * (16 * TW) + tw * 16 + r;
-    const int64_t ow_in = ow < a.OW ? ow : a.OW - 1;
-    pa[tw] = a.in + n * a.in_sn + (oh * a.stride_h) * a.in_sh + (ow_in * a.stride_w) * a.c0 + 4 * q;
+    const int64_t px = pxc * (16 * TW) + tw * 16 + r;
+    const int64_t px_in = px < pixels ? px : pixels - 1;
+    const int64_t oh = px_in / a.OW, ow = px_in - oh * a.OW;
+    pa[tw] = a.in + n * a.in_sn + (oh * a.stride_h) * a.in_sh + (ow * a.stride_w) * a.c0 + 4 * q;
 #pragma unroll
     for (int to = 0; to < TO; ++to) {
       const int64_t oc = occ * TO + to;
       const int64_t oc_in = oc < a.OC ? oc : a.OC - 1;
-      ok[tw][to] = ow < a.OW && oc < a.OC;
-      po[tw][to] = a.out + n * a.out_sn + oc_in * a.out_soc + oh * a.out_soh + ow_in * 16 + 4 * q;
+      ok[tw][to] = wave_ok && px < pixels && oc < a.OC;
+      po[tw][to] = a.out + n * a.out_sn + oc_in * a.out_soc + oh * a.out_soh + ow * 16 + 4 * q;
     }
   }
-#pragma unroll
-  for (int to = 0; to < TO; ++to) {
-    const int64_t oc = occ * TO + to;
-    pb[to] = a.flt + (oc < a.OC ? oc : a.OC - 1) * a.f_soc + (4 * q) * 16 + r;
-  }
+  // Loader lanes (waves 0..TO-1): wave `wave` copies channel block occ*TO+wave,
+  // lane l the 16 bytes [ci = l / 4][ko = 4 * (l % 4) ..].
+  const bool loader = wave < TO;
+  const int64_t oc_ld = min(occ * TO + (loader ? wave : 0), a.OC - 1);
+  const float* pf = a.flt + oc_ld * a.f_soc + lane * 4;
+  const int f_dst = (loader ? wave : 0) * kFilterTile + (lane >> 2) * kFilterRow + (lane & 3) * 4;
+  const int f_src = (4 * q) * kFilterRow + r;   // + to * kFilterTile + w * kFilterRow
 
   v4f acc[TW][TO];
 #pragma unroll
@@ -124,33 +149,70 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
       if (a.accumulate && ok[tw][to]) acc[tw][to] = *reinterpret_cast<const v4f_a4*>(po[tw][to]);
     }
 
-  // Within one (ic_outer, fh) the taps (fw, 16 channels at a time) follow each
-  // other at 16 input floats and 256 filter floats.
+  // Within one (ic_outer, fh) consecutive steps follow each other at 16 input
+  // floats and 256 filter floats.
   const int64_t taps = a.FW * (a.c0 / 16);
-  for (int64_t ic = 0; ic < a.IC; ++ic) {
-    for (int64_t fh = 0; fh < a.FH; ++fh) {
-      const int64_t ao = ic * a.in_sic + fh * a.in_sh;
-      const int64_t bo = ic * a.f_sic + fh * a.f_sfh;
-      for (int64_t tap = 0; tap < taps; ++tap) {
-        v4f av[TW];
-        float bv[TO][4];
+  const int64_t steps = a.IC * a.FH * taps;
+  if (steps > 0) {
+    int64_t ic = 0, fh = 0, tap = 0;  // the step the next prefetch loads
+    v4f av[2][TW];
+    v4f fv = v4f{0.f, 0.f, 0.f, 0.f};
+    auto prefetch = [&](auto buf) {
+      constexpr int B = decltype(buf)::value;
+      const int64_t ao = ic * a.in_sic + fh * a.in_sh + tap * 16;
+      const int64_t bo = ic * a.f_sic + fh * a.f_sfh + tap * 256;
+      // Every wave issues the filter load (the waves that do not stage it read
+      // the first block's tile and drop it): one issue order on all paths
+      // keeps the compiler's wait counts from covering the loads just issued.
+      fv = *reinterpret_cast<const v4f_a4*>(pf + bo);
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) av[B][tw] = *reinterpret_cast<const v4f_a4*>(pa[tw] + ao);
+      // Advance, staying on the last step once it is reached.
+      if (!(ic == a.IC - 1 && fh == a.FH - 1 && tap == taps - 1)) {
+        if (++tap == taps) {
+          tap = 0;
+          if (++fh == a.FH) {
+            fh = 0;
+            ++ic;
+          }
+        }
+      }
+    };
+    auto stage_filter = [&](int b) {
+      if (loader) *reinterpret_cast<v4f*>(&filt[b][f_dst]) = fv;
+    };
+    // Computes the step held in av[B] and filt[B]; meanwhile fetches the next
+    // step into av[1 - B] and, through fv, filt[1 - B].
+    auto iteration = [&](auto buf) {
+      constexpr int B = decltype(buf)::value;
+      prefetch(std::integral_constant<int, 1 - B>{});
+      float bv[TO][4];
+#pragma unroll
+      for (int to = 0; to < TO; ++to)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) bv[to][w] = filt[B][to * kFilterTile + w * kFilterRow + f_src];
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
 #pragma unroll
         for (int tw = 0; tw < TW; ++tw)
-          av[tw] = *reinterpret_cast<const v4f_a4*>(pa[tw] + ao + tap * 16);
 #pragma unroll
-        for (int to = 0; to < TO; ++to)
-#pragma unroll
-          for (int w = 0; w < 4; ++w) bv[to][w] = pb[to][bo + tap * 256 + w * 16];
-#pragma unroll
-        for (int w = 0; w < 4; ++w)
-#pragma unroll
-          for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-            for (int to = 0; to < TO; ++to)
-              acc[tw][to] =
-                  __builtin_amdgcn_mfma_f32_16x16x4f32(bv[to][w], av[tw][w], acc[tw][to], 0, 0, 0);
-      }
+          for (int to = 0; to < TO; ++to)
+            acc[tw][to] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[to][w], av[B][tw][w],
+                                                               acc[tw][to], 0, 0, 0);
+      stage_filter(1 - B);
+      __syncthreads();
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    prefetch(B0{});
+    stage_filter(0);
+    __syncthreads();
+    int64_t s = 0;
+    for (; s + 1 < steps; s += 2) {
+      iteration(B0{});
+      iteration(B1{});
     }
+    if (s < steps) iteration(B0{});
   }
 #pragma unroll
   for (int tw = 0; tw < TW; ++tw)
@@ -161,14 +223,22 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
 
 template <int TW, int TO>
 int launch_mfma(const ConvArgs& a, int64_t N, hipStream_t stream) {
-  const int64_t ow_chunks = uk::ceil_div(a.OW, (int64_t)16 * TW);
+  const int64_t px_chunks = uk::ceil_div(a.OH * a.OW, (int64_t)16 * TW);
+  const int64_t px_groups = uk::ceil_div(px_chunks, (int64_t)(kThreads / 64));
   const int64_t oc_chunks = uk::ceil_div(a.OC, (int64_t)TO);
-  const int64_t items = N * oc_chunks * a.OH * ow_chunks;
-  const int64_t blocks = uk::ceil_div(items, (int64_t)(kThreads / 64));
+  const int64_t blocks = N * oc_chunks * px_groups;
   if (blocks >= (1ll << 31)) return -1;
   uk::launch(3, conv_nchwc_mfma_kernel<TW, TO>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
-             a, items, ow_chunks, oc_chunks);
+             a, px_chunks, px_groups, oc_chunks);
   return (int)hipGetLastError();
+}
+
+template <int TO>
+int launch_mfma_for_pixels(const ConvArgs& a, int64_t N, hipStream_t stream) {
+  const int64_t pixels = a.OH * a.OW;
+  if (pixels > 48) return launch_mfma<4, TO>(a, N, stream);
+  if (pixels > 16) return launch_mfma<2, TO>(a, N, stream);
+  return launch_mfma<1, TO>(a, N, stream);
 }
 
 }  // namespace
@@ -205,9 +275,8 @@ extern "C" int iree_uk_amd_hip_launch_conv_nchwc(const iree_uk_conv_nchwc_params
   }
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC &&
       iree_uk_amd_hip_conv_nchwc_has_mfma_kernel(p->k0, p->c0, p->flags)) {
-    const bool wide = a.OW > 16, deep = a.OC > 1;
-    int st = wide ? (deep ? launch_mfma<2, 2>(a, p->N, stream) : launch_mfma<2, 1>(a, p->N, stream))
-                  : (deep ? launch_mfma<1, 2>(a, p->N, stream) : launch_mfma<1, 1>(a, p->N, stream));
+    int st = a.OC > 1 ? launch_mfma_for_pixels<2>(a, p->N, stream)
+                      : launch_mfma_for_pixels<1>(a, p->N, stream);
     if (st >= 0) {
       *kernel_name = "conv_nchwc_mfma";
       return st;

@@ -358,6 +358,30 @@ class Runner:
                             ops, 2.0 * M * N * K, sum(o.bytes for o in ops), "f8",
                             dict(a=a, bt=bt, lhs4=lhs4, rhs4=rhs4, out4=out4, M=M, N=N, K=K,
                                  M1=M1, N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
+        if name == "conv_nchwc_f32_n16_56x56_c256_k256_3x3":
+            # iree_uk_conv_nchwc at the reference's tuned tile shape (k0 = c0 = 16):
+            # a 3x3 stride-1 layer, 256 -> 256 channels, 56x56 outputs, batch 16.
+            N, ICo, OCo, OH, OW, FH, FW, k0, c0 = 16, 16, 16, 56, 56, 3, 3, 16, 16
+            H, W = OH + FH - 1, OW + FW - 1
+            x = self.normal((N * ICo * H * W * c0,), torch.float32, 20)
+            w = self.normal((OCo * ICo * FH * FW * c0 * k0,), torch.float32, 21)
+            y = self.empty(N * OCo * OH * OW * k0, torch.float32)
+            lib = self.lib
+            xp, wp, yp = x.data_ptr(), w.data_ptr(), y.data_ptr()
+            in_strides = (ICo * H * W * c0, H * W * c0, W * c0)
+            f_strides = (ICo * FH * FW * c0 * k0, FH * FW * c0 * k0, FW * c0 * k0)
+            out_strides = (OCo * OH * OW * k0, OH * OW * k0, OW * k0)
+
+            def launch():
+                lib.conv_nchwc(xp, 0, *in_strides, wp, 0, *f_strides, yp, 0, *out_strides,
+                               N, OCo, OH, OW, ICo, FH, FW, k0, c0, 1, 1, 0x01)
+            flops = 2.0 * N * OCo * k0 * OH * OW * ICo * c0 * FH * FW
+            nbytes = 4.0 * (x.numel() + w.numel() + y.numel())
+            op = Op("conv", launch, flops, nbytes, "mfma", "f32")
+            return Workload(name, "conv_nchwc f32 N=16 256->256 channels 56x56 outputs 3x3 stride 1, "
+                            "tiles k0=16 c0=16", [op], flops, nbytes, "f32",
+                            dict(x=x, w=w, y=y, N=N, ICo=ICo, OCo=OCo, OH=OH, OW=OW, FH=FH, FW=FW,
+                                 k0=k0, c0=c0))
         if name in ("c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288"):
             rows, cols = (12288, 12289) if name.endswith("12289") else (12289, 12288)
             x = self.normal((rows, cols), torch.float32, 12)
