@@ -31,6 +31,7 @@ EXTRA_WORKLOADS = [
     "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "f32_mmt4d_4096_k1",
     "f32_mmt4d_4096_k4",
     "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288",
+    "conv_nchwc_f32_n16_56x56_c256_k256_3x3",
 ]
 
 
@@ -169,6 +170,31 @@ def cpu_baseline_extra(wl, target_seconds: float = 3.0):
                 "kind": "reference" if have_ref else "port",
                 "sample": f"pack + unpack of the first {slab_rows} of {rows} rows, 1 thread "
                           f"({t_pack:.2f} s + {t_un:.2f} s); round trip exact: {ok}"}
+    if wl.name.startswith("conv_nchwc"):
+        # One image of the batch, single thread, the reference's AVX-512
+        # 16x16x16 tile when the host has it (else its generic tile); the GPU
+        # result of the same image is compared on the way.
+        chk = uk_oracle.Checker("reference" if have_ref else "oracle")
+        chk.use_host_cpu_features(True)
+        d = {k: keep[k] for k in ("N", "ICo", "OCo", "OH", "OW", "FH", "FW", "k0", "c0")}
+        H, W = d["OH"] + d["FH"] - 1, d["OW"] + d["FW"] - 1
+        in_s = (d["ICo"] * H * W * d["c0"], H * W * d["c0"], W * d["c0"])
+        f_s = (d["ICo"] * d["FH"] * d["FW"] * d["c0"] * d["k0"], d["FH"] * d["FW"] * d["c0"] * d["k0"],
+               d["FW"] * d["c0"] * d["k0"])
+        o_s = (d["OCo"] * d["OH"] * d["OW"] * d["k0"], d["OH"] * d["OW"] * d["k0"], d["OW"] * d["k0"])
+        x = keep["x"][:in_s[0]].cpu().numpy()
+        w = keep["w"].cpu().numpy()
+        y = np.zeros(o_s[0], np.float32)
+        t0 = time.perf_counter()
+        chk.conv_nchwc(x, 0, *in_s, w, 0, *f_s, y, 0, *o_s, 1, d["OCo"], d["OH"], d["OW"], d["ICo"],
+                       d["FH"], d["FW"], d["k0"], d["c0"], 1, 1, 0x01 | 0x200)
+        t = time.perf_counter() - t0
+        got = keep["y"][:o_s[0]].cpu().numpy()
+        err = float(np.abs(got - y).max() / np.abs(y).max())
+        return {"value": round(wl.flops / d["N"] / t / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                "kind": "reference" if have_ref else "port",
+                "sample": f"image 0 of {d['N']}, 1 thread ({t:.2f} s), host ISA paths enabled; "
+                          f"GPU result of that image: max|gpu-ref|/max|ref| = {err:.2e}"}
     if "lhs4" not in keep or "M1" not in keep and "M" not in keep:
         return None
     dtype = wl.dtype
@@ -271,7 +297,9 @@ def main() -> int:
                                "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"]}
 
     if wl.flops:
-        metric, unit = "mmt4d TFLOP/s over the pack->mmt4d->unpack chain", "TFLOP/s"
+        metric = ("conv_nchwc TFLOP/s" if dominant == "conv"
+                  else "mmt4d TFLOP/s over the pack->mmt4d->unpack chain")
+        unit = "TFLOP/s"
         value = wl.flops / sec_per_step / 1e12
     else:
         metric, unit = "pack/unpack HBM GB/s", "GB/s"

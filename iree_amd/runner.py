@@ -399,7 +399,7 @@ class Runner:
         raise KeyError(name)
 
     # ------------------------------------------------------------------ timing
-    KIND = {"pack": 0, "unpack": 1, "mmt4d": 2}
+    KIND = {"pack": 0, "unpack": 1, "mmt4d": 2, "conv": 3}
 
     def time_op(self, op: Op, iters: int, warmup: int = 5):
         """(average, minimum, median) device duration in microseconds of
@@ -467,7 +467,8 @@ class Runner:
         import time
         torch = self.torch
         dom_kind = self.KIND["mmt4d" if dominant == "mmt4d" else
-                             ("unpack" if dominant.startswith("unpack") else "pack")]
+                             ("conv" if dominant == "conv" else
+                              ("unpack" if dominant.startswith("unpack") else "pack"))]
         n_dom = sum(1 for op in wl.ops if op.name == dominant)
         with torch.cuda.stream(self.stream):
             # The device needs tens of milliseconds of load before its clocks
