@@ -316,7 +316,7 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_pointer_mode(int mode);
  *   MFMA_VARIANT + v : mmt4d takes MFMA workgroup shape v where it can serve
  *             the call (1 = 256x256, 2 = 128x128, 3 = 64x64, 4 = the M-thin
  *             kernels, 5 = the M-thin kernel on the transposed problem,
- *             6 = the 64x64 K-split kernel, 7 = 256x128)
+ *             6 = the 64x64 K-split kernel, 7 = 256x128, 8 = 128x512)
  *             instead of choosing by problem size; pack/unpack as AUTO. */
 enum {
   IREE_UK_AMD_KERNEL_MODE_AUTO = 0,

@@ -52,7 +52,7 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   if (p.M0 > SH::BM || p.N0 > SH::BN) return -1;      // at least one whole panel
   if (p.M0 % R || p.N0 % R) return -1;                // pieces hold whole rows
   if (p.out_rows <= 0 || p.out_cols <= 0) return 0;   // a strip beyond the matrix: nothing to store
-  Args a;
+  Args a{};
   const int64_t kt_bytes_m = (int64_t)p.M0 << p.lrb, kt_bytes_n = (int64_t)p.N0 << p.lrb;
   a.lhs = p.lhs + kt_begin * kt_bytes_m;
   a.rhs = p.rhs + kt_begin * kt_bytes_n;
@@ -89,7 +89,10 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   a.dequant = p.dequant && kt_begin + kt_count == p.K1;
   a.row_scale = p.row_scale;
   a.col_scale = p.col_scale;
-  a.band = 4;
+  // Block rows per rasterization band: an XCD's 32 resident workgroups should
+  // cover a near-square patch of the output (4 x 8 blocks of 256x256, 8 x 4 of
+  // 128x512: 3072 operand rows either way).
+  a.band = (WGM == 1 && WGN == 8) ? 8 : 4;
   // Four consecutive output columns of one row are contiguous when they lie in
   // one tile row (N0 % 4 == 0) or when column panels follow each other without
   // a gap (row-major output, or tiles that are single rows). 4-byte outputs
@@ -217,7 +220,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //   small 64x64, 4 waves, any K: for problems with too few 128x128 blocks to
 //         occupy the 256 CUs;
 // `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem,
-// 6 the 64x64 K-split kernel, 7 the 256x128 shape; 0 = choose) overrides the
+// 6 the 64x64 K-split kernel, 7 the 256x128 shape, 8 the 128x512 shape;
+// 0 = choose) overrides the
 // size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
 //         streaming the RHS: the barrier-free kernel of mmt4d_mfma_thin.h (16,
@@ -235,7 +239,9 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced >= 1 && forced <= 7) {
+  if (forced == 8) {
+    choice = 1;  // the big variant in its 128x512 shape (square where that one cannot serve)
+  } else if (forced >= 1 && forced <= 7) {
     choice = forced;
   } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
     choice = 4;
@@ -329,9 +335,28 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   const int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
   if (choice == 1) {
     if (kt_main > 0) {
-      int st = launch_variant<E, RBC, 8, 4, 2, 4, 1, BIG_PIPE>(p, 0, kt_main, p.accumulate, stream);
+      int st = -1;
+      bool wide = false;
+      if constexpr (RBC >= 16 && H == 1) {
+        // 128 rows x 512 columns, the 8 waves side by side (each 128x64): no two
+        // waves load the same RHS fragments and the LDS holds half as much LHS,
+        // i.e. fewer bytes moved per MFMA, which is what a power-bound kernel
+        // is short of (8192^3 s8 418-423 -> 403-412 us, 4096^3 f16 101 -> 98 us,
+        // 8192^3 bf16 unchanged). Taken where it tiles the problem exactly;
+        // ragged problems keep the square shape and its strip logic.
+        const int bpm_w = 128 / p.M0, bpn_w = 512 / p.N0;
+        if (forced == 8 || (forced == 0 && bpm_w >= 1 && bpn_w >= 1 && p.M1 % bpm_w == 0 &&
+                            p.N1 % bpn_w == 0 && workgroups(p, 128, 512) >= 192)) {
+          st = launch_variant<E, RBC, 8, 4, 1, 8, 1, BIG_PIPE>(p, 0, kt_main, p.accumulate, stream);
+          wide = st == 0;
+        }
+      }
+      if (st < 0) {
+        st = launch_variant<E, RBC, 8, 4, 2, 4, 1, BIG_PIPE>(p, 0, kt_main, p.accumulate, stream);
+      }
       if (st == 0) {
-        *name = RBC >= 16 ? "mmt4d_mfma_256x256_rhs_direct" : "mmt4d_mfma_256x256_regroup";
+        *name = wide ? "mmt4d_mfma_128x512_rhs_direct"
+                     : (RBC >= 16 ? "mmt4d_mfma_256x256_rhs_direct" : "mmt4d_mfma_256x256_regroup");
         if (kt_main == p.K1) return 0;
         return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
       }

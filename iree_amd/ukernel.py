@@ -53,7 +53,7 @@ POINTER_MODE_AUTO = 0
 POINTER_MODE_DEVICE = 1
 KERNEL_MODE_AUTO = 0
 KERNEL_MODE_GENERIC = 1
-KERNEL_MODE_MFMA_VARIANT = 16  # + 1..4: force an mmt4d MFMA workgroup shape
+KERNEL_MODE_MFMA_VARIANT = 16  # + 1..8: force an mmt4d MFMA workgroup shape
 
 # (lhs bits, rhs bits, out bits) per mmt4d type value.
 MMT4D_TYPE_BITS = {

@@ -30,7 +30,8 @@ def _want(oracle, c, lhs, rhs, acc_tiled, rows, cols, rs, cs, ok):
 
 
 MODES = [uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_GENERIC, uk.KERNEL_MODE_MFMA_VARIANT + 1,
-         uk.KERNEL_MODE_MFMA_VARIANT + 4, uk.KERNEL_MODE_MFMA_VARIANT + 5]
+         uk.KERNEL_MODE_MFMA_VARIANT + 4, uk.KERNEL_MODE_MFMA_VARIANT + 5,
+         uk.KERNEL_MODE_MFMA_VARIANT + 8]
 
 
 @pytest.mark.gpu
@@ -152,7 +153,7 @@ def test_dequant_unpack_with_remainder_strips(gpu, accumulate):
     lib.mmt4d_dequant_unpack(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0,
                              acc.data_ptr(), 0, N1 * M0 * N0, got.data_ptr(), 0, cols, rows, cols,
                              rs.data_ptr(), cs.data_ptr(), M1, N1, K1, M0, N0, K0, flags)
-    assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256")
+    assert lib.last_kernel_name().startswith(("mmt4d_mfma_256x256", "mmt4d_mfma_128x512"))
     lib.synchronize()
     assert torch.equal(got, want)
 

@@ -86,8 +86,9 @@ def _mfma_shapes(M0, N0, K0, bits):
 # kernel when K is a whole number of 64-byte steps and rows are at least 8
 # bytes wide, else the 32x64 kernel through LDS: the shapes below have both;
 # 5 is the thin kernel on the transposed problem and 6 the same kernel with
-# 64x64 blocks, under the same conditions; 7 is the 256x128 shape).
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+# 64x64 blocks, under the same conditions; 7 is the 256x128 shape, 8 the
+# 128x512 shape).
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("n", range(len(MFMA_TILES)))
 def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu
@@ -127,14 +128,14 @@ def test_mmt4d_split_off_remainder_strips(gpu, oracle, shape):
         G.run_mmt4d_case(oracle, c, lhs, rhs, want)
         got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
         assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
-        assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256"), lib.last_kernel_name()
+        assert lib.last_kernel_name().startswith(("mmt4d_mfma_256x256", "mmt4d_mfma_128x512")), lib.last_kernel_name()
 
 
 # 16-bit float outputs: an MFMA kernel serves them when the caller allows a
 # single rounding at the end (SKIP_INTERMEDIATE_ROUNDINGS); on the reference
 # tests' small-integer inputs every f32 partial sum is exact, so the result must
 # equal the oracle's bit for bit, final rounding included.
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 8])
 @pytest.mark.parametrize("tf,M0,N0,K0", [
     (uk.MMT4D_TYPE_F16F16F16, 16, 16, 8), (uk.MMT4D_TYPE_F16F16F16, 16, 16, 1),
     (uk.MMT4D_TYPE_BF16BF16BF16, 16, 16, 8), (uk.MMT4D_TYPE_BF16BF16BF16, 8, 32, 2)])
@@ -195,7 +196,7 @@ def _normal_operand(rng, kind, n, scale=1.0):
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
     (uk.MMT4D_TYPE_F32F32F32, 8, 8, 4), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1)])
 @pytest.mark.parametrize("accumulate", [0, 1])
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 8])
 def test_mmt4d_float_tolerance_on_normal_inputs(gpu, oracle, tf, M0, N0, K0, accumulate, variant):
     lib, torch = gpu
     lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
@@ -359,14 +360,14 @@ def test_fused_mmt4d_unpack_with_remainder_strips(gpu, accumulate):
                  M1, N1, M0, N0, 0, uk.PACK_TYPE_I32I32)
     lib.mmt4d(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, tiled.data_ptr(), 0,
               N1 * M0 * N0, M1, N1, K1, M0, N0, K0, flags)
-    assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256")
+    assert lib.last_kernel_name().startswith(("mmt4d_mfma_256x256", "mmt4d_mfma_128x512"))
     want = init.clone()
     lib.unpack(tiled.data_ptr(), 0, N1 * M0 * N0, M0 * N0, want.data_ptr(), 0, cols, 1, M1, N1, M0, N0,
                rows, cols, uk.UNPACK_TYPE_I32I32)
     got = init.clone()
     lib.mmt4d_unpack(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, got.data_ptr(),
                      0, cols, rows, cols, M1, N1, K1, M0, N0, K0, flags)
-    assert lib.last_kernel_name().startswith("mmt4d_mfma_256x256")
+    assert lib.last_kernel_name().startswith(("mmt4d_mfma_256x256", "mmt4d_mfma_128x512"))
     lib.synchronize()
     assert torch.equal(got, want)
     # closed form on the last rows (they cross the row strip)

@@ -151,7 +151,7 @@ def test_mmt4d_random_sweep_larger_shapes_and_forced_variants(gpu, oracle):
         lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
         want = out0.copy()
         G.run_mmt4d_case(oracle, c, lhs, rhs, want)
-        variant = int(rng.integers(0, 8))
+        variant = int(rng.integers(0, 9))
         lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
         got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
         assert np.array_equal(got, want), (ci, c, variant, lib.last_kernel_name())
