@@ -337,12 +337,12 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     if (kt_main > 0) {
       int st = -1;
       bool wide = false;
-      if constexpr (RBC >= 16 && H == 1) {
+      if constexpr (RBC >= 16) {
         // 128 rows x 512 columns, the 8 waves side by side (each 128x64): no two
         // waves load the same RHS fragments and the LDS holds half as much LHS,
         // i.e. fewer bytes moved per MFMA, which is what a power-bound kernel
         // is short of (8192^3 s8 418-423 -> 403-412 us, 4096^3 f16 101 -> 98 us,
-        // 8192^3 bf16 unchanged). Taken where it tiles the problem exactly;
+        // 8192^3 f8 401-408 -> 389 us, 8192^3 bf16 unchanged). Taken where it tiles the problem exactly;
         // ragged problems keep the square shape and its strip logic.
         const int bpm_w = 128 / p.M0, bpn_w = 512 / p.N0;
         if (forced == 8 || (forced == 0 && bpm_w >= 1 && bpn_w >= 1 && p.M1 % bpm_w == 0 &&
