@@ -35,32 +35,52 @@ EXTRA_WORKLOADS = [
 ]
 
 
-def recorded_traffic(workload: str, op: str):
-    """HBM-side bytes per launch of the dominant kernel, from the committed
-    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of this workload (counters
-    cannot be read from inside the process); None when there is none."""
+def recorded_traffic(workload: str, op: str, kernel: str):
+    """(bytes, source): HBM-side bytes per launch of the dominant kernel from
+    the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of this
+    workload (counters cannot be read from inside the process), and the file
+    it was read from. (None, reason) when there is no summary or when the
+    summary was recorded for another kernel than the one that ran now."""
     if op != "mmt4d":
-        return None
-    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt")
+        return None, "no counter summary for this op"
+    rel = os.path.join("profiles", f"{workload}_hbm_traffic.txt")
+    value, recorded_kernel = None, None
     try:
-        with open(path) as f:
+        with open(os.path.join(ROOT, rel)) as f:
             for line in f:
                 if line.startswith("mmt4d_traffic_bytes_per_launch:"):
-                    return int(line.split(":")[1])
+                    value = int(line.split(":")[1])
+                if line.startswith("mmt4d_kernel:"):
+                    recorded_kernel = line.split(":")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, f"{rel} not found"
+    if value is None:
+        return None, f"{rel} holds no figure"
+    if recorded_kernel != kernel:
+        return None, f"{rel} was recorded for kernel {recorded_kernel!r}, this run used {kernel!r}"
+    return value, f"{rel} (recorded rocprofv3 --pmc run of this command, not measured in this run)"
+
+
+CPU_THREAD_CAP = 16   # a one-GPU box gives a job 16 cores' worth of CPU whatever nproc says
+
+
+def cpu_info() -> dict:
+    """Host cores as seen and threads as used by the CPU baselines."""
+    nproc = os.cpu_count() or 1
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except AttributeError:
+        affinity = nproc
+    n = affinity
+    omp = os.environ.get("OMP_NUM_THREADS", "")
+    if omp.isdigit():
+        n = min(n, int(omp))
+    return {"nproc": nproc, "affinity": affinity, "OMP_NUM_THREADS": omp or None,
+            "thread_cap": CPU_THREAD_CAP, "threads_used": max(1, min(n, CPU_THREAD_CAP))}
 
 
 def cpu_threads() -> int:
-    try:
-        n = len(os.sched_getaffinity(0))
-    except AttributeError:
-        n = os.cpu_count() or 1
-    for var in ("OMP_NUM_THREADS",):
-        if os.environ.get(var, "").isdigit():
-            n = min(n, int(os.environ[var]))
-    return max(1, min(n, 16))
+    return cpu_info()["threads_used"]
 
 
 def cpu_baseline_c2(keep: dict, target_seconds: float = 12.0) -> dict:
@@ -259,6 +279,68 @@ def verify_c2(runner, keep, cpu_out4, slab) -> dict:
             "ok": bool(err <= 1e-2)}
 
 
+def verify_sampled_tiles(wl, n_random: int = 64, seed: int = 0) -> dict:
+    """The mmt4d output of a workload, as the timed launches left it in HBM,
+    against the CPU oracle on sampled output tiles: the four corners plus
+    `n_random` tiles drawn at random, each over all of K (one oracle call with
+    M = N = 1 on that tile's panels). s8: bit-exact; floats: max|gpu-ref| /
+    max|ref| over the sampled elements against the tolerance of the type."""
+    import numpy as np
+    from oracle import uk_oracle
+    from iree_amd import ukernel as uk
+
+    k = wl.keep
+    dtype = wl.dtype
+    M0, N0, K0 = k["M0"], k["N0"], k["K0"]
+    if "M1" in k:
+        M1, N1, K1 = k["M1"], k["N1"], k["K1"]
+    else:
+        M1, N1, K1 = -(-k["M"] // M0), -(-k["N"] // N0), k["K"] // K0
+    es = {"s8": 1, "f8": 1, "f16": 2, "bf16": 2, "f32": 4}[dtype]
+    view = {1: np.uint8, 2: np.uint16, 4: np.uint32}[es]
+    chk = uk_oracle.get("oracle")
+    lhs = _host_bytes(k["lhs4"]).reshape(M1, K1 * M0 * K0 * es)
+    rhs = _host_bytes(k["rhs4"]).reshape(N1, K1 * N0 * K0 * es)
+    out_dt = np.int32 if dtype == "s8" else np.float32
+    got_all = _host_bytes(k["out4"]).view(out_dt).reshape(M1, N1, M0 * N0)
+    rng = np.random.default_rng(seed)
+    tiles = {(0, 0), (0, N1 - 1), (M1 - 1, 0), (M1 - 1, N1 - 1)}
+    while len(tiles) < min(n_random + 4, M1 * N1):
+        tiles.add((int(rng.integers(M1)), int(rng.integers(N1))))
+    flags = _mmt4d_type_flag(dtype, uk) | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
+    exact, max_err, max_ref = True, 0.0, 0.0
+    for (m, n) in sorted(tiles):
+        want = np.zeros(M0 * N0, out_dt)
+        chk.mmt4d(lhs[m].view(view), 0, K1 * M0 * K0, rhs[n].view(view), 0, K1 * N0 * K0, want, 0,
+                  M0 * N0, 1, 1, K1, M0, N0, K0, flags)
+        got = got_all[m, n]
+        if dtype == "s8":
+            exact = exact and bool(np.array_equal(got, want))
+        else:
+            if not (np.isfinite(got).all() and np.isfinite(want).all()):
+                return {"tiles": len(tiles), "ok": False, "error": f"non-finite value in tile ({m}, {n})"}
+            max_err = max(max_err, float(np.abs(got - want).max()))
+            max_ref = max(max_ref, float(np.abs(want).max()))
+    if dtype == "s8":
+        return {"tiles": len(tiles), "bit_exact": exact, "ok": exact}
+    tol = {"f16": 1e-2, "bf16": 1e-2, "f8": 2e-2, "f32": 1e-5}[dtype]
+    err = max_err / max_ref if max_ref else 0.0
+    return {"tiles": len(tiles), "max_err_over_max_ref": float(f"{err:.3e}"), "tolerance": tol,
+            "ok": bool(err <= tol)}
+
+
+# The north-star workloads whose figures are repeated, compactly, in the
+# top-level `targets` block at the END of the JSON line.
+TARGET_MMT4D = ["s8_mmt4d_8192_k16", "s8_mmt4d_8192_k2", "s8_mmt4d_1024_k2", "bf16_mmt4d_8192_k2",
+                "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "c4_f8_prefill"]
+TARGET_PACK = {
+    # name: (rows, row_bytes, src_pitch, dst_pitch) of the plain copy that moves
+    # the same matrix between the same two pitches
+    "c5_pack_f32_12288x12289": (12288, 49152, 49156, 49152),
+    "c5_pack_f32_12289x12288": (12288, 49152, 49152, 49216),
+}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -287,13 +369,14 @@ def main() -> int:
     roof = R.roofline(dom, dom_us)
     roof["kernel"] = dom.kernel
     roof["avg_us"] = round(dom_us, 2)
-    roof["traffic"] = recorded_traffic(args.workload, dominant)
+    roof["traffic"], roof["traffic_source"] = recorded_traffic(args.workload, dominant, dom.kernel)
 
     per_kernel = {}
     for op in wl.ops:
         avg, mn, med = R.time_op(op, max(5, min(args.steps, 30)))
         r = R.roofline(op, avg)
         per_kernel[op.name] = {"kernel": op.kernel, "avg_us": round(avg, 2), "min_us": round(mn, 2),
+                               "median_us": round(med, 2),
                                "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"]}
 
     if wl.flops:
@@ -314,7 +397,14 @@ def main() -> int:
         "config": {"workload": wl.name, "description": wl.description},
         "roofline": roof, "kernels": per_kernel,
         "measured_copy_GBps": round(R.measured_copy_gbps(), 1),
+        "host": cpu_info(),
     }
+    # Ceilings measured on this device in this run: a loop of nothing but the
+    # type's MFMA instruction (random operands; and zeros for s8, which shows
+    # what the power limit costs), beside the published peaks.
+    peaks = {dt: round(R.measured_mfma_peak(dt), 1) for dt in ("s8", "f8", "f16", "bf16", "f32")}
+    peaks["s8_zero_operands"] = round(R.measured_mfma_peak("s8", zeros=True), 1)
+    result["measured_mfma_only_TOPS"] = peaks
 
     if not args.no_cpu and args.workload.startswith("c2_f16_chain"):
         base, cpu_out4, slab = cpu_baseline_c2(wl.keep)
@@ -339,6 +429,7 @@ def main() -> int:
                 total_us += avg
                 entry["kernels"][op.name] = {
                     "kernel": op.kernel, "avg_us": round(avg, 2), "min_us": round(mn, 2),
+                    "median_us": round(med, 2),
                     "bound": r["bound"], "achieved": r["achieved"], "unit": r["unit"],
                     "frac": r["frac"]}
             if w.flops:
@@ -349,9 +440,55 @@ def main() -> int:
                     entry["cpu_baseline"] = cpu_baseline_extra(w)
                 except Exception as e:  # the baseline is a reported aside, never fatal
                     entry["cpu_baseline"] = {"error": repr(e)}
+            if not args.no_cpu and name in TARGET_MMT4D:
+                entry["parity"] = verify_sampled_tiles(w)
+            if name in TARGET_PACK:
+                rows, row_bytes, sp, dp = TARGET_PACK[name]
+                gbps = R.copy2d_ceiling_gbps(rows, row_bytes, sp, dp)
+                entry["copy2d_ceiling"] = {
+                    "GBps": round(gbps, 1), "frac": round(gbps / rn.PEAK_HBM_GBPS, 4),
+                    "what": f"plain copy of {rows} rows x {row_bytes} B, pitch {sp} -> {dp} B"}
+                keep = w.keep
+                entry["parity"] = {"round_trip_bit_exact": bool(
+                    torch.equal(keep["back"].view(keep["rows"], keep["cols"]), keep["x"]))}
             extra[name] = entry
             del w
         result["extra"] = extra
+
+        # ---- targets: compact, last in the line -------------------------------
+        targets = {"_": "frac: of the published peak (s8/f8 5000, f16/bf16 2500 TOP/s, HBM 8000 GB/s); "
+                        "of_mfma_only / of_copy2d: of the ceiling measured in this run"}
+        for name in TARGET_MMT4D:
+            e = extra.get(name)
+            if not e:
+                continue
+            kk = e["kernels"]["mmt4d"]
+            dt = name.split("_")[0] if not name.startswith("c4") else "f8"
+            t = {"kernel": kk["kernel"].replace("mmt4d_mfma_", ""), "us": kk["avg_us"],
+                 "TOPS": round(kk["achieved"], 1), "frac": round(kk["frac"], 3),
+                 "of_mfma_only": round(kk["achieved"] / peaks[dt], 3)}
+            if "parity" in e:
+                par = e["parity"]
+                t["parity"] = ("bit-exact on %d sampled tiles" % par["tiles"] if par.get("bit_exact")
+                               else ("MISMATCH" if "bit_exact" in par else
+                                     par.get("error") or
+                                     "err %.1e <= %g: %s" % (par["max_err_over_max_ref"], par["tolerance"], par["ok"])))
+            cb = e.get("cpu_baseline") or {}
+            if "value" in cb:
+                t["cpu"] = "%.3g %s, %d thr, %s" % (cb["value"], cb["unit"], cb["cores"], cb["kind"])
+            for pk in ("pack_lhs", "pack_rhs"):
+                if pk in e["kernels"]:
+                    t[pk + "_frac"] = round(e["kernels"][pk]["frac"], 3)
+            targets[name] = t
+        for name in TARGET_PACK:
+            e = extra.get(name)
+            if not e:
+                continue
+            targets[name] = {"pack_frac": round(e["kernels"]["pack"]["frac"], 3),
+                             "unpack_frac": round(e["kernels"]["unpack"]["frac"], 3),
+                             "copy2d_frac": round(e["copy2d_ceiling"]["frac"], 3),
+                             "round_trip_bit_exact": e["parity"]["round_trip_bit_exact"]}
+        result["targets"] = targets
 
     R.close()
     print(json.dumps(result))

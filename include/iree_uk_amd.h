@@ -316,7 +316,8 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_pointer_mode(int mode);
  *   MFMA_VARIANT + v : mmt4d takes MFMA workgroup shape v where it can serve
  *             the call (1 = 256x256, 2 = 128x128, 3 = 64x64, 4 = the M-thin
  *             kernels, 5 = the M-thin kernel on the transposed problem,
- *             6 = the 64x64 K-split kernel, 7 = 256x128, 8 = 128x512)
+ *             6 = the 64x64 K-split kernel, 7 = 256x128, 8 = 128x512,
+ *             9 / 10 = the persistent kernel in the 128x512 / 256x256 shape)
  *             instead of choosing by problem size; pack/unpack as AUTO. */
 enum {
   IREE_UK_AMD_KERNEL_MODE_AUTO = 0,
@@ -325,9 +326,54 @@ enum {
 };
 IREE_UK_AMD_EXPORT void iree_uk_amd_set_kernel_mode(int mode);
 
+/* iree_uk_mmt4d_info's bit promises a matrix-core kernel for the tile shape at
+ * every M, N, K, for operands at any element-aligned address, as long as
+ * strides are non-negative and every operand spans less than 2 GiB from its
+ * first panel. Outside those limits the call is still served, with the same
+ * result, by the scalar kernel (64-bit indexing), about 100x slower; this
+ * counts such calls of the calling thread since it started, so a caller (or a
+ * test) can see the cliff. iree_uk_amd_last_kernel_name names the kernel of
+ * the latest call. No counterpart in the reference, whose tile functions take
+ * any stride. */
+IREE_UK_AMD_EXPORT uint64_t iree_uk_amd_mfma_decline_count(void);
+
+/* Tuning / test knob of the calling thread: how many workgroups the
+ * persistent mmt4d kernels launch (each walks its share of the output blocks
+ * with one software pipeline running across block boundaries). 0, the
+ * default, is one workgroup per compute unit. No counterpart in the
+ * reference. */
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_persistent_workgroups(int n);
+
 /* Name of the kernel variant the most recent call on this thread launched
  * ("" if it returned early). Static storage; never NULL. */
 IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_kernel_name(void);
+
+/* Measured ceilings for benchmark reports (no counterpart in the reference,
+ * whose tools/mmt4d_benchmark.c and tools/pack_benchmark.c print rates with
+ * nothing beside them).
+ *
+ * iree_uk_amd_probe_mfma_peak: a loop of nothing but matrix-core instructions
+ * of the element type in `type_flags` (S8S8S32, F16F16F32, BF16BF16F32,
+ * F32F32F32 or the f8 extension), 8 waves per workgroup with the register
+ * blocking of the mmt4d kernels, `workgroups` workgroups (0 = two per compute
+ * unit), `iters` passes over a wave's 32 accumulator blocks. The lanes take
+ * their register operands once from `operands` (`operand_bytes` of device
+ * memory, a multiple of 16): all-zero and random bytes give different clocks
+ * on a power-limited part. `sink`: device memory, one int per thread, never
+ * written in practice. Runs on `stream` (a hipStream_t) and waits for it.
+ * Returns 0 or a hipError_t value; *ops_per_second receives the rate.
+ *
+ * iree_uk_amd_probe_copy2d: `iters` plain copies of `rows` rows of `row_bytes`
+ * bytes between two pitches (everything 4-byte aligned): the ceiling of a
+ * pack / unpack that moves the same matrix between the same pitches.
+ * *seconds_per_copy receives the average. */
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(
+    uint32_t type_flags, const void* operands, int64_t operand_bytes, int iters,
+    int workgroups, void* sink, void* stream, double* ops_per_second);
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(
+    const void* src, int64_t src_pitch, void* dst, int64_t dst_pitch,
+    int64_t row_bytes, int64_t rows, int iters, void* stream,
+    double* seconds_per_copy);
 
 /* Per-kernel device timing for the calling thread. Between begin and end,
  * every kernel an entry point launches carries its own start/stop event pair

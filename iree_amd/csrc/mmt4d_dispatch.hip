@@ -13,6 +13,14 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(
 extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
                                                     int32_t K0, uint32_t flags);
 
+namespace {
+// Calls on this thread that iree_uk_mmt4d_info advertises a matrix-core kernel
+// for but that the scalar kernel served (see iree_uk_amd_mfma_decline_count).
+thread_local uint64_t g_declined = 0;
+}  // namespace
+
+extern "C" IREE_UK_AMD_EXPORT uint64_t iree_uk_amd_mfma_decline_count(void) { return g_declined; }
+
 extern "C" int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0,
                                                      int32_t K0,
                                                      uint32_t flags) {
@@ -32,8 +40,12 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
                            ? kernel_mode - IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT
                            : 0;
     int st = iree_uk_amd_hip_launch_mmt4d_mfma(p, rowmajor, stream, forced, kernel_name);
-    // A negative status means "shape not served after all"; fall through.
+    // A negative status means "not served after all" (a negative stride, an
+    // operand spanning 2 GiB or more, a zero-fill): the scalar kernel, which
+    // indexes with 64 bits, computes the same result. When the tile shape is
+    // one the info query advertises, count the call so that the cliff shows.
     if (st >= 0) return st;
+    if (!maybe && kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO && p->K != 0) ++g_declined;
   }
   *kernel_name = "mmt4d_generic";
   return iree_uk_amd_hip_launch_mmt4d_generic(p, rowmajor, stream);

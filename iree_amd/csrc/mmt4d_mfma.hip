@@ -17,6 +17,18 @@ int launch_s8s4(const Problem& p, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 
 namespace {
+thread_local int g_persistent_workgroups = 0;
+}  // namespace
+
+namespace uk_mfma {
+int persistent_workgroups_override() { return g_persistent_workgroups; }
+}  // namespace uk_mfma
+
+extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_persistent_workgroups(int n) {
+  g_persistent_workgroups = n > 0 ? n : 0;
+}
+
+namespace {
 
 using uk_mfma::Elem;
 
@@ -67,7 +79,7 @@ extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
 }
 
 // Returns a HIP status (>= 0), or -1 when the call is not served after all
-// (operands not 16-byte aligned, spans beyond 2 GiB, ...).
+// (negative strides, spans beyond 2 GiB, ...).
 extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p,
                                                  const iree_uk_amd_rowmajor_out_t* rowmajor,
                                                  void* stream_v, int forced_variant,
@@ -137,10 +149,9 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
       pr.acc_stride < 0) {
     return -1;
   }
-  // 16-byte vector loads need 16-byte aligned panels (8-byte loads of 4-bit
-  // rows: 8-byte aligned).
-  if (((uintptr_t)pr.lhs | (uint64_t)pr.lhs_stride) & 15) return -1;
-  if (((uintptr_t)pr.rhs | (uint64_t)pr.rhs_stride) & (s8s4 ? 7 : 15)) return -1;
+  // Operands need no alignment beyond their element's: the kernels read them
+  // with vector loads that take any address (v4i_g in the kernel header).
+  if (((uintptr_t)pr.lhs | (uintptr_t)pr.rhs) & (uintptr_t)(s8s4 ? 0 : eb - 1)) return -1;
   if ((uintptr_t)pr.out & (uintptr_t)(ob - 1)) return -1;
   pr.M1 = (int32_t)p->M;
   pr.N1 = (int32_t)p->N;

@@ -53,6 +53,11 @@
 namespace uk_mfma {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+// Operand pieces as they are read from global memory: no alignment beyond the
+// element's is asked of the caller's buffers. The HSA ABI runs the memory
+// pipeline in its unaligned mode, in which a 16-byte global load takes any
+// address (the compiler itself emits one global_load_dwordx4 for this type).
+typedef v4i v4i_g __attribute__((aligned(1)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -212,6 +217,8 @@ struct Args {
   // the caller's order of the two multiplications).
   uint32_t out_sn0, acc_sn0;
   uint32_t col_scale_first;
+  // mmt4d_mfma_persistent.h only: log2 of M0 and N0 (powers of two there).
+  int32_t lm0, ln0;
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that
@@ -491,7 +498,7 @@ void mmt4d_mfma_kernel(Args a) {
   // only ever reaches accumulator rows or columns that are never stored.
   // `tail` marks the one step in which K-tiles past K1 must read as zero.
   auto load_piece = [&](int i, uint32_t off) {
-    return *reinterpret_cast<const v4i*>(sbase[i] + off);
+    return *reinterpret_cast<const v4i_g*>(sbase[i] + off);
   };
   auto load_global = [&](v4i (&dst)[NU][R], int step, bool tail) {
 #pragma unroll
@@ -737,7 +744,7 @@ void mmt4d_mfma_kernel(Args a) {
     auto load_b = [&](v4i (&dst)[HALVES], int tn, int step) {
 #pragma unroll
       for (int h = 0; h < HALVES; ++h)
-        dst[h] = *reinterpret_cast<const v4i*>(sbase_b + (voff_b[tn][h] + (uint32_t)step * sstep_b));
+        dst[h] = *reinterpret_cast<const v4i_g*>(sbase_b + (voff_b[tn][h] + (uint32_t)step * sstep_b));
     };
     auto read_a = [&](v4i (&dst)[HALVES], uint32_t stage_off, int tm) {
 #pragma unroll
@@ -836,7 +843,7 @@ void mmt4d_mfma_kernel(Args a) {
     auto load_b = [&](v4i (&dst)[HALVES], int tn, int step) {
 #pragma unroll
       for (int h = 0; h < HALVES; ++h)
-        dst[h] = *reinterpret_cast<const v4i*>(sbase_b + (voff_b[tn][h] + (uint32_t)step * sstep_b));
+        dst[h] = *reinterpret_cast<const v4i_g*>(sbase_b + (voff_b[tn][h] + (uint32_t)step * sstep_b));
     };
     auto read_a = [&](v4i (&dst)[HALVES], uint32_t stage_off, int tm) {
 #pragma unroll

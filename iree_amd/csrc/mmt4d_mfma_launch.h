@@ -10,6 +10,7 @@
 #include <climits>
 
 #include "mmt4d_mfma_kernel.h"
+#include "mmt4d_mfma_persistent.h"
 #include "mmt4d_mfma_thin.h"
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
@@ -131,6 +132,83 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   return (int)hipGetLastError();
 }
 
+// Workgroup count set with iree_uk_amd_set_persistent_workgroups on this
+// thread; 0 = one per compute unit (defined in mmt4d_mfma.hip).
+int persistent_workgroups_override();
+
+// Compute units of the current device (one persistent workgroup each).
+inline int compute_units() {
+  static thread_local int cached_device = -1, cached_cus = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev != cached_device) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached_device = dev;
+    cached_cus = cus;
+  }
+  return cached_cus;
+}
+
+// Launches the persistent kernel (mmt4d_mfma_persistent.h) over K-tiles
+// [0, kt_count): one workgroup per CU, each walking several output blocks
+// without draining its pipeline in between. Returns a HIP status, or -1 if
+// the kernel cannot serve the shape (or would not gain: fewer than two blocks
+// per workgroup).
+template <Elem E, int TM, int TN, int WGM, int WGN>
+int launch_persistent(const Problem& p, int kt_count, bool force, hipStream_t stream) {
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16, KS = 64;
+  auto pow2 = [](int v) { return v > 0 && (v & (v - 1)) == 0; };
+  if (p.rb < 16 || p.rb > KS) return -1;
+  if (!pow2(p.M0) || !pow2(p.N0) || p.N0 < 4 || p.M0 > BM || p.N0 > BN) return -1;
+  if (p.dequant) return -1;
+  const int bpm = BM / p.M0, bpn = BN / p.N0;
+  if (p.M1 % bpm || p.N1 % bpn) return -1;
+  if (p.out_rows < (int64_t)p.M1 * p.M0 || p.out_cols < (int64_t)p.N1 * p.N0) return -1;
+  const int64_t k_bytes = (int64_t)kt_count << p.lrb;
+  if (k_bytes % (4 * KS) || k_bytes / KS < 8 || k_bytes / KS >= (1 << 24)) return -1;
+  const int64_t grid_m = p.M1 / bpm, grid_n = p.N1 / bpn;
+  const int64_t total = grid_m * grid_n;
+  int cus = compute_units() & ~7;  // a multiple of the 8 XCDs keeps blocks on their XCD
+  if (persistent_workgroups_override() > 0) cus = persistent_workgroups_override();
+  if (cus < 1 || total >= (1ll << 30)) return -1;
+  if (!force && total < 2 * (int64_t)cus) return -1;
+  const int64_t grid = std::min<int64_t>(total, cus);
+  Args a{};
+  a.lhs = p.lhs; a.rhs = p.rhs; a.out = p.out;
+  a.lhs_stride = p.lhs_stride; a.rhs_stride = p.rhs_stride; a.out_stride = p.out_stride;
+  a.out_sm0 = (uint32_t)p.out_sm0; a.out_spn = (uint32_t)p.out_spn;
+  a.out_rows = (int32_t)std::min<int64_t>(p.out_rows, INT32_MAX);
+  a.out_cols = (int32_t)std::min<int64_t>(p.out_cols, INT32_MAX);
+  a.M1 = p.M1; a.N1 = p.N1; a.K1 = kt_count;
+  a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
+  a.bpm = bpm; a.bpn = bpn;
+  a.grid_m = (int32_t)grid_m; a.grid_n = (int32_t)grid_n;
+  a.steps = (int32_t)(k_bytes / KS);
+  a.accumulate = p.accumulate;
+  a.band = (WGM == 1 && WGN == 8) ? 8 : 4;
+  a.vec_out = 1;
+  a.acc = p.acc; a.acc_stride = p.acc_stride;
+  a.acc_sm0 = (uint32_t)p.acc_sm0; a.acc_spn = (uint32_t)p.acc_spn;
+  while ((1 << a.lm0) < p.M0) ++a.lm0;
+  while ((1 << a.ln0) < p.N0) ++a.ln0;
+  const int64_t kt_bytes_m = (int64_t)p.M0 << p.lrb, kt_bytes_n = (int64_t)p.N0 << p.lrb;
+  const int64_t span_m = (int64_t)bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
+  const int64_t span_n = (int64_t)bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
+  const int64_t span_o = (int64_t)bpm * p.out_stride + (int64_t)p.M0 * p.out_sm0 +
+                         (int64_t)p.N1 * p.out_spn;
+  const int64_t span_a = (int64_t)bpm * p.acc_stride + (int64_t)p.M0 * p.acc_sm0 +
+                         (int64_t)p.N1 * p.acc_spn;
+  if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31) ||
+      span_a >= (1ll << 31)) {
+    return -1;
+  }
+  constexpr size_t kLds = 4 * (size_t)BM * KS;
+  auto kernel = mmt4d_mfma_persistent_kernel<E, TM, TN, WGM, WGN>;
+  uk::launch(2, kernel, dim3((uint32_t)grid), dim3(WGM * WGN * 64), kLds, stream, a);
+  return (int)hipGetLastError();
+}
+
 // Launches the M-thin kernel (mmt4d_mfma_thin.h) over all of K. Returns a HIP
 // status, or -1 if it cannot serve the shape.
 // `swapped`: the caller's problem is N-thin and is computed as its transpose
@@ -205,6 +283,12 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+// Status of the second, accumulating launch over the remainder of K. The
+// first launch has already written the output: "not served" (negative) must
+// not reach the dispatcher, which would recompute the whole problem on the
+// scalar kernel on top of it.
+inline int finish_k(int st) { return st < 0 ? (int)hipErrorUnknown : st; }
+
 // Number of workgroups a BM x BN blocking gives for the problem.
 inline int64_t workgroups(const Problem& p, int BM, int BN) {
   const int bpm = BM / p.M0, bpn = BN / p.N0;
@@ -220,7 +304,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //   small 64x64, 4 waves, any K: for problems with too few 128x128 blocks to
 //         occupy the 256 CUs;
 // `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem,
-// 6 the 64x64 K-split kernel, 7 the 256x128 shape, 8 the 128x512 shape;
+// 6 the 64x64 K-split kernel, 7 the 256x128 shape, 8 the 128x512 shape,
+// 9 / 10 the persistent kernel in the 128x512 / 256x256 shape;
 // 0 = choose) overrides the
 // size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
@@ -239,8 +324,11 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced == 8) {
-    choice = 1;  // the big variant in its 128x512 shape (square where that one cannot serve)
+  if (forced >= 8 && forced <= 10) {
+    // The big variant in its 128x512 shape (8), the persistent kernel in that
+    // shape (9) or in the square one (10); the plain square shape where the
+    // requested one cannot serve.
+    choice = 1;
   } else if (forced >= 1 && forced <= 7) {
     choice = forced;
   } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
@@ -337,6 +425,23 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     if (kt_main > 0) {
       int st = -1;
       bool wide = false;
+      if constexpr (RBC >= 16 && H == 1 && ElemTraits<E>::Out::kOutBytes == 4) {
+        // Several rounds of blocks: one persistent workgroup per CU whose
+        // pipeline runs across block boundaries.
+        if (forced == 0 || forced == 9) {
+          st = launch_persistent<E, 8, 4, 1, 8>(p, kt_main, forced == 9, stream);
+          if (st == 0) *name = "mmt4d_mfma_128x512_persistent";
+        }
+        if (st < 0 && (forced == 0 || forced == 10)) {
+          st = launch_persistent<E, 8, 4, 2, 4>(p, kt_main, forced == 10, stream);
+          if (st == 0) *name = "mmt4d_mfma_256x256_persistent";
+        }
+        if (st == 0) {
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
       if constexpr (RBC >= 16) {
         // 128 rows x 512 columns, the 8 waves side by side (each 128x64): no two
         // waves load the same RHS fragments and the LDS holds half as much LHS,
@@ -358,7 +463,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         *name = wide ? "mmt4d_mfma_128x512_rhs_direct"
                      : (RBC >= 16 ? "mmt4d_mfma_256x256_rhs_direct" : "mmt4d_mfma_256x256_regroup");
         if (kt_main == p.K1) return 0;
-        return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+        return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
       }
       if (st > 0) return st;
     }
@@ -374,7 +479,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         if (st == 0) {
           *name = "mmt4d_mfma_256x128_rhs_direct";
           if (kt_main == p.K1) return 0;
-          return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
         }
         if (st > 0) return st;
       }
@@ -437,7 +542,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         if (st == 0) {
           *name = "mmt4d_mfma_128x128_rhs_direct";
           if (kt_main == p.K1) return 0;
-          return launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
         }
         if (st > 0) return st;
       }
@@ -451,7 +556,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
       if (st == 0) {
         *name = "mmt4d_mfma_64x64_rhs_direct";
         if (kt_main == p.K1) return 0;
-        return launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream);
+        return finish_k(launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
       }
       if (st > 0) return st;
     }

@@ -41,6 +41,7 @@
 namespace uk_mfma {
 
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef v2i v2i_g __attribute__((aligned(1)));  // as v4i_g: read from global memory at any address
 
 template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
 __global__ __launch_bounds__(KSPLIT * 64)
@@ -111,10 +112,10 @@ void mmt4d_thin_kernel(Args a) {
 
   auto load_operand = [&](const char* base, const uint32_t (&off)[PIECES], uint32_t adv) {
     if constexpr (RBC >= 16) {
-      return *reinterpret_cast<const v4i*>(base + (off[0] + adv));
+      return *reinterpret_cast<const v4i_g*>(base + (off[0] + adv));
     } else {
-      const v2i lo = *reinterpret_cast<const v2i*>(base + (off[0] + adv));
-      const v2i hi = *reinterpret_cast<const v2i*>(base + (off[1] + adv));
+      const v2i lo = *reinterpret_cast<const v2i_g*>(base + (off[0] + adv));
+      const v2i hi = *reinterpret_cast<const v2i_g*>(base + (off[1] + adv));
       return v4i{lo[0], lo[1], hi[0], hi[1]};
     }
   };
@@ -129,7 +130,7 @@ void mmt4d_thin_kernel(Args a) {
 #pragma unroll
       for (int h = 0; h < HALVES; ++h) {
         if constexpr (S4) {
-          fb[d][tn][h] = *reinterpret_cast<const v2i*>(base_b + (offb[tn][h][0] + s * sstep_b));
+          fb[d][tn][h] = *reinterpret_cast<const v2i_g*>(base_b + (offb[tn][h][0] + s * sstep_b));
         } else {
           fb[d][tn][h] = load_operand(base_b, offb[tn][h], s * sstep_b);
         }

@@ -1,0 +1,209 @@
+// Measured ceilings for the runner: what the matrix cores and the memory
+// system of the device at hand sustain when nothing else is in the way. The
+// benchmark reports its kernels against these next to the published peaks.
+//
+//   iree_uk_amd_probe_mfma_peak   a loop of nothing but MFMAs, 8 waves per CU
+//                                 with the register blocking of the mmt4d
+//                                 kernels (8 x 4 accumulator blocks per wave),
+//                                 operands held in registers: no memory traffic
+//   iree_uk_amd_probe_copy2d      a plain 2-D copy between two pitches (the
+//                                 traffic of a pack / unpack without the
+//                                 transposition)
+//
+// Counterpart in the reference: none; its benchmarks
+// (runtime/src/iree/builtins/ukernel/tools/mmt4d_benchmark.c:82-84,
+// tools/pack_benchmark.c:97-101) report rates without a ceiling beside them.
+#include <hip/hip_runtime.h>
+
+#include "mmt4d_mfma_kernel.h"
+#include "uk_hip_abi.h"
+
+namespace {
+
+using uk_mfma::Elem;
+using uk_mfma::ElemTraits;
+using uk_mfma::v4i;
+
+constexpr int kTM = 8, kTN = 4, kWaves = 8;
+
+template <Elem E>
+__global__ __launch_bounds__(kWaves * 64) void mfma_peak_kernel(const v4i* operands, int n_operands,
+                                                               int iters, int* sink) {
+  using TT = ElemTraits<E>;
+  using Acc = typename TT::Acc;
+  constexpr int H = TT::kHalves;
+  v4i fa[kTM][H], fb[kTN][H];
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < kTM; ++i)
+#pragma unroll
+    for (int h = 0; h < H; ++h) fa[i][h] = operands[(t * 31u + (uint32_t)(i * H + h) * 977u) % (uint32_t)n_operands];
+#pragma unroll
+  for (int i = 0; i < kTN; ++i)
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+      fb[i][h] = operands[(t * 17u + 7919u + (uint32_t)(i * H + h) * 613u) % (uint32_t)n_operands];
+  Acc acc[kTM][kTN];
+#pragma unroll
+  for (int i = 0; i < kTM; ++i)
+#pragma unroll
+    for (int j = 0; j < kTN; ++j) acc[i][j] = Acc{0, 0, 0, 0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < kTM; ++i)
+#pragma unroll
+      for (int j = 0; j < kTN; ++j) acc[i][j] = TT::mfma(fb[j], fa[i], acc[i][j]);
+  }
+  // Keep the accumulators alive without writing anything in practice.
+  Acc s = acc[0][0];
+#pragma unroll
+  for (int i = 0; i < kTM; ++i)
+#pragma unroll
+    for (int j = 0; j < kTN; ++j)
+      if (i || j) s = s + acc[i][j];
+  const v4i bits = __builtin_bit_cast(v4i, s);
+  if ((bits[0] ^ bits[1] ^ bits[2] ^ bits[3]) == 0x5a17c0de && iters < 0) sink[t] = bits[0];
+}
+
+// K elements per MFMA instruction group issued by ElemTraits<E>::mfma.
+template <Elem E> constexpr int k_per_mfma() {
+  return E == Elem::kS8 ? 64 : E == Elem::kF8 ? 128 : E == Elem::kF32 ? 16 : 32;
+}
+
+template <Elem E>
+int run_mfma_peak(const v4i* operands, int n_operands, int iters, int workgroups, int* sink,
+                  hipStream_t stream, double* ops) {
+  hipLaunchKernelGGL(mfma_peak_kernel<E>, dim3(workgroups), dim3(kWaves * 64), 0, stream, operands,
+                     n_operands, iters, sink);
+  *ops = 2.0 * 16 * 16 * k_per_mfma<E>() * kTM * kTN * (double)iters * kWaves * workgroups;
+  return (int)hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void copy2d_kernel(const char* src, int64_t src_pitch, char* dst,
+                                                     int64_t dst_pitch, int64_t row_bytes,
+                                                     int64_t rows) {
+  // A workgroup copies 4 KiB pieces of rows (16 bytes per lane, 4-byte
+  // aligned like the pack kernels' 2-D side), walking pieces grid-stride.
+  typedef uk_mfma::v4i v4i_a4 __attribute__((aligned(4)));
+  const int64_t pieces_per_row = (row_bytes + 4095) / 4096;
+  const int64_t total = pieces_per_row * rows;
+  for (int64_t p = blockIdx.x; p < total; p += gridDim.x) {
+    const int64_t row = p / pieces_per_row, piece = p - row * pieces_per_row;
+    const int64_t off = piece * 4096 + (int64_t)threadIdx.x * 16;
+    if (off + 16 <= row_bytes) {
+      *reinterpret_cast<v4i_a4*>(dst + row * dst_pitch + off) =
+          *reinterpret_cast<const v4i_a4*>(src + row * src_pitch + off);
+    } else {
+      for (int64_t b = off; b < row_bytes && b < off + 16; b += 4)
+        *reinterpret_cast<int*>(dst + row * dst_pitch + b) =
+            *reinterpret_cast<const int*>(src + row * src_pitch + b);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// Runs the MFMA-only loop of the element type in `type_flags` (an
+// IREE_UK_FLAG_MMT4D_TYPE_* value: S8S8S32, F16F16F32, BF16BF16F32, F32F32F32
+// or the f8 extension) on `stream`: `workgroups` workgroups of 8 waves (0 = two
+// per compute unit), `iters` passes over the 32 accumulator blocks of a wave.
+// `operands` points to `operand_bytes` (a multiple of 16, at least 16) of
+// device memory from which the lanes take their register operands once;
+// all-zero bytes and random bytes give different clocks on a power-limited
+// part. `sink` is device memory for one int per thread that is never written
+// in practice. Returns 0 and the operations per second in *ops_per_second.
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(uint32_t type_flags, const void* operands,
+                                                   int64_t operand_bytes, int iters,
+                                                   int workgroups, void* sink, void* stream_v,
+                                                   double* ops_per_second) {
+  hipStream_t stream = (hipStream_t)stream_v;
+  if (!operands || operand_bytes < 16 || iters < 1 || !sink || !ops_per_second) return (int)hipErrorInvalidValue;
+  if (workgroups <= 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+      return (int)hipErrorUnknown;
+    }
+    workgroups = 2 * cus;
+  }
+  const v4i* ops_ptr = (const v4i*)operands;
+  const int n = (int)(operand_bytes / 16);
+  hipEvent_t start, stop;
+  if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return (int)hipErrorUnknown;
+  double ops = 0;
+  int st = 0;
+  auto run = [&](int it) {
+    switch (type_flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
+      case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32:
+        return run_mfma_peak<Elem::kS8>(ops_ptr, n, it, workgroups, (int*)sink, stream, &ops);
+      case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32:
+        return run_mfma_peak<Elem::kF16>(ops_ptr, n, it, workgroups, (int*)sink, stream, &ops);
+      case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32:
+        return run_mfma_peak<Elem::kBF16>(ops_ptr, n, it, workgroups, (int*)sink, stream, &ops);
+      case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32:
+        return run_mfma_peak<Elem::kF32>(ops_ptr, n, it, workgroups, (int*)sink, stream, &ops);
+      case IREE_UK_AMD_FLAG_MMT4D_TYPE_F8E4M3FNF8E4M3FNF32:
+        return run_mfma_peak<Elem::kF8>(ops_ptr, n, it, workgroups, (int*)sink, stream, &ops);
+      default:
+        return (int)hipErrorInvalidValue;
+    }
+  };
+  st = run(iters / 8 + 1);  // warm-up
+  if (st == 0) st = (int)hipEventRecord(start, stream);
+  if (st == 0) st = run(iters);
+  if (st == 0) st = (int)hipEventRecord(stop, stream);
+  if (st == 0) st = (int)hipEventSynchronize(stop);
+  float ms = 0.f;
+  if (st == 0) st = (int)hipEventElapsedTime(&ms, start, stop);
+  (void)hipEventDestroy(start);
+  (void)hipEventDestroy(stop);
+  if (st != 0) return st;
+  *ops_per_second = ops / ((double)ms * 1e-3);
+  return 0;
+}
+
+// Copies `rows` rows of `row_bytes` bytes (a multiple of 4) from `src` (rows
+// `src_pitch` bytes apart) to `dst` (`dst_pitch`) `iters` times on `stream`
+// and returns the average seconds per copy: the ceiling of a pack / unpack
+// that moves the same matrix between the same two pitches. All pointers and
+// pitches 4-byte aligned.
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(const void* src, int64_t src_pitch, void* dst,
+                                                int64_t dst_pitch, int64_t row_bytes,
+                                                int64_t rows, int iters, void* stream_v,
+                                                double* seconds_per_copy) {
+  hipStream_t stream = (hipStream_t)stream_v;
+  if (!src || !dst || !seconds_per_copy || iters < 1 || row_bytes < 4 || (row_bytes & 3) || rows < 1 ||
+      (((uintptr_t)src | (uintptr_t)dst | (uint64_t)src_pitch | (uint64_t)dst_pitch) & 3)) {
+    return (int)hipErrorInvalidValue;
+  }
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    return (int)hipErrorUnknown;
+  }
+  const int grid = cus * 8;
+  hipEvent_t start, stop;
+  if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return (int)hipErrorUnknown;
+  auto run = [&]() {
+    hipLaunchKernelGGL(copy2d_kernel, dim3(grid), dim3(256), 0, stream, (const char*)src, src_pitch,
+                       (char*)dst, dst_pitch, row_bytes, rows);
+  };
+  run();
+  run();
+  int st = (int)hipEventRecord(start, stream);
+  for (int i = 0; i < iters; ++i) run();
+  if (st == 0) st = (int)hipGetLastError();
+  if (st == 0) st = (int)hipEventRecord(stop, stream);
+  if (st == 0) st = (int)hipEventSynchronize(stop);
+  float ms = 0.f;
+  if (st == 0) st = (int)hipEventElapsedTime(&ms, start, stop);
+  (void)hipEventDestroy(start);
+  (void)hipEventDestroy(stop);
+  if (st != 0) return st;
+  *seconds_per_copy = (double)ms * 1e-3 / iters;
+  return 0;
+}
+
+}  // extern "C"

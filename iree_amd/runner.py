@@ -161,6 +161,15 @@ class Runner:
 
     # --------------------------------------------------------------- workloads
     def workload(self, name: str) -> Workload:
+        """Builds the named workload. Its tensors are generated by torch on
+        torch's current stream while the ops launch on the runner's own: the
+        device is synchronized before the workload is handed out, so a first
+        launch never reads an operand that is still being generated."""
+        wl = self._build_workload(name)
+        self.torch.cuda.synchronize()
+        return wl
+
+    def _build_workload(self, name: str) -> Workload:
         torch = self.torch
         if name in ("c2_f16_chain_4096", "c2_f16_chain_ragged"):
             M, N, K = (4096, 4096, 4096) if name.endswith("4096") else (4095, 4097, 4096)
@@ -319,7 +328,7 @@ class Runner:
             # The same layer through the fused entry point: accumulators read
             # from the tiled s32 buffer, result scaled into the row-major f32
             # matrix by the mmt4d kernel itself (no separate epilogue pass).
-            base = self.workload("c3_s8_decode")
+            base = self._build_workload("c3_s8_decode")
             t = base.keep
             Mlog, N = t["act"].shape[0], t["w"].shape[0]
             M1, N1, K1, M0, N0, K0 = (t[k] for k in ("M1", "N1", "K1", "M0", "N0", "K0"))
@@ -509,6 +518,57 @@ class Runner:
         n_kind = sum(1 for op in wl.ops if self.KIND.get(op.name.split("_")[0], -1) == dom_kind)
         dom_us = dom_total / (steps * max(1, n_kind if n_dom == 0 else n_kind)) if recs else math.nan
         return (t1 - t0) / steps, (t3 - t2) / steps, dom_us
+
+    MMT4D_TYPE = {"s8": uk.MMT4D_TYPE_S8S8S32, "f16": uk.MMT4D_TYPE_F16F16F32,
+                  "bf16": uk.MMT4D_TYPE_BF16BF16F32, "f32": uk.MMT4D_TYPE_F32F32F32,
+                  "f8": uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32}
+
+    def measured_mfma_peak(self, dtype: str, zeros: bool = False, seconds: float = 0.02) -> float:
+        """TOP/s (TFLOP/s) of a loop of nothing but this type's MFMA
+        instruction with the mmt4d kernels' register blocking, 8 waves per CU,
+        register operands taken from random bytes of the type's value range (or
+        zeros): the ceiling the matrix cores hold on this device at the clock
+        its power limit allows, before a single operand is moved. Runs about
+        `seconds` after a settle phase of the same loop."""
+        torch = self.torch
+        n = 1 << 16
+        if zeros:
+            operands = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        elif dtype == "s8":
+            operands = self.uniform_s8((n,), 901).view(torch.uint8)
+        elif dtype == "f8":
+            operands = self.normal_f8((n,), 902)
+        elif dtype == "f32":
+            operands = self.normal((n // 4,), torch.float32, 903).view(torch.uint8)
+        else:
+            operands = self.normal((n // 2,), torch.float16 if dtype == "f16" else torch.bfloat16,
+                                   904).view(torch.uint8)
+        sink = torch.zeros(4 * 512 * 1024, dtype=torch.int32, device="cuda")
+        st = self.stream.cuda_stream
+        tf = self.MMT4D_TYPE[dtype]
+        self.stream.synchronize()
+        # Size the loop from a short run, then let the clocks settle under it.
+        rate = self.lib.probe_mfma_peak(tf, operands.data_ptr(), n, 2000, sink.data_ptr(), st)
+        per_iter = 2.0 * 16 * 16 * {"s8": 64, "f8": 128, "f32": 16}.get(dtype, 32) * 32 * 8 * 512
+        iters = max(1000, int(rate * seconds / per_iter))
+        best = 0.0
+        for _ in range(4):
+            best = max(best, self.lib.probe_mfma_peak(tf, operands.data_ptr(), n, iters,
+                                                      sink.data_ptr(), st))
+        return best / 1e12
+
+    def copy2d_ceiling_gbps(self, rows: int, row_bytes: int, src_pitch: int, dst_pitch: int,
+                            iters: int = 10) -> float:
+        """GB/s (read + write) of a plain copy of rows x row_bytes between the
+        two pitches: what a pack / unpack of that matrix could reach if the
+        transposition were free."""
+        torch = self.torch
+        src = torch.empty(rows * src_pitch, dtype=torch.uint8, device="cuda")
+        dst = torch.empty(rows * dst_pitch, dtype=torch.uint8, device="cuda")
+        self.stream.synchronize()
+        sec = self.lib.probe_copy2d(src.data_ptr(), src_pitch, dst.data_ptr(), dst_pitch, row_bytes,
+                                    rows, iters, self.stream.cuda_stream)
+        return 2.0 * rows * row_bytes / sec / 1e9
 
     def measured_copy_gbps(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """Device-to-device copy rate (read + write bytes), for a measured HBM

@@ -53,7 +53,7 @@ POINTER_MODE_AUTO = 0
 POINTER_MODE_DEVICE = 1
 KERNEL_MODE_AUTO = 0
 KERNEL_MODE_GENERIC = 1
-KERNEL_MODE_MFMA_VARIANT = 16  # + 1..8: force an mmt4d MFMA workgroup shape
+KERNEL_MODE_MFMA_VARIANT = 16  # + 1..10: force an mmt4d MFMA workgroup shape
 
 # (lhs bits, rhs bits, out bits) per mmt4d type value.
 MMT4D_TYPE_BITS = {
@@ -158,12 +158,21 @@ class UKernelLibrary:
         L.iree_uk_amd_synchronize.restype = ctypes.c_int
         L.iree_uk_amd_set_pointer_mode.argtypes = [ctypes.c_int]
         L.iree_uk_amd_set_kernel_mode.argtypes = [ctypes.c_int]
+        L.iree_uk_amd_set_persistent_workgroups.argtypes = [ctypes.c_int]
+        L.iree_uk_amd_set_persistent_workgroups.restype = None
         L.iree_uk_amd_device_count.restype = ctypes.c_int
+        L.iree_uk_amd_mfma_decline_count.restype = ctypes.c_uint64
         L.iree_uk_amd_version.restype = ctypes.c_char_p
         L.iree_uk_amd_set_assert_handler.argtypes = [_vp]
         L.iree_uk_amd_timing_begin.restype = None
         L.iree_uk_amd_timing_end.argtypes = [_vp, _vp, ctypes.c_int]
         L.iree_uk_amd_timing_end.restype = ctypes.c_int
+        L.iree_uk_amd_probe_mfma_peak.argtypes = [_u32, _vp, _i64, ctypes.c_int, ctypes.c_int, _vp,
+                                                  _vp, ctypes.POINTER(ctypes.c_double)]
+        L.iree_uk_amd_probe_mfma_peak.restype = ctypes.c_int
+        L.iree_uk_amd_probe_copy2d.argtypes = [_vp, _i64, _vp, _i64, _i64, _i64, ctypes.c_int, _vp,
+                                               ctypes.POINTER(ctypes.c_double)]
+        L.iree_uk_amd_probe_copy2d.restype = ctypes.c_int
         self._handler_ref = None
         self._violations: list[str] = []
 
@@ -232,6 +241,26 @@ class UKernelLibrary:
                                     stride_w, flags, cpu_data)
         self._check()
 
+    # ---------------------------------------------------------------- probes
+    def probe_mfma_peak(self, type_flags, operands, operand_bytes, iters, sink, stream,
+                        workgroups=0) -> float:
+        """Operations per second of an MFMA-only loop (see the header)."""
+        rate = ctypes.c_double(0.0)
+        st = self.lib.iree_uk_amd_probe_mfma_peak(type_flags, operands, operand_bytes, iters,
+                                                  workgroups, sink, stream, ctypes.byref(rate))
+        if st != 0:
+            raise RuntimeError(f"iree_uk_amd_probe_mfma_peak: status {st}")
+        return rate.value
+
+    def probe_copy2d(self, src, src_pitch, dst, dst_pitch, row_bytes, rows, iters, stream) -> float:
+        """Average seconds per plain 2-D copy between two pitches."""
+        sec = ctypes.c_double(0.0)
+        st = self.lib.iree_uk_amd_probe_copy2d(src, src_pitch, dst, dst_pitch, row_bytes, rows,
+                                               iters, stream, ctypes.byref(sec))
+        if st != 0:
+            raise RuntimeError(f"iree_uk_amd_probe_copy2d: status {st}")
+        return sec.value
+
     # --------------------------------------------------------------- control
     def _check(self):
         if self._violations:
@@ -273,6 +302,16 @@ class UKernelLibrary:
 
     def set_kernel_mode(self, mode: int):
         self.lib.iree_uk_amd_set_kernel_mode(mode)
+
+    def mfma_decline_count(self) -> int:
+        """Calls of this thread that the info query advertises an MFMA kernel
+        for but that the scalar kernel served."""
+        return int(self.lib.iree_uk_amd_mfma_decline_count())
+
+    def set_persistent_workgroups(self, n: int):
+        """Workgroups the persistent mmt4d kernels launch on this thread
+        (0 = one per compute unit)."""
+        self.lib.iree_uk_amd_set_persistent_workgroups(n)
 
     def last_kernel_name(self) -> str:
         return self.lib.iree_uk_amd_last_kernel_name().decode()

@@ -88,13 +88,24 @@ def _mfma_shapes(M0, N0, K0, bits):
 # 5 is the thin kernel on the transposed problem and 6 the same kernel with
 # 64x64 blocks, under the same conditions; 7 is the 256x128 shape, 8 the
 # 128x512 shape).
+# Tile rows of one byte (s8, K0 = 1) have no MFMA kernel: iree_uk_mmt4d_info
+# says so and the reference grid above covers them on the scalar kernel. The
+# entry stays in the list, named for what it is, and is asserted unserved.
+def _tile_id(n):
+    tf, M0, N0, K0 = MFMA_TILES[n]
+    name = f"{n}-type{tf:#x}_{M0}x{N0}x{K0}"
+    return name + "_one_byte_rows_have_no_mfma_kernel" if (tf, K0) == (uk.MMT4D_TYPE_S8S8S32, 1) else name
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
-@pytest.mark.parametrize("n", range(len(MFMA_TILES)))
+@pytest.mark.parametrize("n", range(len(MFMA_TILES)), ids=_tile_id)
 def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu
     tf, M0, N0, K0 = MFMA_TILES[n]
-    if not lib.mmt4d_info(M0, N0, K0, tf):
-        pytest.skip("no MFMA kernel for this tile shape; covered by the generic kernel")
+    if (tf, K0) == (uk.MMT4D_TYPE_S8S8S32, 1):
+        assert not lib.mmt4d_info(M0, N0, K0, tf)
+        return
+    assert lib.mmt4d_info(M0, N0, K0, tf)
     lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
     bits = uk.MMT4D_TYPE_BITS[tf][0]
     # Loose strides and offsets in steps of 16 elements: the MFMA kernels need
@@ -375,3 +386,94 @@ def test_fused_mmt4d_unpack_with_remainder_strips(gpu, accumulate):
     b = rhs.permute(0, 2, 1, 3).reshape(N1 * N0, K1 * K0)[:cols].cpu().numpy().astype(np.int64)
     ref = a @ b.T + (init[rows - 40:].cpu().numpy() if accumulate else 0)
     assert np.array_equal(got[rows - 40:].cpu().numpy(), ref.astype(np.int32))
+
+
+# The persistent kernels (one workgroup walks several output blocks with its
+# software pipeline running across block boundaries). Forced, with the number
+# of workgroups capped so that every workgroup owns several blocks even on
+# these small problems: block counts that divide evenly over the workgroups
+# and ones that do not, K of 8 steps (the minimum) and more, ACCUMULATE on and
+# off (the case grid), tiles of 16 and 32 rows. Shapes are tile counts for
+# (M0, N0, K0) so that rows/columns are whole 128x512 and 256x256 blocks.
+@pytest.mark.parametrize("variant", [9, 10])
+@pytest.mark.parametrize("tile", [(uk.MMT4D_TYPE_S8S8S32, 16, 16, 16, (512, 1024, 512)),
+                                  (uk.MMT4D_TYPE_S8S8S32, 16, 16, 64, (512, 1536, 768)),
+                                  (uk.MMT4D_TYPE_S8S8S32, 32, 8, 32, (256, 2560, 1024)),
+                                  (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16, (512, 1024, 256)),
+                                  (uk.MMT4D_TYPE_BF16BF16F32, 16, 32, 8, (512, 1536, 384)),
+                                  (uk.MMT4D_TYPE_F32F32F32, 16, 16, 4, (256, 1024, 192))])
+@pytest.mark.parametrize("workgroups", [1, 3, 4])
+def test_mmt4d_persistent_kernels(gpu, oracle, variant, tile, workgroups):
+    lib, torch = gpu
+    tf, M0, N0, K0, (m, n, k) = tile
+    lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant)
+    lib.set_persistent_workgroups(workgroups)
+    try:
+        shape = (m // M0, n // N0, k // K0)
+        for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=9100 + variant, slack=16,
+                                             shapes=(shape,))):
+            rng = np.random.default_rng(300 + ci)
+            lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+            want = out0.copy()
+            G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+            got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+            assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+            assert lib.last_kernel_name().endswith("_persistent"), lib.last_kernel_name()
+    finally:
+        lib.set_persistent_workgroups(0)
+        lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+
+
+# Operands at odd element offsets and strides (the reference grid's slack of
+# one element: tools/mmt4d_test.c:354-404), WITHOUT the generic-fallback flag:
+# iree_uk_mmt4d_info advertises these tile shapes, so an MFMA kernel has to
+# serve them wherever the buffers happen to start.
+@pytest.mark.parametrize("variant", [0, 1, 3, 4])
+@pytest.mark.parametrize("tile", [(uk.MMT4D_TYPE_S8S8S32, 16, 16, 2), (uk.MMT4D_TYPE_S8S8S32, 16, 16, 16),
+                                  (uk.MMT4D_TYPE_S8S8S32, 32, 16, 8), (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16),
+                                  (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 2),
+                                  (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
+                                  (uk.MMT4D_TYPE_F32F32F32, 16, 16, 4)])
+def test_mmt4d_unaligned_operands_take_the_mfma_kernels(gpu, oracle, tile, variant):
+    lib, torch = gpu
+    tf, M0, N0, K0 = tile
+    lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
+    before = lib.mfma_decline_count()
+    bits = uk.MMT4D_TYPE_BITS[tf][0]
+    kb = K0 * bits // 8
+    shapes = ((1, 1, max(1, 64 // kb)), (3, 5, max(2, 200 // kb)), (17, 18, max(1, 128 // kb)),
+              (1, 40, max(1, 512 // kb)), (2, 2, 3))
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=5200 + variant, slack=1, shapes=shapes)):
+        rng = np.random.default_rng(700 + ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        assert lib.last_kernel_name().startswith("mmt4d_mfma"), (c.label(), lib.last_kernel_name())
+    assert lib.mfma_decline_count() == before
+
+
+def test_mmt4d_declined_call_is_counted_and_still_exact(gpu):
+    """A negative panel stride is outside what the MFMA kernels index; without
+    the fallback flag the call is still served (scalar kernel, same result)
+    and shows in iree_uk_amd_mfma_decline_count."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    M1, N1, K1, M0, N0, K0 = 3, 2, 4, 16, 16, 16
+    panel = K1 * M0 * K0
+    g = torch.Generator(device="cuda"); g.manual_seed(77)
+    lhs = torch.randint(-128, 128, (M1, panel), generator=g, device="cuda", dtype=torch.int8)
+    rhs = torch.randint(-128, 128, (N1, K1 * N0 * K0), generator=g, device="cuda", dtype=torch.int8)
+    fwd = torch.zeros(M1, N1 * M0 * N0, device="cuda", dtype=torch.int32)
+    bwd = torch.zeros_like(fwd)
+    before = lib.mfma_decline_count()
+    lib.mmt4d(lhs.data_ptr(), 0, panel, rhs.data_ptr(), 0, K1 * N0 * K0, fwd.data_ptr(), 0,
+              N1 * M0 * N0, M1, N1, K1, M0, N0, K0, uk.MMT4D_TYPE_S8S8S32)
+    assert lib.mfma_decline_count() == before
+    lib.mmt4d(lhs.data_ptr(), (M1 - 1) * panel, -panel, rhs.data_ptr(), 0, K1 * N0 * K0,
+              bwd.data_ptr(), 0, N1 * M0 * N0, M1, N1, K1, M0, N0, K0, uk.MMT4D_TYPE_S8S8S32)
+    lib.synchronize()
+    assert lib.last_kernel_name() == "mmt4d_generic"
+    assert lib.mfma_decline_count() == before + 1
+    assert torch.equal(bwd, fwd.flip(0))

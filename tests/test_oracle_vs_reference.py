@@ -83,3 +83,56 @@ def test_reference_arch_paths_agree_on_integers(oracle, reference):
     ref_arch.mmt4d(lhs, 0, K * M0 * K0, rhs, 0, K * N0 * K0, b, 0, N * M0 * N0,
                    M, N, K, M0, N0, K0, 0x102)  # no generic fallback allowed
     assert np.array_equal(a, b)
+
+
+def _ref_f8(reference):
+    import ctypes
+    L = reference.lib
+    if not hasattr(L, "ref_f8e4m3fn_to_f32"):
+        pytest.skip("oracle/_ref was built without the f8 conversions")
+    L.ref_f8e4m3fn_to_f32.argtypes = [ctypes.c_uint8]
+    L.ref_f8e4m3fn_to_f32.restype = ctypes.c_float
+    L.ref_f32_to_f8e4m3fn.argtypes = [ctypes.c_float]
+    L.ref_f32_to_f8e4m3fn.restype = ctypes.c_uint8
+    return L
+
+
+def test_f8_decode_all_codes_against_reference_code(oracle, reference):
+    """The oracle's E4M3FN decode (what its f8 mmt4d multiplies) against the
+    reference's own iree_math_f8e4m3fn_to_f32
+    (runtime/src/iree/base/internal/math.h:324-362,557-560), compiled from
+    where it lies: all 256 codes bit for bit, NaNs as NaNs."""
+    L = _ref_f8(reference)
+    for v in range(256):
+        want = np.float32(L.ref_f8e4m3fn_to_f32(v))
+        got = np.float32(oracle.f8e4m3fn_to_f32(v))
+        if np.isnan(want):
+            assert np.isnan(got), hex(v)
+        else:
+            assert got.view(np.uint32) == want.view(np.uint32), hex(v)
+    assert sum(np.float64(L.ref_f8e4m3fn_to_f32(v)) for v in range(0x7F)) == 5407.875
+
+
+def test_f8_test_side_encoder_against_reference_encoder(reference):
+    """The encoder the tests use to make f8 inputs against the reference's
+    iree_math_f32_to_f8e4m3fn (math.h:364-460) on every representable value,
+    on midpoints between neighbours (ties to even) and on random values in
+    range. One known difference is left out: the reference flushes magnitudes
+    inside (2^-10, 2^-9) to zero instead of rounding them up to the minimum
+    subnormal (math.h:431-442)."""
+    L = _ref_f8(reference)
+    table = T.f8e4m3fn_table()
+    finite = [v for v in range(256) if not np.isnan(table[v])]
+    vals = [float(table[v]) for v in finite]
+    pos = sorted(set(abs(x) for x in vals))
+    mids = [(a + b) / 2 for a, b in zip(pos[:-1], pos[1:])]
+    rng = np.random.default_rng(11)
+    rand = list(rng.uniform(-448, 448, 4000)) + list(rng.normal(0, 1, 4000))
+    probe = np.array(vals + mids + [-m for m in mids] + rand, dtype=np.float32)
+    tiny = (np.abs(probe) > 2.0 ** -10) & (np.abs(probe) < 2.0 ** -9)
+    probe = probe[~tiny]
+    ours = T.f32_to_f8e4m3fn_bits(probe)
+    for x, code in zip(probe, ours):
+        want = int(L.ref_f32_to_f8e4m3fn(float(x)))
+        # +0 and -0 of a value that rounds to zero keep their sign in both
+        assert int(code) == want, (float(x), hex(int(code)), hex(want))
