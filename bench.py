@@ -27,7 +27,7 @@ EXTRA_WORKLOADS = [
     "s8_mmt4d_8192_k2", "s8_mmt4d_8192_k16", "s8_mmt4d_8192_k16_zeros", "s8_mmt4d_8192_k64",
     "s8_mmt4d_1024_k2",
     "c2_f16_chain_ragged", "c2_f16_fused_4096", "c2_f16_fused_ragged", "c3_s8_decode",
-    "c3_s8_decode_fused", "c4_f8_prefill",
+    "c3_s8_decode_fused", "c3_s8_decode_down", "c4_f8_prefill",
     "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "f32_mmt4d_4096_k1",
     "f32_mmt4d_4096_k4",
     "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288",

@@ -337,6 +337,13 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_kernel_mode(int mode);
  * any stride. */
 IREE_UK_AMD_EXPORT uint64_t iree_uk_amd_mfma_decline_count(void);
 
+/* Tuning / test knob of the calling thread: into how many slices the M-thin /
+ * N-thin mmt4d kernels split K across workgroups (0, the default: chosen from
+ * the number of output blocks and compute units; 1: never). The slice count
+ * the latest call used is iree_uk_amd_last_k_slices (1 = no split). */
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_k_slices(int n);
+IREE_UK_AMD_EXPORT int iree_uk_amd_last_k_slices(void);
+
 /* Tuning / test knob of the calling thread: how many workgroups the
  * persistent mmt4d kernels launch (each walks its share of the output blocks
  * with one software pipeline running across block boundaries). 0, the

@@ -16,13 +16,82 @@ int launch_bf16bf16(const Problem& p, int forced, hipStream_t stream, const char
 int launch_s8s4(const Problem& p, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 
+#include <mutex>
+#include <vector>
+
+// ---- workspace of the K split over workgroups (mmt4d_mfma_thin.h) -----------
+//
+// A buffer the library allocates, per host thread and stream (two streams of
+// one thread may run their kernels side by side), grown when a call needs more.
 namespace {
+
+struct OwnedWorkspace {
+  int device;
+  hipStream_t stream;
+  char* base;
+  size_t partial_bytes;
+  uint32_t n_counters;
+};
+thread_local std::vector<OwnedWorkspace> g_workspaces;
+thread_local int g_k_slices = 0;
+thread_local int g_last_k_slices = 1;
 thread_local int g_persistent_workgroups = 0;
+
 }  // namespace
 
 namespace uk_mfma {
+
 int persistent_workgroups_override() { return g_persistent_workgroups; }
+int k_slices_override() { return g_k_slices; }
+void note_k_slices(int n) { g_last_k_slices = n; }
+
+int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStream_t stream,
+                             KSplitWorkspace* ws) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 1;
+  for (OwnedWorkspace& w : g_workspaces) {
+    if (w.device == dev && w.stream == stream && w.partial_bytes >= partial_bytes &&
+        w.n_counters >= n_counters) {
+      ws->partials = w.base;
+      ws->counters = (uint32_t*)(w.base + w.partial_bytes);
+      return 0;
+    }
+  }
+  // Nothing fits: allocate (sizes rounded up so that similar calls share it),
+  // unless the stream is being captured, where allocation is not allowed; the
+  // call then runs without the split.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) { (void)hipGetLastError(); return 1; }
+  if (capture != hipStreamCaptureStatusNone) return 1;
+  size_t want_partials = 1u << 20;
+  while (want_partials < partial_bytes) want_partials <<= 1;
+  uint32_t want_counters = 4096;
+  while (want_counters < n_counters) want_counters <<= 1;
+  char* base = nullptr;
+  const size_t bytes = want_partials + (size_t)want_counters * sizeof(uint32_t);
+  if (hipMalloc((void**)&base, bytes) != hipSuccess) { (void)hipGetLastError(); return 1; }
+  // The counters start at zero; the kernels keep them there. The fill is
+  // ordered before the launch that follows on the same stream.
+  if (hipMemsetAsync(base + want_partials, 0, (size_t)want_counters * sizeof(uint32_t), stream) !=
+      hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(base);
+    return 1;
+  }
+  // A smaller workspace of the same stream is kept (a kernel in flight may
+  // still use it) and simply no longer chosen.
+  g_workspaces.push_back(OwnedWorkspace{dev, stream, base, want_partials, want_counters});
+  ws->partials = base;
+  ws->counters = (uint32_t*)(base + want_partials);
+  return 0;
+}
+
 }  // namespace uk_mfma
+
+extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_k_slices(int n) { g_k_slices = n > 0 ? n : 0; }
+
+extern "C" IREE_UK_AMD_EXPORT int iree_uk_amd_last_k_slices(void) { return g_last_k_slices; }
+
 
 extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_persistent_workgroups(int n) {
   g_persistent_workgroups = n > 0 ? n : 0;
@@ -102,6 +171,7 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     if (!iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) return -1;
   }
   if (p->K == 0) return -1;  // zero fill only: the generic kernel does it
+  uk_mfma::note_k_slices(1);
   hipStream_t stream = (hipStream_t)stream_v;
   uk_mfma::Problem pr;
   pr.lhs = (const char*)p->lhs_buffer + p->lhs_offset * eb;

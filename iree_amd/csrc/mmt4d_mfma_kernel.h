@@ -219,6 +219,15 @@ struct Args {
   uint32_t col_scale_first;
   // mmt4d_mfma_persistent.h only: log2 of M0 and N0 (powers of two there).
   int32_t lm0, ln0;
+  // mmt4d_mfma_thin.h only: K split over `kslices` workgroups per output block
+  // (1 = none). Workgroup b works on block b / kslices, K slice b % kslices;
+  // the slices' partial accumulators meet in `ws_partials` (kslices x 16 bytes
+  // per lane and accumulator block, per output block) and the workgroup that
+  // finds `ws_counters[block]` at kslices - 1 adds them up and stores. The
+  // counters are zero between launches (the last workgroup resets its own).
+  uint32_t kslices;
+  char* ws_partials;
+  uint32_t* ws_counters;
 };
 
 // Row-slot swizzle for the regrouping loaders (RB < 16): the eight lanes that

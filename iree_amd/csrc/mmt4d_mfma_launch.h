@@ -132,6 +132,24 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   return (int)hipGetLastError();
 }
 
+// Workspace of the thin kernel's K split over workgroups: `partial_bytes` of
+// partial accumulators and `n_counters` arrival counters that are zero
+// between launches. Defined in mmt4d_mfma.hip: a buffer the library allocates
+// per host thread and stream (grow-only; none while the stream is being
+// captured into a graph and nothing fits yet). Returns 0 and the pointers, 1
+// when there is no workspace but the call can run without the split, or a
+// status (> 1) that has to fail the call.
+struct KSplitWorkspace {
+  char* partials;
+  uint32_t* counters;
+};
+int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStream_t stream,
+                             KSplitWorkspace* ws);
+// K slices set with iree_uk_amd_set_k_slices on this thread; 0 = choose.
+int k_slices_override();
+// Records the slice count of the launch for iree_uk_amd_last_k_slices.
+void note_k_slices(int n);
+
 // Workgroup count set with iree_uk_amd_set_persistent_workgroups on this
 // thread; 0 = one per compute unit (defined in mmt4d_mfma.hip).
 int persistent_workgroups_override();
@@ -214,7 +232,7 @@ int launch_persistent(const Problem& p, int kt_count, bool force, hipStream_t st
 // `swapped`: the caller's problem is N-thin and is computed as its transpose
 // (out^T = rhs * lhs^T): the kernel's rows are the caller's columns.
 template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
-int launch_thin(const Problem& caller, bool swapped, hipStream_t stream) {
+int launch_thin(const Problem& caller, bool swapped, hipStream_t stream, bool allow_k_slices = false) {
   constexpr int OBYTES = ElemTraits<E>::Out::kOutBytes;
   Problem p = caller;
   if (swapped) {
@@ -278,8 +296,40 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream) {
   const int64_t span_n =
       (int64_t)(TN * 16 / p.N0 + 2) * p.rhs_stride + k_bytes * p.N0 / (S4 ? 2 : 1);
   if (span_m >= (1ll << 31) || span_n >= (1ll << 31)) return -1;
-  uk::launch(2, mmt4d_thin_kernel<E, RBC, TM, TN, KSPLIT, D>, dim3((uint32_t)(grid_m * grid_n)),
-             dim3(KSPLIT * 64), 0, stream, a);
+  // Still too few output blocks for the chip, and a long K: split K over
+  // workgroups as well, aiming at one workgroup per compute unit, each wave
+  // keeping at least four steps. The split costs a few microseconds at the end
+  // of the launch (the slices meet through device-scope accesses, three
+  // dependent round trips to where the XCDs meet), so it has to at least halve
+  // the streaming time to pay.
+  int64_t kslices = 1;
+  if (allow_k_slices) {
+    const int64_t blocks = grid_m * grid_n;
+    const int cus = compute_units();
+    if (k_slices_override() > 0) {
+      kslices = k_slices_override();
+    } else if (cus > 0 && 2 * blocks <= cus) {
+      kslices = std::min<int64_t>(8, cus / blocks);
+    }
+    kslices = std::max<int64_t>(1, std::min<int64_t>(kslices, a.steps / (4 * KSPLIT)));
+    if (blocks * kslices >= (1ll << 31)) kslices = 1;
+  }
+  if (kslices > 1) {
+    KSplitWorkspace ws{};
+    const int got = acquire_ksplit_workspace((size_t)(grid_m * grid_n * kslices) * TM * TN * 1024,
+                                             (uint32_t)(grid_m * grid_n), stream, &ws);
+    if (got > 1) return got;
+    if (got == 0) {
+      a.kslices = (uint32_t)kslices;
+      a.ws_partials = ws.partials;
+      a.ws_counters = ws.counters;
+      note_k_slices((int)kslices);
+    } else {
+      kslices = 1;
+    }
+  }
+  uk::launch(2, mmt4d_thin_kernel<E, RBC, TM, TN, KSPLIT, D>,
+             dim3((uint32_t)(grid_m * grid_n * kslices)), dim3(KSPLIT * 64), 0, stream, a);
   return (int)hipGetLastError();
 }
 
@@ -305,7 +355,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 //         occupy the 256 CUs;
 // `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem,
 // 6 the 64x64 K-split kernel, 7 the 256x128 shape, 8 the 128x512 shape,
-// 9 / 10 the persistent kernel in the 128x512 / 256x256 shape;
+// 9 / 10 the persistent kernel in the 128x512 / 256x256 shape, 11 the 64x64
+// shape with 256-byte steps three steps ahead (tile rows under 16 bytes);
 // 0 = choose) overrides the
 // size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
@@ -324,7 +375,9 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced >= 8 && forced <= 10) {
+  if (forced == 11) {
+    choice = 3;  // the 64x64 shape with the deep pipeline (narrow tile rows only)
+  } else if (forced >= 8 && forced <= 10) {
     // The big variant in its 128x512 shape (8), the persistent kernel in that
     // shape (9) or in the square one (10); the plain square shape where the
     // requested one cannot serve.
@@ -495,33 +548,39 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     }
     choice = 3;
   }
+  // The thin kernel for a problem with `thin_rows` rows on its thin side and
+  // `wide_cols` columns on the other (M-thin as it is, N-thin transposed):
+  // 32 columns per workgroup, or 16 when 32 would leave compute units without
+  // a workgroup (a decode step against a weight matrix of few rows, e.g.
+  // 16 x 4096 x 14336 s8: 16.1 -> 12.8 us); what K split over workgroups adds
+  // on top is decided in launch_thin.
+  // (A generic lambda: its body is only instantiated for the row widths that call it.)
+  auto thin_launch = [&](auto swapped_c, int64_t thin_rows, int64_t wide_cols) {
+    const bool swapped = swapped_c;
+    const bool narrow = uk::ceil_div(wide_cols, (int64_t)32) < compute_units();
+    if (thin_rows <= 16) {
+      return narrow ? launch_thin<E, RBC, 1, 1, 4, 4>(p, swapped, stream, true)
+                    : launch_thin<E, RBC, 1, 2, 4, 4>(p, swapped, stream, true);
+    }
+    if (thin_rows <= 32) {
+      return narrow ? launch_thin<E, RBC, 2, 1, 4, 4>(p, swapped, stream, true)
+                    : launch_thin<E, RBC, 2, 2, 4, 4>(p, swapped, stream, true);
+    }
+    return narrow ? launch_thin<E, RBC, 4, 1, 4, 4>(p, swapped, stream, true)
+                  : launch_thin<E, RBC, 4, 2, 4, 3>(p, swapped, stream, true);
+  };
   if (choice == 5) {
     // N-thin (a few columns against many rows, e.g. the last column strip of
     // a ragged problem): the thin kernel on the transposed problem.
     if constexpr (RBC >= 8) {
-      const int64_t cols_n = (int64_t)p.N1 * p.N0;
-      int st;
-      if (cols_n <= 16) {
-        st = launch_thin<E, RBC, 1, 2, 4, 4>(p, true, stream);
-      } else if (cols_n <= 32) {
-        st = launch_thin<E, RBC, 2, 2, 4, 4>(p, true, stream);
-      } else {
-        st = launch_thin<E, RBC, 4, 2, 4, 3>(p, true, stream);
-      }
+      int st = thin_launch(std::true_type{}, (int64_t)p.N1 * p.N0, rows_m);
       if (st >= 0) { *name = "mmt4d_mfma_thin_transposed"; return st; }
     }
     choice = 3;
   }
   if (choice == 4) {
     if constexpr (RBC >= 8) {
-      int st;
-      if (rows_m <= 16) {
-        st = launch_thin<E, RBC, 1, 2, 4, 4>(p, false, stream);
-      } else if (rows_m <= 32) {
-        st = launch_thin<E, RBC, 2, 2, 4, 4>(p, false, stream);
-      } else {
-        st = launch_thin<E, RBC, 4, 2, 4, 3>(p, false, stream);
-      }
+      int st = thin_launch(std::false_type{}, rows_m, (int64_t)p.N1 * p.N0);
       if (st >= 0) { *name = "mmt4d_mfma_thin"; return st; }
     }
     // With 2-byte rows a 16-byte piece spans 8 rows and 32 rows do not fill a
@@ -559,6 +618,16 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         return finish_k(launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
       }
       if (st > 0) return st;
+    }
+  }
+  if constexpr (RBC < 16) {
+    // Narrow tile rows, small problem: latency-bound (a 64x64 block computes a
+    // 64-byte step in 64 MFMA cycles against a global round trip of well over a
+    // thousand). 256-byte steps with the loads three steps ahead put the whole K
+    // of such a problem in flight at once.
+    if (forced == 11 || (forced == 0 && ((int64_t)p.K1 << p.lrb) <= 8192)) {
+      int st = launch_variant<E, RBC, 2, 2, 2, 2, 4 / H, 4>(p, 0, p.K1, p.accumulate, stream);
+      if (st >= 0) { *name = "mmt4d_mfma_64x64_deep"; return st; }
     }
   }
   int st = launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);

@@ -7,11 +7,11 @@ int launch_s8s4(const Problem& p, hipStream_t stream, const char** name) {
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int st;
   if (rows_m <= 16) {
-    st = launch_thin<Elem::kS8S4, 16, 1, 2, 4, 4>(p, false, stream);
+    st = launch_thin<Elem::kS8S4, 16, 1, 2, 4, 4>(p, false, stream, true);
   } else if (rows_m <= 32) {
-    st = launch_thin<Elem::kS8S4, 16, 2, 2, 4, 4>(p, false, stream);
+    st = launch_thin<Elem::kS8S4, 16, 2, 2, 4, 4>(p, false, stream, true);
   } else {
-    st = launch_thin<Elem::kS8S4, 16, 4, 2, 4, 3>(p, false, stream);
+    st = launch_thin<Elem::kS8S4, 16, 4, 2, 4, 3>(p, false, stream, true);
   }
   if (st >= 0) *name = "mmt4d_mfma_thin_s8s4";
   return st;

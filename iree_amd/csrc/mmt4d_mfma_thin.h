@@ -10,7 +10,12 @@
 //     from HBM and the (small, shared) LHS from L2, D steps ahead of the MFMAs
 //     through D register buffers;
 //   * the KSPLIT partial accumulators meet in LDS once, at the end, and wave 0
-//     adds them in wave order and stores.
+//     adds them in wave order and stores;
+//   * when the problem has too few output blocks to occupy the chip (a decode
+//     step against a weight matrix with few rows and a long K), K is split
+//     over several workgroups per block as well: each publishes its partial
+//     block in a workspace, and the one that arrives last (an atomic counter
+//     per block) adds the slices in slice order and stores.
 //
 // Operand layout, K-order freedom of the MFMA and the output addressing are
 // those of mmt4d_mfma_kernel.h, whose Args this kernel takes. With TM = TN = 4
@@ -63,8 +68,15 @@ void mmt4d_thin_kernel(Args a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t q = lane >> 4, r = lane & 15;
-  const int bm = (int)(blockIdx.x / (uint32_t)a.grid_n);
-  const int bn = (int)(blockIdx.x - (uint32_t)bm * a.grid_n);
+  // With K split over workgroups, consecutive workgroups share an output block.
+  const uint32_t kslices = a.kslices > 1 ? a.kslices : 1;
+  const uint32_t block_id = kslices > 1 ? blockIdx.x / kslices : blockIdx.x;
+  const uint32_t slice = kslices > 1 ? blockIdx.x - block_id * kslices : 0;
+  const int bm = (int)(block_id / (uint32_t)a.grid_n);
+  const int bn = (int)(block_id - (uint32_t)bm * a.grid_n);
+  // K steps of this workgroup: [step_begin, step_begin + wg_steps).
+  const uint32_t step_begin = (uint32_t)(((uint64_t)slice * (uint32_t)a.steps) / kslices);
+  const int wg_steps = (int)((((uint64_t)(slice + 1) * (uint32_t)a.steps) / kslices) - step_begin);
   const int lrb = a.lrb;
   const int lrb_b = S4 ? lrb - 1 : lrb;       // log2 of the RHS row bytes
   const uint32_t kt_m = (uint32_t)a.M0 << lrb, kt_n = (uint32_t)a.N0 << lrb_b;
@@ -122,9 +134,9 @@ void mmt4d_thin_kernel(Args a) {
   using BFrag = typename std::conditional<S4, v2i, v4i>::type;
   v4i fa[D][TM][HALVES];
   BFrag fb[D][TN][HALVES];
-  // Local step i of this wave is K step wave + i * KSPLIT.
+  // Local step i of this wave is K step step_begin + wave + i * KSPLIT.
   auto load_step = [&](int d, int i) {
-    const uint32_t s = (uint32_t)(wave + i * KSPLIT);
+    const uint32_t s = step_begin + (uint32_t)(wave + i * KSPLIT);
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -185,7 +197,7 @@ void mmt4d_thin_kernel(Args a) {
     for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
 
   // ---- K loop ---------------------------------------------------------------
-  const int my_steps = (a.steps - wave + KSPLIT - 1) / KSPLIT;
+  const int my_steps = wg_steps > wave ? (wg_steps - wave + KSPLIT - 1) / KSPLIT : 0;
 #pragma unroll
   for (int d = 0; d < D; ++d)
     if (d < my_steps) load_step(d, d);
@@ -199,7 +211,8 @@ void mmt4d_thin_kernel(Args a) {
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) sn[tn] = v4f{1.0f, 1.0f, 1.0f, 1.0f};
   // With the 4-bit RHS the accumulators hold 16 times the sum, so the
-  // ACCUMULATE input waits in registers of its own.
+  // ACCUMULATE input waits in registers of its own. With K split over
+  // workgroups only the first slice starts from the ACCUMULATE input.
   Acc cin[S4 ? TM : 1][S4 ? TN : 1];
   if constexpr (S4) {
 #pragma unroll
@@ -208,7 +221,7 @@ void mmt4d_thin_kernel(Args a) {
       for (int tn = 0; tn < TN; ++tn) cin[tm][tn] = Acc{0, 0, 0, 0};
   }
   if (wave == 0) {
-    if (a.accumulate) {
+    if (a.accumulate && slice == 0) {
       for_each_output(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn, a.acc_sn0,
                       [&](int tm, int tn, char* p) {
                         if constexpr (S4) cin[tm][tn] = Out::load4(p);
@@ -307,10 +320,71 @@ void mmt4d_thin_kernel(Args a) {
   }
 
   if constexpr (S4) {
+    // Every slice holds 16 times its part of the sum (plus, in slice 0, nothing
+    // else: the ACCUMULATE input waits in cin), so the shift is exact per slice.
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = (acc[tm][tn] >> 4) + cin[tm][tn];
+  }
+
+  // ---- meet the K slices of the other workgroups -----------------------------------
+  // Only wave 0 is left. It publishes this workgroup's partial block, then
+  // counts itself in; the workgroup that arrives last adds the slices up in
+  // slice order (so a float result does not depend on who arrived when) and
+  // goes on to store. The slices run on different XCDs, each with an L2 of
+  // its own, so partials and counter are moved with device-scope atomic
+  // accesses (relaxed 32-bit stores and loads: they go through to the point
+  // where the XCDs meet and leave the caches alone). A device-scope FENCE
+  // would be correct too and is far too expensive here: it writes back and
+  // invalidates the whole L2, under the feet of every workgroup that streams
+  // weights through it. What the counter increment has to wait for is only
+  // that this wave's own partial stores are complete.
+  if (kslices > 1) {
+    uint32_t* mine = reinterpret_cast<uint32_t*>(a.ws_partials) +
+                     (((size_t)block_id * kslices + slice) * (TM * TN * 64) + lane) * 4;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const v4i v = __builtin_bit_cast(v4i, acc[tm][tn]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          __hip_atomic_store(mine + (tm * TN + tn) * 256 + e, (uint32_t)v[e], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      }
+    // All of the wave's stores above have been acknowledged before the count.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    uint32_t arrived = 0;
+    if (lane == 0) {
+      arrived = __hip_atomic_fetch_add(a.ws_counters + block_id, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    }
+    arrived = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrived);
+    if (arrived != kslices - 1) return;
+    if (lane == 0) {
+      __hip_atomic_store(a.ws_counters + block_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const uint32_t* all = reinterpret_cast<const uint32_t*>(a.ws_partials) +
+                          ((size_t)block_id * kslices * (TM * TN * 64) + lane) * 4;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = Acc{0, 0, 0, 0};
+    for (uint32_t sl = 0; sl < kslices; ++sl) {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+          v4i v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[e] = (int)__hip_atomic_load(all + ((size_t)sl * (TM * TN) + tm * TN + tn) * 256 + e,
+                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          acc[tm][tn] += __builtin_bit_cast(Acc, v);
+        }
+    }
   }
 
   // ---- store --------------------------------------------------------------------

@@ -281,11 +281,13 @@ class Runner:
                             op.flops, op.bytes, "f32",
                             dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
                                  M0=M0, N0=N0, K0=K0))
-        if name == "c3_s8_decode":
+        if name in ("c3_s8_decode", "c3_s8_decode_down"):
             # Decode-shaped quantized linear layer: 16 activations rows padded to
             # M0=32, weights [14336, 4096] pre-packed once (not timed), ACCUMULATE
-            # into a seeded s32 buffer.
-            Mlog, K, N = 16, 4096, 14336
+            # into a seeded s32 buffer. `_down` is its mate in a transformer MLP,
+            # the projection back (weights [4096, 14336]): few output blocks and a
+            # long K, the shape the K split over workgroups is for.
+            Mlog, K, N = (16, 4096, 14336) if name == "c3_s8_decode" else (16, 14336, 4096)
             M0, N0, K0 = 32, 16, 8
             M1, N1, K1 = 1, N // N0, K // K0
             act = self.clipped_normal_s8((Mlog, K), 7, 40.0)
@@ -319,7 +321,7 @@ class Runner:
                     torch.mul(acc_view, scale, out=y_view)  # one kernel: s32 * f32 -> f32
             ep = Op("scale_epilogue", epilogue, 0.0, float(Mlog * N * 8), "hbm", "f32",
                     kernel="torch (harness, not a ukernel)", external=True)
-            return Workload(name, "mmt4d s8 decode M=16(32) K=4096 N=14336 tiles 32x16x8 ACCUMULATE "
+            return Workload(name, f"mmt4d s8 decode M=16(32) K={K} N={N} tiles 32x16x8 ACCUMULATE "
                             "+ per-row/per-column scale epilogue",
                             [op, ep], op.flops, op.bytes, "s8",
                             dict(act=act, w=w, lhs4=lhs4, rhs4=rhs4, out4=out4, y=y, scale_m=scale_m,

@@ -78,6 +78,16 @@ _u32 = ctypes.c_uint32
 _u64 = ctypes.c_uint64
 _vp = ctypes.c_void_p
 
+class Mmt4dParams(ctypes.Structure):
+    """iree_uk_mmt4d_params_t (include/iree_uk_amd.h; field order of
+    runtime/src/iree/builtins/ukernel/mmt4d_internal.h:14-32)."""
+    _fields_ = [("lhs_buffer", _vp), ("lhs_offset", _i64), ("lhs_stride0", _i64),
+                ("rhs_buffer", _vp), ("rhs_offset", _i64), ("rhs_stride0", _i64),
+                ("out_buffer", _vp), ("out_offset", _i64), ("out_stride0", _i64),
+                ("M", _i64), ("N", _i64), ("K", _i64), ("M0", _i32), ("N0", _i32),
+                ("K0", _i32), ("flags", _u32), ("cpu_data", _vp)]
+
+
 ASSERT_HANDLER = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_int,
                                   ctypes.c_char_p, ctypes.c_char_p)
 
@@ -161,6 +171,9 @@ class UKernelLibrary:
         L.iree_uk_amd_set_persistent_workgroups.argtypes = [ctypes.c_int]
         L.iree_uk_amd_set_persistent_workgroups.restype = None
         L.iree_uk_amd_device_count.restype = ctypes.c_int
+        L.iree_uk_amd_set_k_slices.argtypes = [ctypes.c_int]
+        L.iree_uk_amd_set_k_slices.restype = None
+        L.iree_uk_amd_last_k_slices.restype = ctypes.c_int
         L.iree_uk_amd_mfma_decline_count.restype = ctypes.c_uint64
         L.iree_uk_amd_version.restype = ctypes.c_char_p
         L.iree_uk_amd_set_assert_handler.argtypes = [_vp]
@@ -184,6 +197,20 @@ class UKernelLibrary:
                                rhs_stride0, out, out_offset, out_stride0, M, N,
                                K, M0, N0, K0, flags, cpu_data)
         self._check()
+
+    def last_status(self) -> int:
+        return int(self.lib.iree_uk_amd_last_status())
+
+    def last_status_string(self) -> str:
+        return self.lib.iree_uk_amd_last_status_string().decode()
+
+    def set_k_slices(self, n: int):
+        """K slices across workgroups of the thin mmt4d kernels on this thread
+        (0 = choose, 1 = never split)."""
+        self.lib.iree_uk_amd_set_k_slices(n)
+
+    def last_k_slices(self) -> int:
+        return int(self.lib.iree_uk_amd_last_k_slices())
 
     def mmt4d_info(self, M0, N0, K0, flags, cpu_data=None) -> int:
         return int(self.lib.iree_uk_mmt4d_info(M0, N0, K0, flags, cpu_data))

@@ -1,0 +1,132 @@
+"""K split over workgroups in the M-thin / N-thin mmt4d kernels (decode-shaped
+problems with too few output blocks to occupy the chip): every slice count
+against the CPU oracle, through the C-ABI. Integer types bit-exact; float types
+bit-exact too, on the small-integer inputs of the reference's own tests
+(tools/util.c:131-165: every partial sum is exact, so neither the split nor the
+order in which the slices are added can show)."""
+import numpy as np
+import pytest
+
+import uk_testing as T
+from golden import make_golden as G
+from iree_amd import ukernel as uk
+
+pytestmark = pytest.mark.gpu
+
+TILES = [(uk.MMT4D_TYPE_S8S8S32, 32, 16, 8), (uk.MMT4D_TYPE_S8S8S32, 16, 16, 16),
+         (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16), (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
+         (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 4),
+         (uk.MMT4D_TYPE_S8S4S32, 16, 16, 32)]
+
+
+@pytest.fixture(autouse=True)
+def _reset(lib):
+    yield
+    lib.set_k_slices(0)
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+
+
+# (tile, N-thin?): the 4-bit RHS kernel serves M-thin problems only.
+CASES = [(t, n_thin) for t in TILES for n_thin in (False, True)
+         if not (n_thin and t[0] == uk.MMT4D_TYPE_S8S4S32)]
+
+
+@pytest.mark.parametrize("slices", [2, 3, 5])
+@pytest.mark.parametrize("tile,n_thin", CASES)
+def test_thin_kernels_with_k_slices(gpu, oracle, tile, n_thin, slices):
+    lib, torch = gpu
+    tf, M0, N0, K0 = tile
+    lb = uk.MMT4D_TYPE_BITS[tf][0]
+    step_elems = (128 if tf == uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32 else 64) * 8 // lb
+    # Each wave keeps at least four steps: 16 steps per slice, plus a few so
+    # that the slices are not all the same length.
+    k_tiles = (16 * slices + 3) * step_elems // K0
+    thin, wide = (1, 7)
+    shape = (wide, thin, k_tiles) if n_thin else (thin, wide, k_tiles)
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lib.set_k_slices(slices)
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=4300 + slices, slack=16, shapes=(shape,))):
+        rng = np.random.default_rng(900 + ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        assert lib.last_kernel_name().startswith("mmt4d_mfma_thin"), lib.last_kernel_name()
+        assert lib.last_k_slices() == slices
+
+
+def test_k_slices_are_chosen_for_a_decode_step_with_few_columns(gpu):
+    """A decode step against a weight matrix of few rows and a long K (16 rows,
+    K = 14336, N = 1024, tiles 32x16x8, ACCUMULATE): 64 output blocks of 16
+    columns for 256 compute units. The library splits K on its own, and the
+    result is the exact integer product plus the initial accumulators."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lib.set_k_slices(0)
+    Mlog, K, N, M0, N0, K0 = 16, 14336, 1024, 32, 16, 8
+    N1, K1 = N // N0, K // K0
+    g = torch.Generator(device="cuda"); g.manual_seed(41)
+    act = torch.randint(-128, 128, (Mlog, K), generator=g, device="cuda", dtype=torch.int8)
+    w = torch.randint(-128, 128, (N, K), generator=g, device="cuda", dtype=torch.int8)
+    lhs4 = torch.zeros(K1 * M0 * K0, device="cuda", dtype=torch.int8)
+    rhs4 = torch.zeros(N1 * K1 * N0 * K0, device="cuda", dtype=torch.int8)
+    lib.pack(act.data_ptr(), 0, K, 1, lhs4.data_ptr(), 0, K1 * M0 * K0, M0 * K0, Mlog, K, 1, K1, M0, K0, 0,
+             uk.PACK_TYPE_I8I8)
+    lib.pack(w.data_ptr(), 0, K, 1, rhs4.data_ptr(), 0, K1 * N0 * K0, N0 * K0, N, K, N1, K1, N0, K0, 0,
+             uk.PACK_TYPE_I8I8)
+    acc0 = torch.randint(-2 ** 15, 2 ** 15, (N1, M0, N0), generator=g, device="cuda", dtype=torch.int32)
+    out4 = acc0.clone()
+    lib.mmt4d(lhs4.data_ptr(), 0, K1 * M0 * K0, rhs4.data_ptr(), 0, K1 * N0 * K0, out4.data_ptr(), 0,
+              N1 * M0 * N0, 1, N1, K1, M0, N0, K0, uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE)
+    lib.synchronize()
+    assert lib.last_kernel_name() == "mmt4d_mfma_thin"
+    assert lib.last_k_slices() > 1
+    prod = act.cpu().to(torch.int64) @ w.cpu().to(torch.int64).T                       # [16][N]
+    want = acc0.cpu().to(torch.int64)
+    want[:, :Mlog, :] += prod.view(Mlog, N1, N0).permute(1, 0, 2)
+    assert torch.equal(out4.cpu().to(torch.int64), want)
+
+
+def test_k_slices_with_the_dequantizing_store(gpu):
+    """The fused dequantizing call under a forced split equals the unsplit one
+    bit for bit (integer accumulators: the split cannot show)."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    rows, K, N, M0, N0, K0 = 16, 4096, 512, 16, 16, 16
+    N1, K1 = N // N0, K // K0
+    g = torch.Generator(device="cuda"); g.manual_seed(43)
+    lhs = torch.randint(-128, 128, (K1 * M0 * K0,), generator=g, device="cuda", dtype=torch.int8)
+    rhs = torch.randint(-128, 128, (N1 * K1 * N0 * K0,), generator=g, device="cuda", dtype=torch.int8)
+    acc = torch.randint(-1000, 1000, (N1 * M0 * N0,), generator=g, device="cuda", dtype=torch.int32)
+    rs = torch.rand(rows, generator=g, device="cuda") * 0.02 + 0.001
+    cs = torch.rand(N, generator=g, device="cuda") * 0.02 + 0.001
+    results = []
+    for slices in (1, 4):
+        lib.set_k_slices(slices)
+        y = torch.full((rows, N), -1.0, device="cuda")
+        lib.mmt4d_dequant_unpack(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0,
+                                 acc.data_ptr(), 0, N1 * M0 * N0, y.data_ptr(), 0, N, rows, N,
+                                 rs.data_ptr(), cs.data_ptr(), 1, N1, K1, M0, N0, K0,
+                                 uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE)
+        lib.synchronize()
+        assert lib.last_k_slices() == slices
+        results.append(y)
+    assert torch.equal(results[0], results[1])
+
+
+def test_k_slices_on_the_32_column_blocks(gpu, oracle):
+    """Enough columns for a 32-column block per compute unit (so the narrow
+    16-column blocks are not chosen) and a forced split."""
+    lib, torch = gpu
+    tf, M0, N0, K0 = uk.MMT4D_TYPE_S8S8S32, 16, 16, 16
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lib.set_k_slices(2)
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=4400, slack=16, shapes=((1, 640, 35 * 4),))):
+        rng = np.random.default_rng(950 + ci)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        assert lib.last_kernel_name() == "mmt4d_mfma_thin" and lib.last_k_slices() == 2
