@@ -287,7 +287,16 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_assert_handler(
 /*===--------------------------------------------------------------------===*/
 
 /* Status of the most recent entry-point call on this thread: 0 = OK, else a
- * hipError_t value (launch or staging failure) or -1 (contract violation). */
+ * hipError_t value (launch or staging failure), -1 (contract violation) or
+ * one of the values below. */
+enum {
+  /* iree_uk_amd_mmt4d_no_alloc: the call's K-split workspace exceeds the
+   * library's static scratch array (iree_uk_amd_no_alloc_scratch_bytes). */
+  IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL = 100001,
+  /* iree_uk_amd_mmt4d_no_alloc: an operand is ordinary host memory, which
+   * would have to be staged through a device allocation. */
+  IREE_UK_AMD_STATUS_NEEDS_ALLOCATION = 100002,
+};
 IREE_UK_AMD_EXPORT int iree_uk_amd_last_status(void);
 IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_status_string(void);
 
@@ -336,6 +345,31 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_kernel_mode(int mode);
  * the latest call. No counterpart in the reference, whose tile functions take
  * any stride. */
 IREE_UK_AMD_EXPORT uint64_t iree_uk_amd_mfma_decline_count(void);
+
+/* iree_uk_mmt4d_p for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference. Same parameters, same result (bit
+ * for bit, floats included: both entry points take the same kernel with the
+ * same split of K), with two differences:
+ *   - every operand must already be device-accessible memory; a host operand
+ *     fails with IREE_UK_AMD_STATUS_NEEDS_ALLOCATION (iree_uk_mmt4d would
+ *     stage it through a device allocation);
+ *   - when the kernel splits K over workgroups (M-thin or N-thin problems of
+ *     few output blocks and a long K: the decode step of a linear layer), the
+ *     slices' partial accumulators and arrival counters live in a static
+ *     device array of the library, iree_uk_amd_no_alloc_scratch_bytes() bytes
+ *     (8 MiB of partials + 16384 counters) held by every GPU the library runs
+ *     on, instead of a buffer iree_uk_mmt4d allocates on first need. A call
+ *     whose split needs more fails with IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL
+ *     and writes nothing.
+ * The call allocates nothing: no hipMalloc / hipFree, no allocating library
+ * routine. All calls on one GPU share that GPU's array; the kernels leave its
+ * counters at zero and write partials before reading them, so consecutive
+ * calls need no clearing, but calls that OVERLAP on one GPU (two streams, two
+ * threads) race on it: serialize them. Results through the status functions
+ * as for every entry point. */
+IREE_UK_AMD_EXPORT void iree_uk_amd_mmt4d_no_alloc(const iree_uk_mmt4d_params_t* params);
+IREE_UK_AMD_EXPORT int64_t iree_uk_amd_no_alloc_scratch_bytes(void);
 
 /* Tuning / test knob of the calling thread: into how many slices the M-thin /
  * N-thin mmt4d kernels split K across workgroups (0, the default: chosen from

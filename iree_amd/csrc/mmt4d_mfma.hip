@@ -21,9 +21,44 @@ int launch_s8s4(const Problem& p, hipStream_t stream, const char** name);
 
 // ---- workspace of the K split over workgroups (mmt4d_mfma_thin.h) -----------
 //
-// A buffer the library allocates, per host thread and stream (two streams of
-// one thread may run their kernels side by side), grown when a call needs more.
+// Ordinary calls: a buffer the library allocates, per host thread and stream
+// (two streams of one thread may run their kernels side by side), grown when a
+// call needs more. Calls through iree_uk_amd_mmt4d_no_alloc: the static device
+// array below, one copy per GPU, shared by every such call on that GPU.
 namespace {
+
+constexpr size_t kScratchPartialBytes = 8u << 20;   // partial accumulator blocks
+constexpr uint32_t kScratchCounters = 16384;        // one arrival counter per output block
+constexpr size_t kScratchBytes = kScratchPartialBytes + kScratchCounters * sizeof(uint32_t);
+
+// Zero when the code object is loaded; the kernels leave the counters at zero
+// (the workgroup that arrives last at a block resets that block's counter), and
+// partial blocks are written before they are read, so nothing needs clearing
+// between calls. Calls that overlap on one GPU would race on it.
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, looked up once
+
+// The array's name is a host-side stand-in, not a device address: ask the
+// runtime for the address on the current device, once per device.
+int scratch_address(void** ptr) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return (int)err;
+  if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return (int)err;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
 
 struct OwnedWorkspace {
   int device;
@@ -33,6 +68,7 @@ struct OwnedWorkspace {
   uint32_t n_counters;
 };
 thread_local std::vector<OwnedWorkspace> g_workspaces;
+thread_local bool g_no_alloc = false;
 thread_local int g_k_slices = 0;
 thread_local int g_last_k_slices = 1;
 thread_local int g_persistent_workgroups = 0;
@@ -47,6 +83,17 @@ void note_k_slices(int n) { g_last_k_slices = n; }
 
 int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStream_t stream,
                              KSplitWorkspace* ws) {
+  if (g_no_alloc) {
+    if (partial_bytes > kScratchPartialBytes || n_counters > kScratchCounters) {
+      return IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL;
+    }
+    void* base = nullptr;
+    const int st = scratch_address(&base);
+    if (st != 0) return st;
+    ws->partials = (char*)base;
+    ws->counters = (uint32_t*)((char*)base + kScratchPartialBytes);
+    return 0;
+  }
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 1;
   for (OwnedWorkspace& w : g_workspaces) {
@@ -88,10 +135,15 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
 
 }  // namespace uk_mfma
 
+extern "C" void iree_uk_amd_hip_set_no_alloc(int on) { g_no_alloc = on != 0; }
+
 extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_k_slices(int n) { g_k_slices = n > 0 ? n : 0; }
 
 extern "C" IREE_UK_AMD_EXPORT int iree_uk_amd_last_k_slices(void) { return g_last_k_slices; }
 
+extern "C" IREE_UK_AMD_EXPORT int64_t iree_uk_amd_no_alloc_scratch_bytes(void) {
+  return (int64_t)kScratchBytes;
+}
 
 extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_persistent_workgroups(int n) {
   g_persistent_workgroups = n > 0 ? n : 0;

@@ -134,11 +134,12 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
 
 // Workspace of the thin kernel's K split over workgroups: `partial_bytes` of
 // partial accumulators and `n_counters` arrival counters that are zero
-// between launches. Defined in mmt4d_mfma.hip: a buffer the library allocates
-// per host thread and stream (grow-only; none while the stream is being
-// captured into a graph and nothing fits yet). Returns 0 and the pointers, 1
-// when there is no workspace but the call can run without the split, or a
-// status (> 1) that has to fail the call.
+// between launches. Defined in mmt4d_mfma.hip: ordinary calls get a buffer
+// the library allocates per host thread and stream (grow-only; none while the
+// stream is being captured into a graph and nothing fits yet), calls through
+// iree_uk_amd_mmt4d_no_alloc get the library's static device array. Returns 0
+// and the pointers, 1 when there is no workspace but the call can run without
+// the split, or a status (> 1) that has to fail the call.
 struct KSplitWorkspace {
   char* partials;
   uint32_t* counters;

@@ -62,6 +62,10 @@ int iree_uk_amd_hip_conv_nchwc_has_mfma_kernel(int32_t k0, int32_t c0,
 int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0, int32_t K0,
                                           uint32_t flags);
 
+/* 1: until switched off again, mmt4d launches of this thread take their K-split
+ * workspace from the library's static device array and never allocate. */
+void iree_uk_amd_hip_set_no_alloc(int on);
+
 /* Runtime wrappers. */
 int iree_uk_amd_hip_device_count(void);
 /* *is_device = 1 if `ptr` is device-accessible memory known to HIP (device,

@@ -368,6 +368,37 @@ void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params) {
   mmt4d_run(params, 0);
 }
 
+/* iree_uk_mmt4d_p without any allocation (see the header). */
+void iree_uk_amd_mmt4d_no_alloc(const iree_uk_mmt4d_params_t* params) {
+  tls_status = 0;
+  tls_kernel_name = "";
+  if (!mmt4d_validate(params)) return;
+  /* mmt4d.c:106-114 */
+  if (params->M == 0 || params->N == 0 ||
+      (params->K == 0 && (params->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE))) {
+    return;
+  }
+  /* A host operand would be staged through a device allocation: refuse it
+   * before anything is launched. (K == 0 without ACCUMULATE reads no operand
+   * but still writes the output.) */
+  mmt4d_bits_t bits;
+  mmt4d_type_bits(params->flags, &bits);
+  const void* first_bytes[3] = {
+      (const char*)params->lhs_buffer + params->lhs_offset * bits.lhs_bits / 8,
+      (const char*)params->rhs_buffer + params->rhs_offset * bits.rhs_bits / 8,
+      (const char*)params->out_buffer + params->out_offset * (bits.out_bits / 8)};
+  for (int i = params->K == 0 ? 2 : 0; i < 3; ++i) {
+    int st = 0;
+    if (!is_device_pointer(first_bytes[i], &st)) {
+      tls_status = st ? st : IREE_UK_AMD_STATUS_NEEDS_ALLOCATION;
+      return;
+    }
+  }
+  iree_uk_amd_hip_set_no_alloc(1);
+  mmt4d_run(params, 0);
+  iree_uk_amd_hip_set_no_alloc(0);
+}
+
 /* Fused mmt4d + unpack: validation is that of the two calls it stands for. */
 static int mmt4d_unpack_validate(const iree_uk_amd_mmt4d_unpack_params_t* p,
                                  const iree_uk_mmt4d_params_t* mm) {

@@ -138,6 +138,14 @@ int iree_uk_amd_timing_end(double* elapsed_us, int* kinds, int capacity) {
 }
 
 const char* iree_uk_amd_hip_error_string(int status) {
+  if (status == IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL) {
+    return "the call's K-split workspace exceeds the static scratch array of "
+           "iree_uk_amd_mmt4d_no_alloc (iree_uk_amd_no_alloc_scratch_bytes); use iree_uk_mmt4d";
+  }
+  if (status == IREE_UK_AMD_STATUS_NEEDS_ALLOCATION) {
+    return "iree_uk_amd_mmt4d_no_alloc takes device-accessible operands only: a host operand "
+           "would have to be staged through a device allocation; use iree_uk_mmt4d";
+  }
   return hipGetErrorString((hipError_t)status);
 }
 

@@ -78,6 +78,10 @@ _u32 = ctypes.c_uint32
 _u64 = ctypes.c_uint64
 _vp = ctypes.c_void_p
 
+STATUS_SCRATCH_TOO_SMALL = 100001
+STATUS_NEEDS_ALLOCATION = 100002
+
+
 class Mmt4dParams(ctypes.Structure):
     """iree_uk_mmt4d_params_t (include/iree_uk_amd.h; field order of
     runtime/src/iree/builtins/ukernel/mmt4d_internal.h:14-32)."""
@@ -171,6 +175,9 @@ class UKernelLibrary:
         L.iree_uk_amd_set_persistent_workgroups.argtypes = [ctypes.c_int]
         L.iree_uk_amd_set_persistent_workgroups.restype = None
         L.iree_uk_amd_device_count.restype = ctypes.c_int
+        L.iree_uk_amd_mmt4d_no_alloc.argtypes = [_vp]
+        L.iree_uk_amd_mmt4d_no_alloc.restype = None
+        L.iree_uk_amd_no_alloc_scratch_bytes.restype = _i64
         L.iree_uk_amd_set_k_slices.argtypes = [ctypes.c_int]
         L.iree_uk_amd_set_k_slices.restype = None
         L.iree_uk_amd_last_k_slices.restype = ctypes.c_int
@@ -198,11 +205,25 @@ class UKernelLibrary:
                                K, M0, N0, K0, flags, cpu_data)
         self._check()
 
+    def mmt4d_no_alloc(self, lhs, lhs_offset, lhs_stride0, rhs, rhs_offset, rhs_stride0,
+                       out, out_offset, out_stride0, M, N, K, M0, N0, K0, flags, check=True):
+        """iree_uk_amd_mmt4d_no_alloc: same arguments as mmt4d, passed as the
+        params struct. With check=False the status is left for the caller to
+        read (last_status) instead of being raised."""
+        p = Mmt4dParams(lhs, lhs_offset, lhs_stride0, rhs, rhs_offset, rhs_stride0, out,
+                        out_offset, out_stride0, M, N, K, M0, N0, K0, flags, None)
+        self.lib.iree_uk_amd_mmt4d_no_alloc(ctypes.byref(p))
+        if check:
+            self._check()
+
     def last_status(self) -> int:
         return int(self.lib.iree_uk_amd_last_status())
 
     def last_status_string(self) -> str:
         return self.lib.iree_uk_amd_last_status_string().decode()
+
+    def no_alloc_scratch_bytes(self) -> int:
+        return int(self.lib.iree_uk_amd_no_alloc_scratch_bytes())
 
     def set_k_slices(self, n: int):
         """K slices across workgroups of the thin mmt4d kernels on this thread

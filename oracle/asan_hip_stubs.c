@@ -87,6 +87,8 @@ int iree_uk_amd_hip_mmt4d_has_mfma_kernel(int32_t M0, int32_t N0, int32_t K0, ui
   return 0;
 }
 
+void iree_uk_amd_hip_set_no_alloc(int on) { (void)on; }
+
 int iree_uk_amd_hip_device_count(void) { return 1; }
 
 int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device) {
