@@ -10,6 +10,7 @@
 #include <climits>
 
 #include "mmt4d_mfma_kernel.h"
+#include "mmt4d_mfma_narrow.h"
 #include "mmt4d_mfma_persistent.h"
 #include "mmt4d_mfma_thin.h"
 #include "uk_device_common.h"
@@ -228,6 +229,53 @@ int launch_persistent(const Problem& p, int kt_count, bool force, hipStream_t st
   return (int)hipGetLastError();
 }
 
+// Launches the narrow-row kernel (mmt4d_mfma_narrow.h: tile rows of 2 or 4
+// bytes, N0 = 16, RHS fragments loaded straight into registers) over K-tiles
+// [0, kt_count). Returns a HIP status, or -1 if it cannot serve the shape.
+template <Elem E, int RBC, int TM, int WGM, int WGN>
+int launch_narrow(const Problem& p, int kt_count, hipStream_t stream) {
+  constexpr int BM = WGM * TM * 16, BN = WGN * 64, KS = 64;
+  if (p.rb != RBC || p.N0 != 16 || p.M0 % 4 || p.M0 > BM || BM % p.M0) return -1;
+  if (p.dequant) return -1;
+  if (p.out_rows <= 0 || p.out_cols <= 0) return 0;
+  if (p.out_cols < (int64_t)p.N1 * p.N0) return -1;   // a row-major matrix narrower than the tiles
+  const int64_t k_bytes = (int64_t)kt_count << p.lrb;
+  if (kt_count <= 0 || k_bytes % KS) return -1;
+  Args a{};
+  a.lhs = p.lhs; a.rhs = p.rhs; a.out = p.out;
+  a.lhs_stride = p.lhs_stride; a.rhs_stride = p.rhs_stride; a.out_stride = p.out_stride;
+  a.out_sm0 = (uint32_t)p.out_sm0; a.out_spn = (uint32_t)p.out_spn;
+  a.out_rows = (int32_t)std::min<int64_t>(p.out_rows, INT32_MAX);
+  a.out_cols = (int32_t)std::min<int64_t>(p.out_cols, INT32_MAX);
+  a.M1 = p.M1; a.N1 = p.N1; a.K1 = kt_count;
+  a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
+  a.bpm = BM / p.M0; a.bpn = BN / p.N0;
+  const int64_t grid_m = uk::ceil_div(p.M1, a.bpm), grid_n = uk::ceil_div(p.N1, a.bpn);
+  if (grid_m * grid_n >= (1ll << 31)) return -1;
+  a.grid_m = (int32_t)grid_m; a.grid_n = (int32_t)grid_n;
+  a.steps = (int32_t)(k_bytes / KS);
+  a.accumulate = p.accumulate;
+  a.band = (WGM == 1 && WGN == 8) ? 8 : 4;
+  a.vec_out = 1;
+  a.acc = p.acc; a.acc_stride = p.acc_stride;
+  a.acc_sm0 = (uint32_t)p.acc_sm0; a.acc_spn = (uint32_t)p.acc_spn;
+  const int64_t kt_bytes_m = (int64_t)p.M0 << p.lrb, kt_bytes_n = (int64_t)p.N0 << p.lrb;
+  const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
+  const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
+  const int64_t span_o = (int64_t)a.bpm * p.out_stride + (int64_t)p.M0 * p.out_sm0 +
+                         (int64_t)p.N1 * p.out_spn;
+  const int64_t span_a = (int64_t)a.bpm * p.acc_stride + (int64_t)p.M0 * p.acc_sm0 +
+                         (int64_t)p.N1 * p.acc_spn;
+  if (span_m >= (1ll << 31) || span_n >= (1ll << 31) || span_o >= (1ll << 31) ||
+      span_a >= (1ll << 31)) {
+    return -1;
+  }
+  constexpr size_t kLds = 3 * (size_t)BM * KS;
+  uk::launch(2, mmt4d_mfma_narrow_kernel<E, RBC, TM, WGM, WGN>, dim3((uint32_t)(grid_m * grid_n)),
+             dim3(WGM * WGN * 64), kLds, stream, a);
+  return (int)hipGetLastError();
+}
+
 // Launches the M-thin kernel (mmt4d_mfma_thin.h) over all of K. Returns a HIP
 // status, or -1 if it cannot serve the shape.
 // `swapped`: the caller's problem is N-thin and is computed as its transpose
@@ -357,7 +405,9 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 // `forced` (1 big, 2 mid, 3 small, 4 thin, 5 thin on the transposed problem,
 // 6 the 64x64 K-split kernel, 7 the 256x128 shape, 8 the 128x512 shape,
 // 9 / 10 the persistent kernel in the 128x512 / 256x256 shape, 11 the 64x64
-// shape with 256-byte steps three steps ahead (tile rows under 16 bytes);
+// shape with 256-byte steps three steps ahead (tile rows under 16 bytes),
+// 12 .. 15 the narrow-row kernel (tile rows of 2 or 4 bytes, N0 = 16) in the
+// 256x256 / 128x512 / 128x128 / 64x64 shape;
 // 0 = choose) overrides the
 // size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
@@ -376,8 +426,12 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   constexpr int BIG_KS = 64 * H;
   const int64_t rows_m = (int64_t)p.M1 * p.M0;
   int choice;
-  if (forced == 11) {
-    choice = 3;  // the 64x64 shape with the deep pipeline (narrow tile rows only)
+  if (forced == 11 || forced == 15) {
+    choice = 3;  // 64x64: the deep pipeline (11) or the narrow-row kernel (15)
+  } else if (forced == 12 || forced == 13) {
+    choice = 1;  // the narrow-row kernel in the 256x256 (12) or 128x512 (13) shape
+  } else if (forced == 14) {
+    choice = 2;  // the narrow-row kernel in the 128x128 shape
   } else if (forced >= 8 && forced <= 10) {
     // The big variant in its 128x512 shape (8), the persistent kernel in that
     // shape (9) or in the square one (10); the plain square shape where the
@@ -475,19 +529,51 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   // smaller workgroup shape, as a second, accumulating launch.
   const int kts_per_step = BIG_KS >> p.lrb;
   const int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
+  constexpr bool NARROW = (RBC == 2 || RBC == 4) && H == 1 && ElemTraits<E>::Out::kOutBytes == 4;
   if (choice == 1) {
+    if constexpr (NARROW) {
+      // Tile rows of 2 or 4 bytes with N0 = 16 (the x86-style tiles): the RHS
+      // goes straight to registers here too (mmt4d_mfma_narrow.h).
+      // Measured: at 8192^3 (four rounds of blocks) it is ahead of the kernel
+      // with both operands through LDS (s8 16x16x2: 540 us against 558 us,
+      // bf16 16x16x2: 880 us against 955 us), at 4096^3 (one round) behind it
+      // (76 us against 69 us, 122 us against 117 us), so it is chosen from two
+      // rounds on. The square shape is the faster one for 2-byte rows (540 us
+      // against 567 us) and equal to the wide one for 4-byte rows, so the wide
+      // shape is taken only when asked for.
+      if (kt_main > 0 && ((forced == 0 && workgroups(p, 256, 256) >= 512) || forced == 12 || forced == 13)) {
+        int st = -1;
+        const char* nm = "";
+        if (forced == 13) {
+          st = launch_narrow<E, RBC, 8, 1, 8>(p, kt_main, stream);
+          nm = "mmt4d_mfma_128x512_narrow";
+        }
+        if (st < 0 && forced != 13) {
+          st = launch_narrow<E, RBC, 8, 2, 4>(p, kt_main, stream);
+          nm = "mmt4d_mfma_256x256_narrow";
+        }
+        if (st == 0) {
+          *name = nm;
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
+    }
     if (kt_main > 0) {
       int st = -1;
       bool wide = false;
       if constexpr (RBC >= 16 && H == 1 && ElemTraits<E>::Out::kOutBytes == 4) {
-        // Several rounds of blocks: one persistent workgroup per CU whose
-        // pipeline runs across block boundaries.
-        if (forced == 0 || forced == 9) {
-          st = launch_persistent<E, 8, 4, 1, 8>(p, kt_main, forced == 9, stream);
+        // One persistent workgroup per CU whose pipeline runs across block
+        // boundaries. Measured equal to the one-block-per-workgroup launches
+        // below (s8 8192^3: 410-420 us either way: the time is not in the block
+        // boundaries), so it is taken only when asked for.
+        if (forced == 9) {
+          st = launch_persistent<E, 8, 4, 1, 8>(p, kt_main, true, stream);
           if (st == 0) *name = "mmt4d_mfma_128x512_persistent";
         }
-        if (st < 0 && (forced == 0 || forced == 10)) {
-          st = launch_persistent<E, 8, 4, 2, 4>(p, kt_main, forced == 10, stream);
+        if (st < 0 && forced == 10) {
+          st = launch_persistent<E, 8, 4, 2, 4>(p, kt_main, true, stream);
           if (st == 0) *name = "mmt4d_mfma_256x256_persistent";
         }
         if (st == 0) {
@@ -596,6 +682,19 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 3;
   }
   if (choice == 2) {
+    if constexpr (NARROW) {
+      // (Not chosen by size: measured level with or behind the 128x128 kernel
+      // that sends both operands through LDS.)
+      if (kt_main > 0 && forced == 14) {
+        int st = launch_narrow<E, RBC, 4, 2, 2>(p, kt_main, stream);
+        if (st == 0) {
+          *name = "mmt4d_mfma_128x128_narrow";
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
+    }
     if constexpr (RBC >= 16) {
       if (kt_main > 0) {
         int st = launch_variant<E, RBC, 4, 2, 2, 4, 1, 3>(p, 0, kt_main, p.accumulate, stream);
@@ -615,6 +714,17 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
       int st = launch_variant<E, RBC, 2, 2, 2, 2, 1, 3>(p, 0, kt_main, p.accumulate, stream);
       if (st == 0) {
         *name = "mmt4d_mfma_64x64_rhs_direct";
+        if (kt_main == p.K1) return 0;
+        return finish_k(launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+      }
+      if (st > 0) return st;
+    }
+  }
+  if constexpr (NARROW) {
+    if (kt_main > 0 && forced == 15) {
+      int st = launch_narrow<E, RBC, 2, 2, 1>(p, kt_main, stream);
+      if (st == 0) {
+        *name = "mmt4d_mfma_64x64_narrow";
         if (kt_main == p.K1) return 0;
         return finish_k(launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
       }

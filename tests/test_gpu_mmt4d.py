@@ -87,7 +87,9 @@ def _mfma_shapes(M0, N0, K0, bits):
 # bytes wide, else the 32x64 kernel through LDS: the shapes below have both;
 # 5 is the thin kernel on the transposed problem and 6 the same kernel with
 # 64x64 blocks, under the same conditions; 7 is the 256x128 shape, 8 the
-# 128x512 shape).
+# 128x512 shape; 11 is the 64x64 shape with the deep pipeline, and 12 .. 15 are
+# the narrow-row kernels in the 256x256 / 128x512 / 128x128 / 64x64 shape, which
+# serve tile rows of 2 or 4 bytes with N0 = 16 and hand everything else on).
 # Tile rows of one byte (s8, K0 = 1) have no MFMA kernel: iree_uk_mmt4d_info
 # says so and the reference grid above covers them on the scalar kernel. The
 # entry stays in the list, named for what it is, and is asserted unserved.
@@ -97,7 +99,7 @@ def _tile_id(n):
     return name + "_one_byte_rows_have_no_mfma_kernel" if (tf, K0) == (uk.MMT4D_TYPE_S8S8S32, 1) else name
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("n", range(len(MFMA_TILES)), ids=_tile_id)
 def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu

@@ -244,3 +244,41 @@ def test_pack_unpack_random_round_trips_multi_block(gpu):
                    o2, o3, shape[0], shape[1], flags)
         back = d_y.cpu().numpy().view(dtype).reshape(shape)
         assert np.array_equal(back, x), (ci, shape, t0, t1, ti, to, lib.last_kernel_name())
+
+
+def test_mmt4d_random_sweep_narrow_row_kernels(gpu, oracle):
+    """The narrow-row kernels (tile rows of 2 or 4 bytes, N0 = 16: the RHS is
+    read straight into registers with its rows permuted across accumulator
+    blocks, the LHS loader waves take the steps in turns): random tile heights,
+    tile counts ragged against every workgroup shape, K with and without a
+    remainder against the 64-byte step, ACCUMULATE, loose strides, in every
+    shape the kernel is built in (12 .. 15) and as the library chooses (0)."""
+    lib, torch = gpu
+    rng = np.random.default_rng(4242)
+    tiles = [(uk.MMT4D_TYPE_S8S8S32, 2), (uk.MMT4D_TYPE_S8S8S32, 4), (uk.MMT4D_TYPE_F16F16F32, 1),
+             (uk.MMT4D_TYPE_F16F16F32, 2), (uk.MMT4D_TYPE_BF16BF16F32, 2), (uk.MMT4D_TYPE_BF16BF16F32, 1),
+             (uk.MMT4D_TYPE_F32F32F32, 1)]
+    served = set()
+    for ci in range(280):
+        tf, K0 = tiles[ci % len(tiles)]
+        rb = K0 * uk.MMT4D_TYPE_BITS[tf][0] // 8
+        M0 = int(rng.choice([8, 16, 24, 32, 64]))
+        M, N = int(rng.integers(1, 48)), int(rng.integers(1, 48))
+        K = int(rng.integers(1, 900 // rb))
+        if ci % 5 == 0:
+            K = (K // (64 // rb) + 1) * (64 // rb)          # whole steps only
+        acc = uk.MMT4D_ACCUMULATE if rng.integers(0, 2) else 0
+        slack = 16 * int(rng.integers(0, 2))
+        c = T.Mmt4dCase(tf | acc, M, N, K, M0, 16, K0, K * M0 * K0 + slack, K * 16 * K0 + slack,
+                        N * M0 * 16 + slack, slack, 0, slack)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        variant = int(rng.choice([0, 12, 13, 14, 15]))
+        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (ci, c, variant, lib.last_kernel_name())
+        served.add(lib.last_kernel_name())
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    for shape in ("256x256", "128x512", "128x128", "64x64"):
+        assert f"mmt4d_mfma_{shape}_narrow" in served, served
