@@ -338,6 +338,8 @@ TARGET_PACK = {
     # the same matrix between the same two pitches
     "c5_pack_f32_12288x12289": (12288, 49152, 49156, 49152),
     "c5_pack_f32_12289x12288": (12288, 49152, 49152, 49216),
+    # the prefill's RHS pack (1-byte elements, 16x32 tiles: rows of 8192 bytes both sides)
+    "c4_f8_prefill": (28672, 8192, 8192, 8192),
 }
 
 
@@ -449,8 +451,9 @@ def main() -> int:
                     "GBps": round(gbps, 1), "frac": round(gbps / rn.PEAK_HBM_GBPS, 4),
                     "what": f"plain copy of {rows} rows x {row_bytes} B, pitch {sp} -> {dp} B"}
                 keep = w.keep
-                entry["parity"] = {"round_trip_bit_exact": bool(
-                    torch.equal(keep["back"].view(keep["rows"], keep["cols"]), keep["x"]))}
+                if "back" in keep:
+                    entry["parity"] = {"round_trip_bit_exact": bool(
+                        torch.equal(keep["back"].view(keep["rows"], keep["cols"]), keep["x"]))}
             extra[name] = entry
             del w
         result["extra"] = extra
@@ -479,10 +482,12 @@ def main() -> int:
             for pk in ("pack_lhs", "pack_rhs"):
                 if pk in e["kernels"]:
                     t[pk + "_frac"] = round(e["kernels"][pk]["frac"], 3)
+            if "copy2d_ceiling" in e:
+                t["copy2d_frac"] = round(e["copy2d_ceiling"]["frac"], 3)
             targets[name] = t
         for name in TARGET_PACK:
             e = extra.get(name)
-            if not e:
+            if not e or "pack" not in e["kernels"]:
                 continue
             targets[name] = {"pack_frac": round(e["kernels"]["pack"]["frac"], 3),
                              "unpack_frac": round(e["kernels"]["unpack"]["frac"], 3),

@@ -316,8 +316,10 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream, bool al
   a.out_rows = (int32_t)std::min<int64_t>(p.out_rows, INT32_MAX);
   a.out_cols = (int32_t)std::min<int64_t>(p.out_cols, INT32_MAX);
   a.M1 = p.M1; a.N1 = p.N1; a.K1 = p.K1; a.M0 = p.M0; a.N0 = p.N0; a.rb = p.rb; a.lrb = p.lrb;
-  const int64_t grid_m = uk::ceil_div((int64_t)p.M1 * p.M0, TM * 16);
-  const int64_t grid_n = uk::ceil_div((int64_t)p.N1 * p.N0, TN * 16);
+  // Rows and columns that are stored: blocks wholly beyond them (tile padding of
+  // a fused row-major result) are not computed at all.
+  const int64_t grid_m = uk::ceil_div(std::min<int64_t>((int64_t)p.M1 * p.M0, p.out_rows), TM * 16);
+  const int64_t grid_n = uk::ceil_div(std::min<int64_t>((int64_t)p.N1 * p.N0, p.out_cols), TN * 16);
   if (grid_m * grid_n >= (1ll << 31) || p.out_sm0 >= (1ll << 32) || p.out_spn >= (1ll << 32) ||
       p.acc_sm0 >= (1ll << 32) || p.acc_spn >= (1ll << 32)) {
     return -1;
@@ -424,7 +426,10 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   // register quad per block (all types but f8).
   constexpr int BIG_PIPE = RBC >= 16 ? (ElemTraits<E>::kHalves == 1 ? 3 : 2) : 1;
   constexpr int BIG_KS = 64 * H;
-  const int64_t rows_m = (int64_t)p.M1 * p.M0;
+  // Rows / columns that exist in the result (fewer than the tiles hold when a
+  // fused call drops tile padding: a decode step of 16 rows in 32-row tiles).
+  const int64_t rows_m = std::min<int64_t>((int64_t)p.M1 * p.M0, p.out_rows);
+  const int64_t cols_n = std::min<int64_t>((int64_t)p.N1 * p.N0, p.out_cols);
   int choice;
   if (forced == 11 || forced == 15) {
     choice = 3;  // 64x64: the deep pipeline (11) or the narrow-row kernel (15)
@@ -441,7 +446,7 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = forced;
   } else if (rows_m <= (RBC >= 8 ? 64 : 32) && workgroups(p, 32, 64) >= 1) {
     choice = 4;
-  } else if (RBC >= 8 && (int64_t)p.N1 * p.N0 <= 64) {
+  } else if (RBC >= 8 && cols_n <= 64) {
     choice = 5;
   } else if (workgroups(p, 256, 256) >= 192) {
     choice = 1;
@@ -660,14 +665,14 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     // N-thin (a few columns against many rows, e.g. the last column strip of
     // a ragged problem): the thin kernel on the transposed problem.
     if constexpr (RBC >= 8) {
-      int st = thin_launch(std::true_type{}, (int64_t)p.N1 * p.N0, rows_m);
+      int st = thin_launch(std::true_type{}, cols_n, rows_m);
       if (st >= 0) { *name = "mmt4d_mfma_thin_transposed"; return st; }
     }
     choice = 3;
   }
   if (choice == 4) {
     if constexpr (RBC >= 8) {
-      int st = thin_launch(std::false_type{}, rows_m, (int64_t)p.N1 * p.N0);
+      int st = thin_launch(std::false_type{}, rows_m, cols_n);
       if (st >= 0) { *name = "mmt4d_mfma_thin"; return st; }
     }
     // With 2-byte rows a 16-byte piece spans 8 rows and 32 rows do not fill a

@@ -4,7 +4,7 @@
 
 namespace uk_mfma {
 int launch_s8s4(const Problem& p, hipStream_t stream, const char** name) {
-  const int64_t rows_m = (int64_t)p.M1 * p.M0;
+  const int64_t rows_m = std::min<int64_t>((int64_t)p.M1 * p.M0, p.out_rows);  // rows that are stored
   int st;
   if (rows_m <= 16) {
     st = launch_thin<Elem::kS8S4, 16, 1, 2, 4, 4>(p, false, stream, true);
