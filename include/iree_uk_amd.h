@@ -64,6 +64,15 @@ enum {
   IREE_UK_AMD_FLAG_MMT4D_TYPE_F8E4M3FNF8E4M3FNF32 = 0x80,
 };
 
+/* Subnormal f16 / bf16 operands. The reference's generic tile functions read
+ * f16 and bf16 through a software conversion that turns subnormal inputs into
+ * zero (common.h:664-700); its AVX-512 f16 tile function converts with
+ * vcvtph2ps, which keeps them. Here the scalar kernel (GENERIC kernel mode,
+ * and every call no matrix-core kernel serves) flushes them as the generic
+ * tile functions do, bit for bit, and the matrix-core kernels keep them at
+ * their value, as the instruction does. The two therefore differ on inputs
+ * that hold subnormals, by at most the products of the flushed elements. */
+
 /* mmt4d bit flags (exported_bits.h:44-46). */
 enum {
   IREE_UK_FLAG_MMT4D_ACCUMULATE = 0x100,
@@ -326,7 +335,9 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_pointer_mode(int mode);
  *             the call (1 = 256x256, 2 = 128x128, 3 = 64x64, 4 = the M-thin
  *             kernels, 5 = the M-thin kernel on the transposed problem,
  *             6 = the 64x64 K-split kernel, 7 = 256x128, 8 = 128x512,
- *             9 / 10 = the persistent kernel in the 128x512 / 256x256 shape)
+ *             9 / 10 = the persistent kernel in the 128x512 / 256x256 shape,
+ *             11 = 64x64 with the deep pipeline, 12..15 = the narrow-row
+ *             kernels in the 256x256 / 128x512 / 128x128 / 64x64 shapes)
  *             instead of choosing by problem size; pack/unpack as AUTO. */
 enum {
   IREE_UK_AMD_KERNEL_MODE_AUTO = 0,
@@ -426,6 +437,17 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(
 IREE_UK_AMD_EXPORT void iree_uk_amd_timing_begin(void);
 IREE_UK_AMD_EXPORT int iree_uk_amd_timing_end(double* elapsed_us, int* kinds,
                                               int capacity);
+
+/* Host operands (ordinary memory, see the top of this file) are staged
+ * through a device arena owned by the calling thread: one allocation per
+ * device that grows to the largest call's need and is then reused, so that a
+ * caller that always passes host pointers (the HAL executable-plugin thunks)
+ * allocates a handful of times in its life. staging_bytes reports what the
+ * calling thread holds; release_staging frees it (0 or a hipError_t value; a
+ * later host-operand call allocates again). Any pitch is staged, negative and
+ * zero (broadcast) included. No counterpart in the reference. */
+IREE_UK_AMD_EXPORT int64_t iree_uk_amd_staging_bytes(void);
+IREE_UK_AMD_EXPORT int iree_uk_amd_release_staging(void);
 
 /* Number of devices visible to HIP (0 when there is none or no driver). */
 IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);

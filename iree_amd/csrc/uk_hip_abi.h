@@ -71,10 +71,13 @@ int iree_uk_amd_hip_device_count(void);
 /* *is_device = 1 if `ptr` is device-accessible memory known to HIP (device,
  * managed, or registered/pinned host memory), 0 for ordinary host memory. */
 int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device);
-int iree_uk_amd_hip_malloc(void** ptr, int64_t bytes);
-int iree_uk_amd_hip_free(void* ptr);
-/* 2-D copies of `height` rows of `width` bytes; pitches in bytes. Synchronous
- * with respect to the host; ordered after prior work on `stream`. */
+/* The calling thread's staging arena on the current device: one device
+ * allocation that only grows. *base is valid until the thread's next call
+ * that asks for more; whoever uses it synchronizes before reserving again. */
+int iree_uk_amd_hip_staging_reserve(void** base, int64_t bytes);
+/* 2-D copies of `height` rows of `width` bytes; pitches in bytes.
+ * Asynchronous: ordered on `stream`; the host memory must stay untouched
+ * until the stream has been synchronized. */
 int iree_uk_amd_hip_copy2d_to_device(void* dst, int64_t dst_pitch,
                                      const void* src, int64_t src_pitch,
                                      int64_t width, int64_t height,

@@ -145,10 +145,19 @@ static int64_t ceil_pow2(int64_t x) {
  * Staging of host operands.
  *
  * An operand is described as `rows` rows of `row_bytes` bytes, `pitch` bytes
- * apart, starting at `base`. A host operand gets a dense device copy (pitch =
- * row_bytes); only the rows x row_bytes region is ever copied back, so bytes
- * in the stride gaps between rows keep their host values and concurrent
- * calls working on neighbouring slabs do not overwrite each other.
+ * apart (any sign, zero included), starting at `base`. A host operand gets a
+ * device copy carved from the calling thread's staging arena (one grow-only
+ * device allocation per thread, so a call allocates only when it needs more
+ * than any call before it); the copies in and out are asynchronous and the
+ * entry point synchronizes the stream once, before it returns.
+ *   pitch >= row_bytes:   dense copy of the rows (device pitch = row_bytes);
+ *   pitch <= -row_bytes:  the same, rows walked from the lowest address, and
+ *                         the device pitch is -row_bytes;
+ *   |pitch| < row_bytes:  rows overlap (broadcast for pitch 0): the byte range
+ *                         they span is copied whole and the pitch is kept.
+ * Only bytes that belong to a row are ever copied back, so bytes in the
+ * stride gaps keep their host values and concurrent calls working on
+ * neighbouring slabs do not overwrite each other.
  *-------------------------------------------------------------------------*/
 
 typedef struct {
@@ -156,8 +165,25 @@ typedef struct {
   int64_t pitch;     /* caller pitch, bytes */
   int64_t row_bytes; /* bytes per row that the op may touch */
   int64_t rows;
-  void* device;      /* dense device copy, or NULL when used in place */
+  void* device;         /* device address standing for host_base, or NULL when
+                           the operand is used in place */
+  int64_t device_pitch; /* pitch of the device copy, bytes */
+  /* the 2-D copy that moves it: */
+  char* copy_host;
+  int64_t copy_pitch, copy_row_bytes, copy_rows, copy_device_offset, arena_bytes;
+  char* copy_device;
 } staged_t;
+
+static staged_t staged(const void* base, int64_t pitch, int64_t row_bytes,
+                       int64_t rows) {
+  staged_t s;
+  memset(&s, 0, sizeof s);
+  s.host_base = (char*)base;
+  s.pitch = pitch;
+  s.row_bytes = row_bytes;
+  s.rows = rows;
+  return s;
+}
 
 static int is_device_pointer(const void* p, int* status) {
   if (tls_pointer_mode == IREE_UK_AMD_POINTER_MODE_DEVICE) return 1;
@@ -167,38 +193,93 @@ static int is_device_pointer(const void* p, int* status) {
   return is_dev;
 }
 
-/* Prepares operand `s` for the device. `copy_in` says whether the current
- * host contents are needed by the kernel. Returns 0 or a HIP status. */
-static int stage_in(staged_t* s, int copy_in) {
+/* Decides how operand `s` travels; arena_bytes stays 0 for an operand that is
+ * empty or already on the device. Returns 0 or a HIP status. */
+static int stage_plan(staged_t* s) {
   s->device = 0;
+  s->arena_bytes = 0;
   if (s->rows <= 0 || s->row_bytes <= 0) return 0;
   int st = 0;
   if (is_device_pointer(s->host_base, &st)) return st;
   if (st) return st;
-  st = iree_uk_amd_hip_malloc(&s->device, s->rows * s->row_bytes);
-  if (st) return st;
-  if (copy_in) {
-    st = iree_uk_amd_hip_copy2d_to_device(s->device, s->row_bytes, s->host_base,
-                                          s->pitch, s->row_bytes, s->rows,
-                                          tls_stream);
+  const int64_t last = (s->rows - 1) * s->pitch; /* offset of the last row */
+  if (s->rows == 1 || s->pitch >= s->row_bytes) {
+    s->copy_host = s->host_base;
+    s->copy_pitch = s->rows == 1 ? s->row_bytes : s->pitch;
+    s->copy_row_bytes = s->row_bytes;
+    s->copy_rows = s->rows;
+    s->copy_device_offset = 0;
+    s->device_pitch = s->row_bytes;
+  } else if (s->pitch <= -s->row_bytes) {
+    s->copy_host = s->host_base + last;
+    s->copy_pitch = -s->pitch;
+    s->copy_row_bytes = s->row_bytes;
+    s->copy_rows = s->rows;
+    s->copy_device_offset = (s->rows - 1) * s->row_bytes;
+    s->device_pitch = -s->row_bytes;
+  } else {
+    const int64_t lowest = last < 0 ? last : 0;
+    s->copy_host = s->host_base + lowest;
+    s->copy_row_bytes = (last < 0 ? -last : last) + s->row_bytes;
+    s->copy_pitch = s->copy_row_bytes;
+    s->copy_rows = 1;
+    s->copy_device_offset = -lowest;
+    s->device_pitch = s->pitch;
   }
-  return st;
+  s->arena_bytes = (s->copy_row_bytes * s->copy_rows + 255) & ~(int64_t)255;
+  return 0;
+}
+
+/* Gives every host operand of `ops` its device copy and starts the copies in
+ * (`copy_in[i]` says whether the kernel needs operand i's current contents).
+ * Returns 0 or a HIP status. */
+static int stage_in(staged_t** ops, const int* copy_in, int count) {
+  int64_t total = 0;
+  for (int i = 0; i < count; ++i) {
+    int st = stage_plan(ops[i]);
+    if (st) return st;
+    total += ops[i]->arena_bytes;
+  }
+  if (!total) return 0;
+  void* arena = 0;
+  int st = iree_uk_amd_hip_staging_reserve(&arena, total);
+  if (st) return st;
+  char* next = (char*)arena;
+  for (int i = 0; i < count; ++i) {
+    staged_t* s = ops[i];
+    if (!s->arena_bytes) continue;
+    s->copy_device = next;
+    s->device = next + s->copy_device_offset;
+    next += s->arena_bytes;
+    if (!copy_in[i]) continue;
+    st = iree_uk_amd_hip_copy2d_to_device(s->copy_device, s->copy_row_bytes,
+                                          s->copy_host, s->copy_pitch,
+                                          s->copy_row_bytes, s->copy_rows,
+                                          tls_stream);
+    if (st) return st;
+  }
+  return 0;
 }
 
 static int stage_out(staged_t* s) {
   if (!s->device) return 0;
-  return iree_uk_amd_hip_copy2d_to_host(s->host_base, s->pitch, s->device,
-                                        s->row_bytes, s->row_bytes, s->rows,
+  return iree_uk_amd_hip_copy2d_to_host(s->copy_host, s->copy_pitch,
+                                        s->copy_device, s->copy_row_bytes,
+                                        s->copy_row_bytes, s->copy_rows,
                                         tls_stream);
 }
 
-static void stage_free(staged_t* s) {
-  if (s->device) {
-    /* Device work that reads the staging buffer has completed: the only
-     * callers free after a synchronous copy-out or a stream synchronize. */
-    iree_uk_amd_hip_free(s->device);
-    s->device = 0;
+/* Ends a call that staged something: waits for the kernel and the copies, so
+ * the caller's memory is final (and free to reuse) when the entry point
+ * returns, and the arena is free for the thread's next call. */
+static int stage_finish(int st, staged_t** ops, int count) {
+  int any = 0;
+  for (int i = 0; i < count; ++i) any |= ops[i]->device != 0;
+  if (any) {
+    int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
+    if (!st) st = st2;
   }
+  return st;
 }
 
 /*---------------------------------------------------------------------------
@@ -272,15 +353,15 @@ static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
   if (rowmajor) rm = *rowmajor;
   else memset(&rm, 0, sizeof rm);
   const int out_bytes = bits.out_bits / 8;
-  staged_t lhs = {(char*)p.lhs_buffer + p.lhs_offset * bits.lhs_bits / 8,
+  staged_t lhs = staged((char*)p.lhs_buffer + p.lhs_offset * bits.lhs_bits / 8,
                   p.lhs_stride0 * bits.lhs_bits / 8,
-                  p.K * p.M0 * p.K0 * bits.lhs_bits / 8, p.M, 0};
-  staged_t rhs = {(char*)p.rhs_buffer + p.rhs_offset * bits.rhs_bits / 8,
+                  p.K * p.M0 * p.K0 * bits.lhs_bits / 8, p.M);
+  staged_t rhs = staged((char*)p.rhs_buffer + p.rhs_offset * bits.rhs_bits / 8,
                   p.rhs_stride0 * bits.rhs_bits / 8,
-                  p.K * p.N0 * p.K0 * bits.rhs_bits / 8, p.N, 0};
-  staged_t out = {(char*)p.out_buffer + p.out_offset * out_bytes,
+                  p.K * p.N0 * p.K0 * bits.rhs_bits / 8, p.N);
+  staged_t out = staged((char*)p.out_buffer + p.out_offset * out_bytes,
                   p.out_stride0 * out_bytes, p.N * p.M0 * p.N0 * out_bytes,
-                  p.M, 0};
+                  p.M);
   if (rowmajor) {
     out.pitch = rm.stride0 * out_bytes;
     out.row_bytes = rm.size1 * out_bytes;
@@ -290,7 +371,7 @@ static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
    * initial accumulators (ACCUMULATE) come from a tiled buffer of their own. */
   const int dequant = rowmajor && rm.dequant;
   const int accumulate = (p.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0;
-  staged_t acc = {0, 0, 0, 0, 0}, rscale = {0, 0, 0, 0, 0}, cscale = {0, 0, 0, 0, 0};
+  staged_t acc = staged(0, 0, 0, 0), rscale = acc, cscale = acc;
   if (dequant) {
     if (accumulate) {
       acc.host_base = (char*)rm.acc;
@@ -309,50 +390,37 @@ static void mmt4d_run(const iree_uk_mmt4d_params_t* params,
       cscale.rows = 1;
     }
   }
-  int st = stage_in(&lhs, 1);
-  if (!st) st = stage_in(&rhs, 1);
-  if (!st) st = stage_in(&out, accumulate && !dequant);
-  if (!st) st = stage_in(&acc, 1);
-  if (!st) st = stage_in(&rscale, 1);
-  if (!st) st = stage_in(&cscale, 1);
+  staged_t* ops[6] = {&lhs, &rhs, &out, &acc, &rscale, &cscale};
+  const int copy_in[6] = {1, 1, accumulate && !dequant, 1, 1, 1};
+  int st = stage_in(ops, copy_in, 6);
   if (!st) {
     if (acc.device) {
       rm.acc = acc.device;
-      rm.acc_stride0 = p.N * p.M0 * p.N0;
+      rm.acc_stride0 = acc.device_pitch / out_bytes;
     }
     if (rscale.device) rm.row_scale = (const float*)rscale.device;
     if (cscale.device) rm.col_scale = (const float*)cscale.device;
     if (lhs.device) {
       p.lhs_buffer = lhs.device;
       p.lhs_offset = 0;
-      p.lhs_stride0 = p.K * p.M0 * p.K0;
+      p.lhs_stride0 = lhs.device_pitch * 8 / bits.lhs_bits;
     }
     if (rhs.device) {
       p.rhs_buffer = rhs.device;
       p.rhs_offset = 0;
-      p.rhs_stride0 = p.K * p.N0 * p.K0;
+      p.rhs_stride0 = rhs.device_pitch * 8 / bits.rhs_bits;
     }
     if (out.device) {
       p.out_buffer = out.device;
       p.out_offset = 0;
-      p.out_stride0 = p.N * p.M0 * p.N0;
-      rm.stride0 = rm.size1;
+      p.out_stride0 = out.device_pitch / out_bytes;
+      rm.stride0 = out.device_pitch / out_bytes;
     }
     st = iree_uk_amd_hip_launch_mmt4d(&p, rowmajor ? &rm : 0, tls_stream,
                                       tls_kernel_mode, &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
-  if (lhs.device || rhs.device || out.device || acc.device || rscale.device ||
-      cscale.device) {
-    int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
-    if (!st) st = st2;
-  }
-  stage_free(&lhs);
-  stage_free(&rhs);
-  stage_free(&out);
-  stage_free(&acc);
-  stage_free(&rscale);
-  stage_free(&cscale);
+  st = stage_finish(st, ops, 6);
   tls_status = st;
 }
 
@@ -580,33 +648,29 @@ void iree_uk_pack_p(const iree_uk_pack_params_t* params) {
    * apart. Gaps inside a row are copied along (reading them is harmless). */
   const int64_t in_row_elems =
       p.in_size1 > 0 ? (p.in_size1 - 1) * p.in_stride1 + 1 : 0;
-  staged_t in = {(char*)p.in_buffer + p.in_offset * es, p.in_stride0 * es,
-                 in_row_elems * es, p.in_size0, 0};
-  staged_t out = {(char*)p.out_buffer + p.out_offset * es, p.out_stride0 * es,
-                  p.out_size1 * p.out_size2 * p.out_size3 * es, p.out_size0, 0};
-  int st = stage_in(&in, 1);
-  if (!st) st = stage_in(&out, 0); /* every byte of every tile is written */
+  staged_t in = staged((char*)p.in_buffer + p.in_offset * es, p.in_stride0 * es,
+                 in_row_elems * es, p.in_size0);
+  staged_t out = staged((char*)p.out_buffer + p.out_offset * es, p.out_stride0 * es,
+                  p.out_size1 * p.out_size2 * p.out_size3 * es, p.out_size0);
+  staged_t* ops[2] = {&in, &out};
+  const int copy_in[2] = {1, 0}; /* every byte of every tile is written */
+  int st = stage_in(ops, copy_in, 2);
   if (!st) {
     if (in.device) {
       p.in_buffer = in.device;
       p.in_offset = 0;
-      p.in_stride0 = in_row_elems;
+      p.in_stride0 = in.device_pitch / es;
     }
     if (out.device) {
       p.out_buffer = out.device;
       p.out_offset = 0;
-      p.out_stride0 = p.out_size1 * p.out_size2 * p.out_size3;
+      p.out_stride0 = out.device_pitch / es;
     }
     st = iree_uk_amd_hip_launch_pack(&p, tls_stream, tls_kernel_mode,
                                      &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
-  if (in.device || out.device) {
-    int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
-    if (!st) st = st2;
-  }
-  stage_free(&in);
-  stage_free(&out);
+  st = stage_finish(st, ops, 2);
   tls_status = st;
 }
 
@@ -671,36 +735,32 @@ void iree_uk_unpack_p(const iree_uk_unpack_params_t* params) {
   const int es = unpack_elem_bytes(params->flags);
   iree_uk_unpack_params_t p = *params;
   const int64_t out_row_elems = (p.out_size1 - 1) * p.out_stride1 + 1;
-  staged_t in = {(char*)p.in_buffer + p.in_offset * es, p.in_stride0 * es,
-                 p.in_size1 * p.in_size2 * p.in_size3 * es, p.in_size0, 0};
-  staged_t out = {(char*)p.out_buffer + p.out_offset * es, p.out_stride0 * es,
-                  out_row_elems * es, p.out_size0, 0};
-  int st = stage_in(&in, 1);
+  staged_t in = staged((char*)p.in_buffer + p.in_offset * es, p.in_stride0 * es,
+                 p.in_size1 * p.in_size2 * p.in_size3 * es, p.in_size0);
+  staged_t out = staged((char*)p.out_buffer + p.out_offset * es, p.out_stride0 * es,
+                  out_row_elems * es, p.out_size0);
   /* With a unit inner stride every byte of each destination row is written.
    * Otherwise the bytes between elements must survive the round trip, so the
    * rows are copied in first (and come back unchanged). */
-  if (!st) st = stage_in(&out, p.out_stride1 != 1);
+  staged_t* ops[2] = {&in, &out};
+  const int copy_in[2] = {1, p.out_stride1 != 1};
+  int st = stage_in(ops, copy_in, 2);
   if (!st) {
     if (in.device) {
       p.in_buffer = in.device;
       p.in_offset = 0;
-      p.in_stride0 = p.in_size1 * p.in_size2 * p.in_size3;
+      p.in_stride0 = in.device_pitch / es;
     }
     if (out.device) {
       p.out_buffer = out.device;
       p.out_offset = 0;
-      p.out_stride0 = out_row_elems;
+      p.out_stride0 = out.device_pitch / es;
     }
     st = iree_uk_amd_hip_launch_unpack(&p, tls_stream, tls_kernel_mode,
                                        &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
-  if (in.device || out.device) {
-    int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
-    if (!st) st = st2;
-  }
-  stage_free(&in);
-  stage_free(&out);
+  st = stage_finish(st, ops, 2);
   tls_status = st;
 }
 
@@ -801,15 +861,15 @@ void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params) {
   const int64_t out_span = (p.N - 1) * p.output_stride_n +
                            (p.OC_outer - 1) * p.output_stride_oc_outer +
                            (p.OH - 1) * p.output_stride_oh + p.OW * (int64_t)p.k0;
-  staged_t in = {(char*)p.input_buffer + p.input_offset * 4, in_span * 4,
-                 in_span * 4, in_span > 0 ? 1 : 0, 0};
-  staged_t flt = {(char*)p.filter_buffer + p.filter_offset * 4, f_span * 4,
-                  f_span * 4, f_span > 0 ? 1 : 0, 0};
-  staged_t out = {(char*)p.output_buffer + p.output_offset * 4, out_span * 4,
-                  out_span * 4, 1, 0};
-  int st = stage_in(&in, 1);
-  if (!st) st = stage_in(&flt, 1);
-  if (!st) st = stage_in(&out, 1);
+  staged_t in = staged((char*)p.input_buffer + p.input_offset * 4, in_span * 4,
+                 in_span * 4, in_span > 0 ? 1 : 0);
+  staged_t flt = staged((char*)p.filter_buffer + p.filter_offset * 4, f_span * 4,
+                  f_span * 4, f_span > 0 ? 1 : 0);
+  staged_t out = staged((char*)p.output_buffer + p.output_offset * 4, out_span * 4,
+                  out_span * 4, 1);
+  staged_t* ops[3] = {&in, &flt, &out};
+  const int copy_in[3] = {1, 1, 1};
+  int st = stage_in(ops, copy_in, 3);
   if (!st) {
     if (in.device) { p.input_buffer = in.device; p.input_offset = 0; }
     if (flt.device) { p.filter_buffer = flt.device; p.filter_offset = 0; }
@@ -818,13 +878,7 @@ void iree_uk_conv_nchwc_p(const iree_uk_conv_nchwc_params_t* params) {
                                            &tls_kernel_name);
   }
   if (!st) st = stage_out(&out);
-  if (in.device || flt.device || out.device) {
-    int st2 = iree_uk_amd_hip_stream_synchronize(tls_stream);
-    if (!st) st = st2;
-  }
-  stage_free(&in);
-  stage_free(&flt);
-  stage_free(&out);
+  st = stage_finish(st, ops, 3);
   tls_status = st;
 }
 

@@ -78,36 +78,89 @@ int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device) {
   return 0;
 }
 
-int iree_uk_amd_hip_malloc(void** ptr, int64_t bytes) {
-  return (int)hipMalloc(ptr, (size_t)bytes);
+namespace {
+// Staging arenas of the calling thread, one per device it has staged on.
+// Grow-only and kept until iree_uk_amd_release_staging or process end: a
+// thread that keeps passing host operands allocates a handful of times in
+// its life instead of several times per call.
+struct StagingArena {
+  int device;
+  void* base;
+  size_t bytes;
+};
+thread_local std::vector<StagingArena> g_staging;
+}  // namespace
+
+int iree_uk_amd_hip_staging_reserve(void** base, int64_t bytes) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return (int)err;
+  StagingArena* arena = nullptr;
+  for (StagingArena& a : g_staging) {
+    if (a.device == dev) arena = &a;
+  }
+  if (!arena) {
+    g_staging.push_back(StagingArena{dev, nullptr, 0});
+    arena = &g_staging.back();
+  }
+  if (arena->bytes < (size_t)bytes) {
+    // The previous user synchronized before returning: nothing in flight
+    // reads the old block.
+    if (arena->base) (void)hipFree(arena->base);
+    arena->base = nullptr;
+    arena->bytes = 0;
+    size_t want = 1u << 20;
+    while (want < (size_t)bytes) want <<= 1;
+    // Above 256 MiB grow by what is asked, rounded to 64 MiB, not by doubling.
+    if (want > (256u << 20)) want = ((size_t)bytes + (64u << 20) - 1) / (64u << 20) * (64u << 20);
+    err = hipMalloc(&arena->base, want);
+    if (err != hipSuccess) {
+      arena->base = nullptr;
+      return (int)err;
+    }
+    arena->bytes = want;
+  }
+  *base = arena->base;
+  return 0;
 }
 
-int iree_uk_amd_hip_free(void* ptr) { return (int)hipFree(ptr); }
+extern "C" IREE_UK_AMD_EXPORT int64_t iree_uk_amd_staging_bytes(void) {
+  int64_t total = 0;
+  for (const StagingArena& a : g_staging) total += (int64_t)a.bytes;
+  return total;
+}
+
+extern "C" IREE_UK_AMD_EXPORT int iree_uk_amd_release_staging(void) {
+  int status = 0;
+  int current = 0;
+  (void)hipGetDevice(&current);
+  for (StagingArena& a : g_staging) {
+    if (!a.base) continue;
+    (void)hipSetDevice(a.device);
+    const hipError_t err = hipFree(a.base);
+    if (err != hipSuccess && !status) status = (int)err;
+  }
+  (void)hipSetDevice(current);
+  g_staging.clear();
+  return status;
+}
 
 int iree_uk_amd_hip_copy2d_to_device(void* dst, int64_t dst_pitch,
                                      const void* src, int64_t src_pitch,
                                      int64_t width, int64_t height,
                                      void* stream) {
-  hipError_t err =
-      hipMemcpy2DAsync(dst, (size_t)dst_pitch, src, (size_t)src_pitch,
-                       (size_t)width, (size_t)height, hipMemcpyHostToDevice,
-                       (hipStream_t)stream);
-  if (err != hipSuccess) return (int)err;
-  // Pageable host memory: the caller may reuse or free `src` right after the
-  // entry point returns, so wait for the copy.
-  return (int)hipStreamSynchronize((hipStream_t)stream);
+  return (int)hipMemcpy2DAsync(dst, (size_t)dst_pitch, src, (size_t)src_pitch,
+                               (size_t)width, (size_t)height,
+                               hipMemcpyHostToDevice, (hipStream_t)stream);
 }
 
 int iree_uk_amd_hip_copy2d_to_host(void* dst, int64_t dst_pitch,
                                    const void* src, int64_t src_pitch,
                                    int64_t width, int64_t height,
                                    void* stream) {
-  hipError_t err =
-      hipMemcpy2DAsync(dst, (size_t)dst_pitch, src, (size_t)src_pitch,
-                       (size_t)width, (size_t)height, hipMemcpyDeviceToHost,
-                       (hipStream_t)stream);
-  if (err != hipSuccess) return (int)err;
-  return (int)hipStreamSynchronize((hipStream_t)stream);
+  return (int)hipMemcpy2DAsync(dst, (size_t)dst_pitch, src, (size_t)src_pitch,
+                               (size_t)width, (size_t)height,
+                               hipMemcpyDeviceToHost, (hipStream_t)stream);
 }
 
 int iree_uk_amd_hip_stream_synchronize(void* stream) {

@@ -185,6 +185,8 @@ class UKernelLibrary:
         L.iree_uk_amd_version.restype = ctypes.c_char_p
         L.iree_uk_amd_set_assert_handler.argtypes = [_vp]
         L.iree_uk_amd_timing_begin.restype = None
+        L.iree_uk_amd_staging_bytes.restype = _i64
+        L.iree_uk_amd_release_staging.restype = ctypes.c_int
         L.iree_uk_amd_timing_end.argtypes = [_vp, _vp, ctypes.c_int]
         L.iree_uk_amd_timing_end.restype = ctypes.c_int
         L.iree_uk_amd_probe_mfma_peak.argtypes = [_u32, _vp, _i64, ctypes.c_int, ctypes.c_int, _vp,
@@ -376,6 +378,14 @@ class UKernelLibrary:
         n = self.lib.iree_uk_amd_timing_end(us, kinds, capacity)
         n = min(n, capacity)
         return [(kinds[i], us[i]) for i in range(n)]
+
+    def staging_bytes(self) -> int:
+        """Device bytes the calling thread's host-operand staging arena holds."""
+        return int(self.lib.iree_uk_amd_staging_bytes())
+
+    def release_staging(self) -> int:
+        """Frees the calling thread's staging arena; 0 or a hipError_t value."""
+        return int(self.lib.iree_uk_amd_release_staging())
 
     def device_count(self) -> int:
         return int(self.lib.iree_uk_amd_device_count())

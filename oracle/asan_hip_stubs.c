@@ -97,13 +97,18 @@ int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device) {
   return 0;
 }
 
-int iree_uk_amd_hip_malloc(void** ptr, int64_t bytes) {
-  *ptr = calloc(1, bytes > 0 ? (size_t)bytes : 1);
-  return *ptr ? 0 : 2; /* hipErrorOutOfMemory */
+/* A fresh block of exactly the size asked for on every call, so that the
+ * sanitizer sees an overrun of the arena as a whole. */
+static void* g_arena;
+int iree_uk_amd_hip_staging_reserve(void** base, int64_t bytes) {
+  free(g_arena);
+  g_arena = calloc(1, bytes > 0 ? (size_t)bytes : 1);
+  *base = g_arena;
+  return g_arena ? 0 : 2; /* hipErrorOutOfMemory */
 }
-int iree_uk_amd_hip_free(void* ptr) {
-  free(ptr);
-  return 0;
+void asan_stubs_release(void) {
+  free(g_arena);
+  g_arena = 0;
 }
 
 static int copy2d(void* dst, int64_t dst_pitch, const void* src, int64_t src_pitch, int64_t width,

@@ -28,6 +28,7 @@ int uk_oracle_unpack(const void*, int64_t, int64_t, int64_t, void*, int64_t, int
                      int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, uint32_t,
                      const uint64_t*);
 const void* iree_hal_executable_plugin_query(uint32_t max_version, void* reserved);
+void asan_stubs_release(void); /* asan_hip_stubs.c: frees its stand-in for the staging arena */
 
 static int failures = 0;
 static int violations = 0;
@@ -80,6 +81,42 @@ static void mmt4d_case(uint32_t type, int lb, int rb, int ob, int M, int N, int 
   uint8_t* out_b = clone(out_a, obytes);
   CHECK(uk_oracle_mmt4d(lhs, off, ls, rhs, off, rs, out_a, off, os, M, N, K, M0, N0, K0, flags, 0) == 0);
   iree_uk_mmt4d(lhs, off, ls, rhs, off, rs, out_b, off, os, M, N, K, M0, N0, K0, flags, 0);
+  CHECK(iree_uk_amd_last_status() == 0);
+  CHECK(memcmp(out_a, out_b, obytes) == 0);
+  free(lhs); free(rhs); free(out_a); free(out_b);
+}
+
+/* Row pitches that a dense 2-D copy cannot express: `mode` 0 loose positive,
+ * 1 negative (rows walked downwards in memory), 2 zero (every row the same
+ * memory), 3 and 4 positive and negative pitches shorter than a row (rows
+ * overlap). The buffer holds exactly the spanned range. */
+static int64_t pitch_of(int mode, int64_t dense) {
+  switch (mode) {
+    case 1: return -(dense + 2);
+    case 2: return 0;
+    case 3: return dense / 2;
+    case 4: return -(dense / 2);
+    default: return dense + 2;
+  }
+}
+static void mmt4d_pitch_case(uint32_t type, int lb, int rb, int ob, int lhs_mode, int rhs_mode,
+                             int out_mode, int accumulate) {
+  enum { M = 3, N = 2, K = 2, M0 = 4, N0 = 4, K0 = 2 };
+  const uint32_t flags = type | (accumulate ? IREE_UK_FLAG_MMT4D_ACCUMULATE : 0) |
+                         IREE_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION;
+  const int64_t dl = K * M0 * K0, dr = K * N0 * K0, dout = N * M0 * N0;
+  const int64_t ls = pitch_of(lhs_mode, dl), rs = pitch_of(rhs_mode, dr), os = pitch_of(out_mode, dout);
+  const int64_t loff = ls < 0 ? -(M - 1) * ls : 0, roff = rs < 0 ? -(N - 1) * rs : 0,
+                ooff = os < 0 ? -(M - 1) * os : 0;
+  const size_t lbytes = (size_t)(((M - 1) * (ls < 0 ? -ls : ls) + dl) * lb / 8),
+               rbytes = (size_t)(((N - 1) * (rs < 0 ? -rs : rs) + dr) * rb / 8),
+               obytes = (size_t)(((M - 1) * (os < 0 ? -os : os) + dout) * ob / 8);
+  uint8_t* lhs = random_bytes(lbytes, 0);
+  uint8_t* rhs = random_bytes(rbytes, 0);
+  uint8_t* out_a = random_bytes(obytes, 0);
+  uint8_t* out_b = clone(out_a, obytes);
+  CHECK(uk_oracle_mmt4d(lhs, loff, ls, rhs, roff, rs, out_a, ooff, os, M, N, K, M0, N0, K0, flags, 0) == 0);
+  iree_uk_mmt4d(lhs, loff, ls, rhs, roff, rs, out_b, ooff, os, M, N, K, M0, N0, K0, flags, 0);
   CHECK(iree_uk_amd_last_status() == 0);
   CHECK(memcmp(out_a, out_b, obytes) == 0);
   free(lhs); free(rhs); free(out_a); free(out_b);
@@ -185,6 +222,18 @@ int main(void) {
     }
   }
   CHECK(violations == 0);
+  /* Negative, zero and overlapping row pitches on host operands; the output
+   * with a negative pitch (overlapping output rows have no defined result). */
+  for (int lm = 0; lm <= 4; ++lm) {
+    for (int rm = 0; rm <= 4; ++rm) {
+      for (int om = 0; om <= 1; ++om) {
+        mmt4d_pitch_case(IREE_UK_FLAG_MMT4D_TYPE_S8S8S32, 8, 8, 32, lm, rm, om, (lm + rm) & 1);
+        mmt4d_pitch_case(IREE_UK_FLAG_MMT4D_TYPE_S8S4S32, 8, 4, 32, lm, rm, om, rm & 1);
+        mmt4d_pitch_case(IREE_UK_FLAG_MMT4D_TYPE_S16S16S32, 16, 16, 32, lm, rm, om, lm & 1);
+      }
+    }
+  }
+  CHECK(violations == 0);
   for (int slack = 0; slack <= 3; slack += 3) {
     for (uint32_t tr = 0; tr <= 0x300; tr += 0x100) {
       pack_unpack_case(IREE_UK_FLAG_PACK_TYPE_I8I8, 1, 7, 13, 4, 8, tr, slack);
@@ -229,6 +278,7 @@ int main(void) {
   CHECK(iree_uk_mmt4d_info(16, 16, 2, IREE_UK_FLAG_MMT4D_TYPE_S8S8S32, 0) == 0);
   plugin_checks();
   iree_uk_amd_set_assert_handler(0);
+  asan_stubs_release();
   if (failures) {
     fprintf(stderr, "asan_host_driver: %d check(s) failed\n", failures);
     return 1;

@@ -248,6 +248,92 @@ def test_mmt4d_host_pointers_are_staged(gpu, oracle):
         assert np.array_equal(got, want), c.label()
 
 
+def _pow2_bits(tf, exponent: int) -> int:
+    """Bit pattern of 2**exponent as an f16 or bf16 element (subnormals included)."""
+    if tf in (uk.MMT4D_TYPE_F16F16F32, uk.MMT4D_TYPE_F16F16F16):
+        return int(np.float16(2.0 ** exponent).view(np.uint16))
+    return int(np.float32(2.0 ** exponent).view(np.uint32) >> 16)
+
+
+@pytest.mark.parametrize("tf,sub_e,big_e", [(uk.MMT4D_TYPE_F16F16F32, -20, 10),
+                                             (uk.MMT4D_TYPE_BF16BF16F32, -130, 100)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 8])
+def test_mmt4d_subnormal_inputs_matrix_cores_keep_scalar_kernel_flushes(gpu, oracle, tf, sub_e, big_e, variant):
+    """Pins how subnormal f16 / bf16 inputs are read. The reference's generic
+    tile functions flush them to zero (common.h:664-700), and so do the oracle
+    and the scalar kernel, bit for bit. The matrix-core kernels keep them, as
+    the instruction does (and as the reference's own AVX-512 f16 tile function
+    does through vcvtph2ps). Powers of two keep every product and sum exact, so
+    both expectations are exact: LHS = one subnormal value, RHS = one large
+    value, each output K*K0 products."""
+    lib, torch = gpu
+    M0 = N0 = K0 = 16
+    M, N, K = (1, 8, 8) if variant == 4 else (32, 32, 8)
+    lhs = np.full(M * K * M0 * K0, _pow2_bits(tf, sub_e), dtype=np.uint16)
+    rhs = np.full(N * K * N0 * K0, _pow2_bits(tf, big_e), dtype=np.uint16)
+    out0 = np.zeros(M * N * M0 * N0, dtype=np.float32)
+    flags = tf | 0x200
+    flushed = out0.copy()
+    oracle.mmt4d(lhs, 0, K * M0 * K0, rhs, 0, K * N0 * K0, flushed, 0, N * M0 * N0, M, N, K, M0, N0, K0, flags)
+    assert not flushed.any()          # the reference semantics: every product is 0 * big
+    kept = np.full_like(out0, np.float32(K * K0 * 2.0 ** (sub_e + big_e)))
+    d = [T.DeviceBytes(torch, a) for a in (lhs, rhs, out0)]
+    for mode, want, prefix in ((uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO,
+                                kept, "mmt4d_mfma"),
+                               (uk.KERNEL_MODE_GENERIC, flushed, "mmt4d_generic")):
+        lib.set_kernel_mode(mode)
+        try:
+            lib.mmt4d(d[0].ptr, 0, K * M0 * K0, d[1].ptr, 0, K * N0 * K0, d[2].ptr, 0, N * M0 * N0,
+                      M, N, K, M0, N0, K0, flags)
+            lib.synchronize()
+        finally:
+            lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+        assert lib.last_kernel_name().startswith(prefix), lib.last_kernel_name()
+        assert np.array_equal(d[2].numpy().view(np.float32), want), lib.last_kernel_name()
+
+
+def _pitch(mode: int, dense: int) -> int:
+    """Row pitches a dense 2-D copy cannot express: 0 loose, 1 negative,
+    2 zero (broadcast), 3 / 4 shorter than a row (overlapping rows), + and -."""
+    return {0: dense + 2, 1: -(dense + 2), 2: 0, 3: dense // 2, 4: -(dense // 2)}[mode]
+
+
+@pytest.mark.parametrize("tf,M0,N0,K0", [(uk.MMT4D_TYPE_S8S8S32, 16, 16, 16),
+                                         (uk.MMT4D_TYPE_S8S8S32, 16, 16, 2),
+                                         (uk.MMT4D_TYPE_S16S16S32, 8, 8, 2)])
+def test_mmt4d_host_operands_with_negative_zero_and_overlapping_pitches(gpu, oracle, tf, M0, N0, K0):
+    """Strides that are legal for mmt4d (the reference only does pointer
+    arithmetic with them, mmt4d.c:70-83) survive the staging of host operands:
+    negative (rows walked downwards), zero (every row panel the same memory)
+    and shorter than a row; the output with a negative stride."""
+    lib, torch = gpu
+    lb, rb, ob = uk.MMT4D_TYPE_BITS[tf]
+    M, N, K = 3, 5, 8
+    dl, dr, dout = K * M0 * K0, K * N0 * K0, N * M0 * N0
+    rng = np.random.default_rng(77)
+    before = lib.staging_bytes()
+    for lm in range(5):
+        for rm in range(5):
+            for om in (0, 1):
+                ls, rs, os_ = _pitch(lm, dl), _pitch(rm, dr), _pitch(om, dout)
+                loff, roff, ooff = (max(0, -(M - 1) * ls), max(0, -(N - 1) * rs), max(0, -(M - 1) * os_))
+                lhs = rng.integers(0, 256, ((M - 1) * abs(ls) + dl) * lb // 8, dtype=np.uint8)
+                rhs = rng.integers(0, 256, ((N - 1) * abs(rs) + dr) * rb // 8, dtype=np.uint8)
+                out0 = rng.integers(0, 256, ((M - 1) * abs(os_) + dout) * ob // 8, dtype=np.uint8)
+                flags = tf | (uk.MMT4D_ACCUMULATE if (lm + rm) & 1 else 0) | 0x200
+                want = out0.copy()
+                oracle.mmt4d(lhs, loff, ls, rhs, roff, rs, want, ooff, os_, M, N, K, M0, N0, K0, flags)
+                got = out0.copy()
+                lib.mmt4d(lhs.ctypes.data, loff, ls, rhs.ctypes.data, roff, rs, got.ctypes.data, ooff, os_,
+                          M, N, K, M0, N0, K0, flags)
+                assert np.array_equal(got, want), (lm, rm, om, lib.last_kernel_name())
+    # The copies came out of the thread's arena: it grew at most once per size
+    # class, not once per call, and can be handed back.
+    held = lib.staging_bytes()
+    assert held >= before and held > 0
+    assert lib.release_staging() == 0 and lib.staging_bytes() == 0
+
+
 def test_entry_points_from_concurrent_threads(gpu, oracle):
     """The entry points are re-entrant (runtime/src/iree/builtins/ukernel/
     README.md:26): four host threads, each on its own slab of one problem
