@@ -988,7 +988,14 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   // is what bounds them (f32 12288x12289 unpack: 3.3 -> 4.1 TB/s). Smaller
   // problems keep the small blocks: they need the parallelism.
   const int64_t total_bytes = v.outer0 * v.outer1 * tile_bytes;
-  const bool big = allow_big && G == 4 && VEC == 16 && total_bytes >= (192ll << 20);
+  // Whole tile rows as granules (16 bytes contiguous on both sides, no
+  // transposition) gain from the 64 KB blocks too, from smaller sizes on for
+  // pack than for unpack (f8 28672x8192 pack: 85 -> 65 us; f16 4096x4096
+  // pack: 10.6 -> 10.0 us, slower below that; f32 8192x8192 unpack: 98 -> 74
+  // us, f32 4096x4096 unpack: 19.3 -> 20.0 us).
+  const bool big_transposing = G == 4 && total_bytes >= (192ll << 20);
+  const bool big_rows = G == 16 && !to && total_bytes >= ((mat_is_dest ? 192ll : 24ll) << 20);
+  const bool big = allow_big && VEC == 16 && (big_transposing || big_rows);
   const int64_t kMinSpan = big ? 512 : 256;                      // bytes, both sides
   const int64_t kTarget = big ? kStreamBigBlockBytes : kStreamBlockBytes;  // bytes per block, about
   const int64_t stream_block = kTarget;
@@ -1150,16 +1157,25 @@ bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
   const uint32_t lds = 2 * plan.args.lds_buf_bytes;
   if (plan.big) {
     // One workgroup per CU: two 66 KB buffers fill its LDS.
-    if (!(plan.G == 4 && plan.VEC == 16 && plan.MV == 16)) return false;
+    if (!((plan.G == 4 || plan.G == 16) && plan.VEC == 16 && plan.MV == 16)) return false;
     constexpr int kBigThreads = 1024;
-    auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes, kBigThreads, 1>;
+    if (lds > 160 * 1024) return false;
+    auto launch_big = [&](auto kernel, hipError_t attr) {
+      if (attr != hipSuccess) return false;
+      uk::launch(UNPACK ? 1 : 0, kernel, dim3(nblocks < 256 ? nblocks : 256), dim3(kBigThreads), lds,
+                 stream, plan.args);
+      return true;
+    };
+    if (plan.G == 4) {
+      auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes, kBigThreads, 1>;
+      static hipError_t attr = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      return launch_big(kernel, attr);
+    }
+    auto kernel = stream_tiled_kernel<16, 16, 16, UNPACK, kStreamBigBlockBytes, kBigThreads, 1>;
     static hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-        160 * 1024);
-    if (attr != hipSuccess || lds > 160 * 1024) return false;
-    uk::launch(UNPACK ? 1 : 0, kernel, dim3(nblocks < 256 ? nblocks : 256), dim3(kBigThreads), lds,
-               stream, plan.args);
-    return true;
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    return launch_big(kernel, attr);
   }
   const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
 #define UK_CASE(g, vv, mv)                                                          \

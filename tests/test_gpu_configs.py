@@ -214,3 +214,40 @@ def test_c5_pack_unpack_stress_at_size(runner, name):
     assert np.array_equal(got, want), "packed buffer differs from pad + reshape + transpose"
     del want, got
     assert np.array_equal(_host(k["back"]).view(np.uint32).reshape(rows, cols), x), "round trip"
+
+
+@pytest.mark.parametrize("rows,cols,es,t0,t1,pitch_slack", [(8190, 8200, 4, 16, 16, 0),     # f32, 256 MB, ragged
+                                                            (8192, 8192, 4, 16, 16, 1),     # loose pitch, rows only 4-byte aligned
+                                                            (12272, 8192, 1, 16, 32, 0)])   # f8/s8 rows, ragged
+def test_row_granule_pack_unpack_in_64k_blocks_at_size(gpu, rows, cols, es, t0, t1, pitch_slack):
+    """Untransposed pack / unpack of large matrices (whole tile rows move as
+    16-byte granules, 64 KB blocks per workgroup): the packed buffer equals
+    pad + reshape + transpose of the source, padding included, and unpack
+    restores the matrix and leaves the pitch gap alone."""
+    lib, torch = gpu
+    ty = {1: uk.PACK_TYPE_I8I8, 4: uk.PACK_TYPE_F32F32}[es]
+    dt = {1: torch.uint8, 4: torch.int32}[es]
+    npdt = {1: np.uint8, 4: np.uint32}[es]
+    pitch = cols + pitch_slack
+    hi = 256 if es == 1 else 2 ** 31 - 1
+    x = torch.randint(0, hi, (rows, pitch), dtype=dt, device="cuda")
+    o0, o1 = -(-rows // t0), -(-cols // t1)
+    packed = torch.full((o0 * o1 * t0 * t1,), 3, dtype=dt, device="cuda")
+    back = torch.full((rows, pitch), 5, dtype=dt, device="cuda")
+    pad = 0x5A if es == 1 else 0x5A5A5A5A
+    torch.cuda.synchronize()
+    lib.pack(x.data_ptr(), 0, pitch, 1, packed.data_ptr(), 0, o1 * t0 * t1, t0 * t1, rows, cols,
+             o0, o1, t0, t1, pad, ty)
+    assert lib.last_kernel_name() == "pack_stream"
+    if es != 1:     # unpack has no 1-byte type (exported_bits.h:73-79)
+        lib.unpack(packed.data_ptr(), 0, o1 * t0 * t1, t0 * t1, back.data_ptr(), 0, pitch, 1,
+                   o0, o1, t0, t1, rows, cols, uk.UNPACK_TYPE_F32F32)
+        assert lib.last_kernel_name() == "unpack_stream"
+    lib.synchronize()
+    xh = x.cpu().numpy().view(npdt)[:, :cols]
+    want = pack_identity(xh, t0, t1, npdt(pad)).reshape(-1)
+    assert np.array_equal(packed.cpu().numpy().view(npdt), want), "packed buffer"
+    if es != 1:
+        bh = back.cpu().numpy().view(npdt)
+        assert np.array_equal(bh[:, :cols], xh), "round trip"
+        assert (bh[:, cols:] == 5).all(), "pitch gap written"
