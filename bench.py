@@ -8,8 +8,13 @@ A step is one pass of the workload's whole chain over one batch of seeded
 synthetic tensors that are already resident in HBM. The default workload is
 the f16 pack -> mmt4d -> unpack chain at M=N=K=4096 with 16x16x16 tiles. One
 JSON line is printed; `roofline` describes the dominant kernel (mmt4d),
-`cpu_baseline` the same chain on the host cores, and `extra` carries the other
-benchmark configurations (kernel-level event timings).
+`cpu_baseline` the same chain on the host cores, `extra` carries the other
+benchmark configurations (kernel-level event timings, each with its own CPU
+baseline), `measured_mfma_only_TOPS` and `measured_copy_GBps` the ceilings
+measured in this run, `host` the cores the CPU baselines saw and used, and
+`targets`, the last object of the line, one compact row per target workload:
+kernel, time, fraction of the published peak and of the measured ceiling, and
+the parity check made on the result that was just timed.
 """
 from __future__ import annotations
 
