@@ -81,9 +81,16 @@ void mmt4d_mfma_narrow_kernel(Args a) {
   block_of_workgroup(blockIdx.x, a, &wg_m, &wg_n);
   const int pm0 = wg_m * a.bpm;
   const int pn0 = wg_n * a.bpn;
-  const int lrb = a.lrb;
+  constexpr int lrb = RBC == 2 ? 1 : 2;  // the launcher checked a.lrb against it
   const uint32_t kts_per_step = KS >> lrb;
   const uint32_t q = lane >> 4, r = lane & 15;
+
+  // Slot swizzle of the LDS image: row r of chunk (K-slice) g sits in slot
+  // r ^ g. A store instruction writes, per 16 lanes, the rows 4 mg + j of the
+  // four chunks (mg, g = 0 .. 3, one j): r ^ g sends them to 16 different
+  // slots, i.e. over all banks; a fragment read (one chunk, 16 rows) is a
+  // permutation of the slots under any mask.
+  auto piece_mask = [](uint32_t g) { return g & 3u; };
 
   // ---- LHS loader units ------------------------------------------------------------
   // Unit u (lane `lane` of loader block `blk`) = (panel, half h, chunk g, row
@@ -111,24 +118,27 @@ void mmt4d_mfma_narrow_kernel(Args a) {
     const uint32_t rr = row & 15;
     // Row rr + j (j < 4, rr % 4 == 0) sits in slot (rr + j) ^ mask: the store
     // applies the j itself.
-    loff[i] = (((row >> 4) * 64 + g * 16) * 16) + ((rr & 8) | ((rr & 7) ^ swizzle_mask(g, rr >> 3))) * 16 +
-              h * 8;
+    loff[i] = (((row >> 4) * 64 + g * 16) * 16) + ((rr & 8) | ((rr & 7) ^ piece_mask(g))) * 16 + h * 8;
     if (!(pl < a.bpm && pm0 + pl < a.M1) || blk >= BLOCKS) voff[i] = 0;
   }
-  const uint32_t rd_a = (uint32_t)(wm * TM) * 1024 + (q * 16 + (r ^ swizzle_mask(q, r >> 3))) * 16;
+  const uint32_t rd_a = (uint32_t)(wm * TM) * 1024 + (q * 16 + (r ^ piece_mask(q))) * 16;
 
   // ---- RHS: lane (q, r) reads rows 4 (r % 4) .. + 3 of panel r / 4 ---------------
-  const uint32_t kt_bytes_b = 16u << lrb;
-  const uint32_t sstep_b = kts_per_step * kt_bytes_b;
-  const uint32_t skt_b = NCH * kt_bytes_b;
+  // N0 = 16 and the row width is a template parameter: the distances are
+  // compile-time, so a load is scalar base (advanced per step) + one vector
+  // offset + an immediate.
+  constexpr uint32_t kt_bytes_b = 16u * RBC;
+  constexpr uint32_t sstep_b = (KS / RBC) * kt_bytes_b;
+  constexpr uint32_t skt_b = NCH * kt_bytes_b;
   const int my_panel = wn * TN + (int)(r >> 2);          // within the workgroup's panels
   const bool panel_ok = my_panel < a.bpn && pn0 + my_panel < a.N1;
   const char* sbase_b = a.rhs + (int64_t)pn0 * a.rhs_stride;
-  const uint32_t voff_b =
-      panel_ok ? (uint32_t)my_panel * (uint32_t)a.rhs_stride + q * kt_bytes_b + (r & 3) * (4u << lrb) : 0u;
+  uint32_t voff_b =
+      panel_ok ? (uint32_t)my_panel * (uint32_t)a.rhs_stride + q * kt_bytes_b + (r & 3) * (4u * RBC) : 0u;
   auto load_b = [&](int t, int step) -> Raw {
+    const char* sb = sbase_b + (uint64_t)((uint32_t)step * sstep_b);
     return *reinterpret_cast<const typename std::conditional<RBC == 4, v4i_g, v2i_ng>::type*>(
-        sbase_b + (voff_b + (uint32_t)step * sstep_b + (uint32_t)t * skt_b));
+        sb + voff_b + (uint32_t)t * skt_b);
   };
   // Row j (of the piece's four) as a 16-byte operand, from the R pieces of
   // K-tiles x, x + 4, ... that a lane has loaded: its 16 bytes of K. RB = 4:
@@ -184,10 +194,13 @@ void mmt4d_mfma_narrow_kernel(Args a) {
   // ---- pipeline (PIPE 3 of mmt4d_mfma_kernel.h) ------------------------------------
   using RawG = typename std::conditional<RBC == 4, v4i_g, v2i_ng>::type;
   auto load_a = [&](int i, int t, int step) -> Raw {
-    return *reinterpret_cast<const RawG*>(sbase_a + (voff[i] + (uint32_t)step * sstep_a + (uint32_t)t * skt_a));
+    const char* sa = sbase_a + (uint64_t)((uint32_t)step * sstep_a + (uint32_t)t * skt_a);
+    return *reinterpret_cast<const RawG*>(sa + voff[i]);
   };
   auto store_row = [&](uint32_t stage_off, int i, int j, const Raw (&in)[RL]) {
-    if (wave + i * NW >= BLOCKS) return;  // wave-uniform
+    if constexpr (BLOCKS % NW != 0) {
+      if (wave + i * NW >= BLOCKS) return;  // wave-uniform
+    }
     char* dst = lds + stage_off + (loff[i] ^ (uint32_t)(j * 16));
     if constexpr (LH == 1) {
       *reinterpret_cast<v4i*>(dst) = row_operand(in, j);
@@ -254,6 +267,12 @@ void mmt4d_mfma_narrow_kernel(Args a) {
                        st_write = ((P + 2) % 3) * STAGE;
     const int ld_step = min(s + 4, last);
     const int b_step = min(s + 2, last);
+    // The vector offsets are made opaque once per iteration, so that they stay
+    // 32-bit registers beside scalar bases instead of being folded into
+    // hoisted 64-bit vector addresses that need a vector add per load.
+    asm volatile("" : "+v"(voff_b));
+#pragma unroll
+    for (int i = 0; i < NU; ++i) asm volatile("" : "+v"(voff[i]));
     v4i fb[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb[j] = row_operand(raw[P], j);
