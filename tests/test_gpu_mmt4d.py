@@ -99,8 +99,26 @@ def _tile_id(n):
     return name + "_one_byte_rows_have_no_mfma_kernel" if (tf, K0) == (uk.MMT4D_TYPE_S8S8S32, 1) else name
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15])
-@pytest.mark.parametrize("n", range(len(MFMA_TILES)), ids=_tile_id)
+def _variant_applies(n, variant):
+    """Forced shapes that a tile cannot take hand the call on to the choice by
+    size, i.e. repeat variant 0: the deep 64x64 pipeline (11) exists for tile
+    rows under 16 bytes, the narrow-row kernels (12 .. 15) for rows of 2 or 4
+    bytes with N0 = 16."""
+    tf, M0, N0, K0 = MFMA_TILES[n]
+    row_bytes = K0 * uk.MMT4D_TYPE_BITS[tf][0] // 8
+    if variant == 11:
+        return row_bytes < 16
+    if variant in (12, 13, 14, 15):
+        return row_bytes in (2, 4) and N0 == 16
+    return True
+
+
+_TILE_VARIANTS = [pytest.param(n, v, id=f"{_tile_id(n)}-{v}")
+                  for n in range(len(MFMA_TILES))
+                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15) if _variant_applies(n, v)]
+
+
+@pytest.mark.parametrize("n,variant", _TILE_VARIANTS)
 def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     lib, torch = gpu
     tf, M0, N0, K0 = MFMA_TILES[n]
@@ -110,9 +128,8 @@ def test_mmt4d_mfma_shapes_exact_inputs(gpu, oracle, n, variant):
     assert lib.mmt4d_info(M0, N0, K0, tf)
     lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
     bits = uk.MMT4D_TYPE_BITS[tf][0]
-    # Loose strides and offsets in steps of 16 elements: the MFMA kernels need
-    # 16-byte aligned panels (anything else goes to the generic kernel, which
-    # the reference-grid test above exercises with 1-element slack).
+    # Loose strides and offsets in steps of 16 elements (one-element slack on
+    # the matrix-core kernels has a test of its own below).
     for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=14000 + n, slack=16,
                                          shapes=_mfma_shapes(M0, N0, K0, bits))):
         rng = np.random.default_rng(ci)
