@@ -455,6 +455,13 @@ def main() -> int:
                 entry["copy2d_ceiling"] = {
                     "GBps": round(gbps, 1), "frac": round(gbps / rn.PEAK_HBM_GBPS, 4),
                     "what": f"plain copy of {rows} rows x {row_bytes} B, pitch {sp} -> {dp} B"}
+                if "unpack" in w.ops[-1].name:
+                    # unpack moves the matrix the other way: its ceiling is
+                    # the copy into the 2-D side's pitch
+                    back = R.copy2d_ceiling_gbps(rows, row_bytes, dp, sp)
+                    entry["copy2d_ceiling_unpack"] = {
+                        "GBps": round(back, 1), "frac": round(back / rn.PEAK_HBM_GBPS, 4),
+                        "what": f"plain copy of {rows} rows x {row_bytes} B, pitch {dp} -> {sp} B"}
                 keep = w.keep
                 if "back" in keep:
                     entry["parity"] = {"round_trip_bit_exact": bool(
@@ -497,6 +504,7 @@ def main() -> int:
             targets[name] = {"pack_frac": round(e["kernels"]["pack"]["frac"], 3),
                              "unpack_frac": round(e["kernels"]["unpack"]["frac"], 3),
                              "copy2d_frac": round(e["copy2d_ceiling"]["frac"], 3),
+                             "copy2d_unpack_frac": round(e["copy2d_ceiling_unpack"]["frac"], 3),
                              "round_trip_bit_exact": e["parity"]["round_trip_bit_exact"]}
         result["targets"] = targets
 

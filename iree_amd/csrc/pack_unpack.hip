@@ -1000,12 +1000,24 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
   const int64_t kTarget = big ? kStreamBigBlockBytes : kStreamBlockBytes;  // bytes per block, about
   const int64_t stream_block = kTarget;
   int64_t G0 = 1, G1 = uk::ceil_div(kMinSpan, v.tile1 * es);
+  const bool mat_rows_unaligned =
+      uk::pow2_divisor(mat_stride0 * es, 16) < 16 || uk::pow2_divisor((int64_t)(uintptr_t)mat_ptr, 16) < 16;
   if (to && big && mat_is_dest) {
-    // unpack writes matrix rows: 1 KB row segments (and 256-byte runs on the
+    // unpack writes matrix rows: 2 KB row segments (and 128-byte runs on the
     // tiled side, which is only read) leave fewer partly written cache lines
-    // when the rows are not line-aligned (f32 12288x12289: 4.1 -> 4.4 TB/s).
-    G0 = uk::ceil_div(256, tile_bytes);
-    G1 = uk::ceil_div(1024, v.tile1 * es);
+    // when the rows are not line-aligned (f32 12288x12289: 4.1 -> 4.7 TB/s;
+    // no change for aligned rows).
+    G0 = uk::ceil_div(128, tile_bytes);
+    G1 = uk::ceil_div(2048, v.tile1 * es);
+    while (G0 * G1 * tile_bytes * 2 <= kTarget) G1 *= 2;  // (larger tiles: fill the block)
+  } else if (to && big && mat_rows_unaligned) {
+    // pack reads matrix rows that start at odd 4-byte offsets: the side that
+    // is written (the tiles) gets the long spans, 1 KB runs, and the rows are
+    // read in 256-byte segments (f32 12288x12289: 248 -> 233 us; aligned rows
+    // are better off with 512 bytes on both sides).
+    G0 = uk::ceil_div(1024, tile_bytes);
+    G1 = uk::ceil_div(256, v.tile1 * es);
+    while (G0 * G1 * tile_bytes * 2 <= kTarget) G0 *= 2;  // (larger tiles: fill the block)
   } else if (to) {
     G0 = uk::ceil_div(kMinSpan, tile_bytes);
     // widen along dim 1 (more, longer 2-D row segments) up to the target
