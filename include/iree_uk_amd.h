@@ -444,7 +444,7 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_timing_end(double* elapsed_us, int* kinds,
  * caller that always passes host pointers (the HAL executable-plugin thunks)
  * allocates a handful of times in its life. staging_bytes reports what the
  * calling thread holds; release_staging frees it (0 or a hipError_t value; a
- * later host-operand call allocates again). Any pitch is staged, negative and
+ * later host-operand call allocates again), and so does the thread's end. Any pitch is staged, negative and
  * zero (broadcast) included. No counterpart in the reference. */
 IREE_UK_AMD_EXPORT int64_t iree_uk_amd_staging_bytes(void);
 IREE_UK_AMD_EXPORT int iree_uk_amd_release_staging(void);

@@ -67,7 +67,16 @@ struct OwnedWorkspace {
   size_t partial_bytes;
   uint32_t n_counters;
 };
-thread_local std::vector<OwnedWorkspace> g_workspaces;
+// Freed when the thread ends; hipFree waits for the device, so no kernel in
+// flight can still use a workspace then.
+struct OwnedWorkspaces : std::vector<OwnedWorkspace> {
+  ~OwnedWorkspaces() {
+    for (OwnedWorkspace& w : *this) {
+      if (w.base) (void)hipFree(w.base);
+    }
+  }
+};
+thread_local OwnedWorkspaces g_workspaces;
 thread_local bool g_no_alloc = false;
 thread_local int g_k_slices = 0;
 thread_local int g_last_k_slices = 1;

@@ -80,7 +80,7 @@ int iree_uk_amd_hip_classify_pointer(const void* ptr, int* is_device) {
 
 namespace {
 // Staging arenas of the calling thread, one per device it has staged on.
-// Grow-only and kept until iree_uk_amd_release_staging or process end: a
+// Grow-only and kept until iree_uk_amd_release_staging or the thread's end: a
 // thread that keeps passing host operands allocates a handful of times in
 // its life instead of several times per call.
 struct StagingArena {
@@ -88,7 +88,17 @@ struct StagingArena {
   void* base;
   size_t bytes;
 };
-thread_local std::vector<StagingArena> g_staging;
+// Freed when the thread ends (a pool of short-lived threads must not leak
+// device memory); hipFree waits for the device, so nothing in flight can still
+// read the block.
+struct StagingArenas : std::vector<StagingArena> {
+  ~StagingArenas() {
+    for (StagingArena& a : *this) {
+      if (a.base) (void)hipFree(a.base);
+    }
+  }
+};
+thread_local StagingArenas g_staging;
 }  // namespace
 
 int iree_uk_amd_hip_staging_reserve(void** base, int64_t bytes) {

@@ -351,6 +351,38 @@ def test_mmt4d_host_operands_with_negative_zero_and_overlapping_pitches(gpu, ora
     assert lib.release_staging() == 0 and lib.staging_bytes() == 0
 
 
+def test_thread_local_device_memory_is_released_when_the_thread_ends(gpu):
+    """The staging arena (host operands) and the K-split workspace belong to the
+    calling thread and go back to the device when it ends: a pool of
+    short-lived threads must not leak device memory."""
+    import threading
+    lib, torch = gpu
+    torch.cuda.synchronize()
+    tf, M0, N0, K0 = uk.MMT4D_TYPE_S8S8S32, 16, 16, 16
+    M, N, K = 64, 256, 256                     # 4 MiB + 16 MiB of operands, 4 MiB of result
+    rng = np.random.default_rng(5)
+    lhs = rng.integers(-128, 128, M * K * M0 * K0, dtype=np.int8)
+    rhs = rng.integers(-128, 128, N * K * N0 * K0, dtype=np.int8)
+    held = []
+
+    def work():
+        out = np.zeros(M * N * M0 * N0, dtype=np.int32)
+        lib.mmt4d(lhs.ctypes.data, 0, K * M0 * K0, rhs.ctypes.data, 0, K * N0 * K0, out.ctypes.data, 0,
+                  N * M0 * N0, M, N, K, M0, N0, K0, tf)
+        held.append((lib.staging_bytes(), int(out[0])))
+
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        t = threading.Thread(target=work)
+        t.start()
+        t.join()
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert all(h[0] >= 24 << 20 for h in held), held          # each thread staged its own copy
+    assert len({h[1] for h in held}) == 1
+    assert free_before - free_after < (8 << 20), (free_before, free_after)
+
+
 def test_entry_points_from_concurrent_threads(gpu, oracle):
     """The entry points are re-entrant (runtime/src/iree/builtins/ukernel/
     README.md:26): four host threads, each on its own slab of one problem
