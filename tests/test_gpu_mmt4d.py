@@ -561,6 +561,56 @@ def test_mmt4d_persistent_kernels(gpu, oracle, variant, tile, workgroups):
         lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
 
 
+def test_mmt4d_last_partial_round_runs_as_its_own_launch(gpu):
+    """A problem that the 128x512 shape tiles exactly into 1.25 rounds of
+    blocks (2 x 160 = 320 on 256 compute units) is split by columns: whole
+    rounds in one launch, the last 32 block columns in another with a smaller
+    shape. Results equal the single launch of a forced shape bit for bit, the
+    column scales of the dequantizing store included."""
+    lib, torch = gpu
+    tf, M0, N0, K0 = uk.MMT4D_TYPE_S8S8S32, 16, 16, 16
+    M1, N1, K1 = 256 // M0, 160 * 512 // N0, 512 // K0
+    M, N = M1 * M0, N1 * N0
+    g = torch.Generator(device="cuda"); g.manual_seed(33)
+    lhs = torch.randint(-128, 128, (M1 * K1 * M0 * K0,), generator=g, device="cuda", dtype=torch.int8)
+    rhs = torch.randint(-128, 128, (N1 * K1 * N0 * K0,), generator=g, device="cuda", dtype=torch.int8)
+    acc0 = torch.randint(-1000, 1000, (M1 * N1 * M0 * N0,), generator=g, device="cuda", dtype=torch.int32)
+    rs = torch.rand(M, generator=g, device="cuda") + 0.5
+    cs = torch.rand(N, generator=g, device="cuda") + 0.5
+    results = {}
+    for mode in (uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_MFMA_VARIANT + 1):
+        out = acc0.clone()
+        y = torch.zeros(M, N, device="cuda", dtype=torch.float32)
+        torch.cuda.synchronize()
+        lib.set_kernel_mode(mode)
+        try:
+            lib.timing_begin()
+            lib.mmt4d(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, out.data_ptr(), 0,
+                      N1 * M0 * N0, M1, N1, K1, M0, N0, K0, tf | uk.MMT4D_ACCUMULATE)
+            launches = len(lib.timing_end())
+            assert launches == (2 if mode == uk.KERNEL_MODE_AUTO else 1), launches
+            name = lib.last_kernel_name()
+            lib.mmt4d_dequant_unpack(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0,
+                                     None, 0, 0, y.data_ptr(), 0, N, M, N, rs.data_ptr(), cs.data_ptr(),
+                                     M1, N1, K1, M0, N0, K0, tf)
+            lib.synchronize()
+        finally:
+            lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+        results[mode] = (out.cpu(), y.cpu(), name)
+    auto, forced = results[uk.KERNEL_MODE_AUTO], results[uk.KERNEL_MODE_MFMA_VARIANT + 1]
+    assert auto[2] == "mmt4d_mfma_128x512_rhs_direct" and forced[2] == "mmt4d_mfma_256x256_rhs_direct"
+    assert torch.equal(auto[0], forced[0])
+    assert torch.equal(auto[1], forced[1])
+    # and against the integer product on a few rows and columns of both parts
+    a = lhs.view(M1, K1, M0, K0).permute(0, 2, 1, 3).reshape(M, K1 * K0)[:32].cpu().to(torch.int64)
+    for c0 in (0, 128 * 512 - 64, 128 * 512, N - 64):
+        b = rhs.view(N1, K1, N0, K0).permute(0, 2, 1, 3).reshape(N, K1 * K0)[c0:c0 + 64].cpu().to(torch.int64)
+        want = (a @ b.T).to(torch.int32)
+        got = auto[0].view(M1, N1, M0, N0).permute(0, 2, 1, 3).reshape(M, N)[:32, c0:c0 + 64]
+        base = acc0.view(M1, N1, M0, N0).permute(0, 2, 1, 3).reshape(M, N)[:32, c0:c0 + 64].cpu()
+        assert torch.equal(got, want + base), c0
+
+
 # Operands at odd element offsets and strides (the reference grid's slack of
 # one element: tools/mmt4d_test.c:354-404), WITHOUT the generic-fallback flag:
 # iree_uk_mmt4d_info advertises these tile shapes, so an MFMA kernel has to
