@@ -34,7 +34,7 @@ EXTRA_WORKLOADS = [
     "c2_f16_chain_ragged", "c2_f16_fused_4096", "c2_f16_fused_ragged", "c3_s8_decode",
     "c3_s8_decode_fused", "c3_s8_decode_down", "c4_f8_prefill",
     "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "f32_mmt4d_4096_k1",
-    "f32_mmt4d_4096_k4",
+    "f32_mmt4d_4096_k4", "s16_mmt4d_4096_k2",
     "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288",
     "conv_nchwc_f32_n16_56x56_c256_k256_3x3",
 ]
@@ -152,7 +152,7 @@ def _host_bytes(t):
 def _mmt4d_type_flag(dtype: str, uk):
     return {"s8": uk.MMT4D_TYPE_S8S8S32, "f16": uk.MMT4D_TYPE_F16F16F32,
             "bf16": uk.MMT4D_TYPE_BF16BF16F32, "f32": uk.MMT4D_TYPE_F32F32F32,
-            "f8": uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32}[dtype]
+            "f8": uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, "s16": uk.MMT4D_TYPE_S16S16S32}[dtype]
 
 
 def cpu_baseline_extra(wl, target_seconds: float = 3.0):
@@ -223,7 +223,7 @@ def cpu_baseline_extra(wl, target_seconds: float = 3.0):
     if "lhs4" not in keep or "M1" not in keep and "M" not in keep:
         return None
     dtype = wl.dtype
-    if dtype not in ("s8", "f16", "bf16", "f32", "f8"):
+    if dtype not in ("s8", "f16", "bf16", "f32", "f8", "s16"):
         return None
     kind = "reference" if (have_ref and dtype != "f8") else "port"
     chk = uk_oracle.Checker("reference" if kind == "reference" else "oracle")
@@ -236,7 +236,7 @@ def cpu_baseline_extra(wl, target_seconds: float = 3.0):
     flags = _mmt4d_type_flag(dtype, uk) | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
     lhs = _host_bytes(keep["lhs4"])
     rhs = _host_bytes(keep["rhs4"])
-    out = np.zeros(M1 * N1 * M0 * N0, np.int32 if dtype == "s8" else np.float32)
+    out = np.zeros(M1 * N1 * M0 * N0, np.int32 if dtype in ("s8", "s16") else np.float32)
     ls, rs, os_ = K1 * M0 * K0, K1 * N0 * K0, N1 * M0 * N0
 
     def run(m_tiles, n_tiles):
@@ -301,12 +301,13 @@ def verify_sampled_tiles(wl, n_random: int = 64, seed: int = 0) -> dict:
         M1, N1, K1 = k["M1"], k["N1"], k["K1"]
     else:
         M1, N1, K1 = -(-k["M"] // M0), -(-k["N"] // N0), k["K"] // K0
-    es = {"s8": 1, "f8": 1, "f16": 2, "bf16": 2, "f32": 4}[dtype]
+    es = {"s8": 1, "f8": 1, "f16": 2, "bf16": 2, "f32": 4, "s16": 2}[dtype]
     view = {1: np.uint8, 2: np.uint16, 4: np.uint32}[es]
     chk = uk_oracle.get("oracle")
     lhs = _host_bytes(k["lhs4"]).reshape(M1, K1 * M0 * K0 * es)
     rhs = _host_bytes(k["rhs4"]).reshape(N1, K1 * N0 * K0 * es)
-    out_dt = np.int32 if dtype == "s8" else np.float32
+    integer = dtype in ("s8", "s16")
+    out_dt = np.int32 if integer else np.float32
     got_all = _host_bytes(k["out4"]).view(out_dt).reshape(M1, N1, M0 * N0)
     rng = np.random.default_rng(seed)
     tiles = {(0, 0), (0, N1 - 1), (M1 - 1, 0), (M1 - 1, N1 - 1)}
@@ -319,14 +320,14 @@ def verify_sampled_tiles(wl, n_random: int = 64, seed: int = 0) -> dict:
         chk.mmt4d(lhs[m].view(view), 0, K1 * M0 * K0, rhs[n].view(view), 0, K1 * N0 * K0, want, 0,
                   M0 * N0, 1, 1, K1, M0, N0, K0, flags)
         got = got_all[m, n]
-        if dtype == "s8":
+        if integer:
             exact = exact and bool(np.array_equal(got, want))
         else:
             if not (np.isfinite(got).all() and np.isfinite(want).all()):
                 return {"tiles": len(tiles), "ok": False, "error": f"non-finite value in tile ({m}, {n})"}
             max_err = max(max_err, float(np.abs(got - want).max()))
             max_ref = max(max_ref, float(np.abs(want).max()))
-    if dtype == "s8":
+    if integer:
         return {"tiles": len(tiles), "bit_exact": exact, "ok": exact}
     tol = {"f16": 1e-2, "bf16": 1e-2, "f8": 2e-2, "f32": 1e-5}[dtype]
     err = max_err / max_ref if max_ref else 0.0
@@ -447,7 +448,7 @@ def main() -> int:
                     entry["cpu_baseline"] = cpu_baseline_extra(w)
                 except Exception as e:  # the baseline is a reported aside, never fatal
                     entry["cpu_baseline"] = {"error": repr(e)}
-            if not args.no_cpu and name in TARGET_MMT4D:
+            if not args.no_cpu and (name in TARGET_MMT4D or name.startswith("s16_mmt4d_")):
                 entry["parity"] = verify_sampled_tiles(w)
             if name in TARGET_PACK:
                 rows, row_bytes, sp, dp = TARGET_PACK[name]

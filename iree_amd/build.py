@@ -18,7 +18,7 @@ LIB = os.path.join(HERE, "libiree_uk_amd.so")
 HIP_SOURCES = ["mmt4d_mfma_s8.hip", "mmt4d_mfma_f16.hip", "mmt4d_mfma_bf16.hip",
                "mmt4d_mfma_f8.hip", "mmt4d_mfma_f32.hip", "mmt4d_mfma_f16f16.hip", "mmt4d_mfma_bf16bf16.hip", "mmt4d_mfma_s8s4.hip",
                "uk_runtime.hip", "uk_probe.hip", "pack_unpack.hip",
-               "mmt4d_generic.hip", "conv_nchwc.hip", "mmt4d_mfma.hip", "mmt4d_dispatch.hip"]
+               "mmt4d_generic.hip", "mmt4d_dot2.hip", "conv_nchwc.hip", "mmt4d_mfma.hip", "mmt4d_dispatch.hip"]
 C_SOURCES = ["uk_host.c", "uk_plugin.c"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -12,6 +12,9 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(
     void* stream, int forced_variant, const char** kernel_name);
 extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
                                                     int32_t K0, uint32_t flags);
+extern "C" int iree_uk_amd_hip_launch_mmt4d_dot2(
+    const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
+    void* stream);
 
 namespace {
 // Calls on this thread that iree_uk_mmt4d_info advertises a matrix-core kernel
@@ -46,6 +49,17 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
     // one the info query advertises, count the call so that the cliff shows.
     if (st >= 0) return st;
     if (!maybe && kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO && p->K != 0) ++g_declined;
+  }
+  if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC) {
+    // The 16-bit integer LHS types: vector dot products from LDS where the
+    // tile shape allows (not a matrix-core kernel, so the info query does not
+    // advertise it and callers pass the fallback flag as for the CPU library's
+    // generic tiles).
+    const int st = iree_uk_amd_hip_launch_mmt4d_dot2(p, rowmajor, stream);
+    if (st >= 0) {
+      *kernel_name = "mmt4d_dot2";
+      return st;
+    }
   }
   *kernel_name = "mmt4d_generic";
   return iree_uk_amd_hip_launch_mmt4d_generic(p, rowmajor, stream);

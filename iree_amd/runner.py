@@ -22,7 +22,10 @@ from . import ukernel as uk
 
 # Published MI355X peaks (dense).
 PEAK_HBM_GBPS = 8000.0
-PEAK_TFLOPS = {"s8": 5000.0, "f8": 5000.0, "f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+PEAK_TFLOPS = {"s8": 5000.0, "f8": 5000.0, "f16": 2500.0, "bf16": 2500.0, "f32": 157.3,
+               # s16 has no matrix instruction: the rate of the vector dot product
+               # v_dot2_i32_i16 (256 CUs x 4 SIMDs x 16 lanes x 2 multiply-adds at 2.4 GHz).
+               "s16": 157.3}
 
 
 @dataclasses.dataclass
@@ -236,6 +239,26 @@ class Runner:
                             (" on all-zero operands (power probe)" if zeros else ""), [op], op.flops,
                             op.bytes, "s8", dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1,
                                                  N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
+        if name.startswith("s16_mmt4d_"):
+            # s16 x s16 -> s32 (no 16-bit integer matrix instruction: the vector
+            # dot-product kernel), e.g. the reference's AVX-512 VNNI tile 16x16x2
+            _, _, size, k0 = name.split("_")
+            S, K0 = int(size), int(k0[1:])
+            M0 = N0 = 16
+            M1 = N1 = S // 16
+            K1 = S // K0
+            lhs4 = torch.randint(-32768, 32768, (M1 * K1 * M0 * K0,), generator=self._gen(21),
+                                 device="cuda", dtype=torch.int16)
+            rhs4 = torch.randint(-32768, 32768, (N1 * K1 * N0 * K0,), generator=self._gen(22),
+                                 device="cuda", dtype=torch.int16)
+            out4 = self.empty(M1 * N1 * M0 * N0, torch.int32)
+            op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
+                                uk.MMT4D_TYPE_S16S16S32 | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION,
+                                "s16", 2)
+            return Workload(name, f"mmt4d s16xs16->s32 {S}^3 tiles 16x16x{K0} (vector dot products)", [op],
+                            op.flops, op.bytes, "s16",
+                            dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
+                                 M0=M0, N0=N0, K0=K0))
         if name.startswith("bf16_mmt4d_"):
             _, _, size, k0 = name.split("_")
             S, K0 = int(size), int(k0[1:])

@@ -41,7 +41,9 @@ MODES = [uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_GENERIC, uk.KERNEL_MODE_MFMA_VARIAN
     (uk.MMT4D_TYPE_S8S8S32, 16, 16, 2), (uk.MMT4D_TYPE_S8S8S32, 8, 6, 4),
     (uk.MMT4D_TYPE_F16F16F32, 16, 16, 8), (uk.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1),
-    (uk.MMT4D_TYPE_S16S16S32, 4, 6, 3), (uk.MMT4D_TYPE_S8S4S32, 4, 8, 4),
+    (uk.MMT4D_TYPE_S16S16S32, 4, 6, 3), (uk.MMT4D_TYPE_S16S16S32, 16, 16, 2),
+    (uk.MMT4D_TYPE_S16U4S32, 1, 32, 8), (uk.MMT4D_TYPE_S16S8S32, 8, 6, 4),
+    (uk.MMT4D_TYPE_S8S4S32, 4, 8, 4),
     (uk.MMT4D_TYPE_S8S4S32, 16, 16, 16)])
 def test_dequant_unpack_equals_mmt4d_unpack_scale(gpu, oracle, tf, M0, N0, K0, mode):
     """Bit for bit on the reference tests' small-integer inputs (every f32
