@@ -126,7 +126,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_dot2_kernel(Dot2Args a) {
 
   // ---- accumulators: rows ty + 16 i, columns tx + 16 j ----------------------------
   int32_t acc[4][4];
-  int64_t out_index[4][4];   // -1: element does not exist
+  int64_t out_index[4][4];   // may be negative: strides of any sign
+  uint32_t exists = 0;       // bit 4 i + j: the element is part of the result
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int64_t R = row0 + ty + 16 * i;
@@ -138,7 +139,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_dot2_kernel(Dot2Args a) {
       const int64_t n1 = C / a.N0;
       const int64_t j0 = C - n1 * a.N0;
       const bool ok = R < a.rows && C < a.cols && R < a.out_rows && C < a.out_cols;
-      out_index[i][j] = ok ? m1 * a.out_s_i + i0 * a.out_s_i0 + n1 * a.out_s_j + j0 : -1;
+      out_index[i][j] = ok ? m1 * a.out_s_i + i0 * a.out_s_i0 + n1 * a.out_s_j + j0 : 0;
+      if (ok) exists |= 1u << (4 * i + j);
       acc[i][j] = 0;
       if (ok && a.accumulate) {
         const int64_t ai = a.dequant ? m1 * a.acc_s_i + (n1 * a.M0 + i0) * a.N0 + j0 : out_index[i][j];
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_dot2_kernel(Dot2Args a) {
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if (out_index[i][j] < 0) continue;
+      if (!(exists & (1u << (4 * i + j)))) continue;
       if (a.dequant) {
         const int64_t R = row0 + ty + 16 * i, C = col0 + tx + 16 * j;
         const float rs = a.row_scale ? a.row_scale[R] : 1.0f;

@@ -74,3 +74,27 @@ def test_s16_full_range_products_wrap_like_int32(gpu):
     want = (K1 * K0 * (1 << 30)) % (1 << 32)
     want = want - (1 << 32) if want >= (1 << 31) else want
     assert (out.cpu() == want).all()
+
+
+def test_s16_negative_strides_on_device_operands(gpu, oracle):
+    """Row panels walked downwards in memory (negative stride0 on all three
+    operands): legal for mmt4d (the reference only does pointer arithmetic
+    with them, mmt4d.c:70-83) and served by the dot-product kernel."""
+    lib, torch = gpu
+    tf, M0, N0, K0 = uk.MMT4D_TYPE_S16S16S32, 8, 8, 4
+    M, N, K = 5, 9, 11
+    dl, dr, do = K * M0 * K0, K * N0 * K0, N * M0 * N0
+    ls, rs, os_ = -(dl + 2), -(dr + 4), -(do + 3)
+    rng = np.random.default_rng(9)
+    lhs = rng.integers(-32768, 32768, (M - 1) * -ls + dl, dtype=np.int16)
+    rhs = rng.integers(-32768, 32768, (N - 1) * -rs + dr, dtype=np.int16)
+    out0 = rng.integers(-1000, 1000, (M - 1) * -os_ + do, dtype=np.int32)
+    loff, roff, ooff = (M - 1) * -ls, (N - 1) * -rs, (M - 1) * -os_
+    flags = tf | uk.MMT4D_ACCUMULATE | 0x200
+    want = out0.copy()
+    oracle.mmt4d(lhs, loff, ls, rhs, roff, rs, want, ooff, os_, M, N, K, M0, N0, K0, flags)
+    d = [T.DeviceBytes(torch, a) for a in (lhs, rhs, out0)]
+    lib.mmt4d(d[0].ptr, loff, ls, d[1].ptr, roff, rs, d[2].ptr, ooff, os_, M, N, K, M0, N0, K0, flags)
+    lib.synchronize()
+    assert lib.last_kernel_name() == "mmt4d_dot2"
+    assert np.array_equal(d[2].numpy().view(np.int32), want)
