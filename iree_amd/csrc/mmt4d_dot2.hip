@@ -56,13 +56,12 @@ struct Dot2Args {
   uint32_t accumulate;
 };
 
-// The pair of K elements (k, k + 1) of row `r` of an operand whose tiles hold
-// `T0` rows of K0 elements: offset in elements from the operand's base, panel
-// stride excluded.
-__device__ __forceinline__ int64_t pair_offset(int64_t k, int32_t r0, int32_t T0, int32_t K0, int32_t lk0) {
-  const int64_t k1 = k >> lk0;
-  const int32_t k0 = (int32_t)(k & (K0 - 1));
-  return (k1 * T0 + r0) * K0 + k0;
+// The pair of K elements (k, k + 1) of row `r0` of a tile of an operand whose
+// tiles hold `T0` rows of K0 = 1 << lk0 elements: offset in elements from the
+// start of the row panel. 32-bit arithmetic: the launcher checks that a panel
+// spans fewer than 2^31 elements.
+__device__ __forceinline__ uint32_t pair_offset(uint32_t k, uint32_t r0, uint32_t T0, uint32_t K0, uint32_t lk0) {
+  return (((k >> lk0) * T0 + r0) << lk0) + (k & (K0 - 1));
 }
 
 template <Rhs RHS>
@@ -99,23 +98,25 @@ __global__ __launch_bounds__(kThreads) void mmt4d_dot2_kernel(Dot2Args a) {
     a_ptr[n] = a.lhs + m1 * a.lhs_stride_bytes;
     b_ptr[n] = a.rhs + n1 * a.rhs_stride_bytes;
   }
-  auto load_a = [&](int n, int64_t kbase) -> uint32_t {
-    const int64_t k = kbase + pair_k[n];
-    if (!a_ok[n] || k >= a.k_total) return 0u;
-    const int64_t e = pair_offset(k, a_r0[n], a.M0, a.K0, a.lk0);
+  const uint32_t k_total = (uint32_t)a.k_total;
+  auto load_a = [&](int n, uint32_t kbase) -> uint32_t {
+    const uint32_t k = kbase + (uint32_t)pair_k[n];
+    if (!a_ok[n] || k >= k_total) return 0u;
+    const uint32_t e = pair_offset(k, (uint32_t)a_r0[n], (uint32_t)a.M0, (uint32_t)a.K0, (uint32_t)a.lk0);
     typedef uint32_t u32_unaligned __attribute__((aligned(2)));
-    return *reinterpret_cast<const u32_unaligned*>(a_ptr[n] + e * 2);
+    return *reinterpret_cast<const u32_unaligned*>(a_ptr[n] + (uint64_t)e * 2);
   };
-  auto load_b = [&](int n, int64_t kbase) -> uint32_t {
-    const int64_t k = kbase + pair_k[n];
-    if (!b_ok[n] || k >= a.k_total) return 0u;
-    const int64_t e = pair_offset(k, b_r0[n], a.N0, a.K0, a.lk0);
+  auto load_b = [&](int n, uint32_t kbase) -> uint32_t {
+    const uint32_t k = kbase + (uint32_t)pair_k[n];
+    if (!b_ok[n] || k >= k_total) return 0u;
+    const uint32_t e = pair_offset(k, (uint32_t)b_r0[n], (uint32_t)a.N0, (uint32_t)a.K0, (uint32_t)a.lk0);
     if constexpr (RHS == Rhs::kS16) {
       typedef uint32_t u32_unaligned __attribute__((aligned(2)));
-      return *reinterpret_cast<const u32_unaligned*>(b_ptr[n] + e * 2);
+      return *reinterpret_cast<const u32_unaligned*>(b_ptr[n] + (uint64_t)e * 2);
     } else if constexpr (RHS == Rhs::kS8) {
-      const int8_t* p = reinterpret_cast<const int8_t*>(b_ptr[n] + e);
-      const int32_t lo = p[0], hi = p[1];
+      typedef uint16_t u16_unaligned __attribute__((aligned(1)));
+      const uint32_t w = *reinterpret_cast<const u16_unaligned*>(b_ptr[n] + e);
+      const int32_t lo = (int8_t)(w & 0xFF), hi = (int8_t)(w >> 8);
       return ((uint32_t)lo & 0xFFFFu) | ((uint32_t)hi << 16);
     } else {
       // Two 4-bit values per byte, low nibble first; e is even.
@@ -150,14 +151,14 @@ __global__ __launch_bounds__(kThreads) void mmt4d_dot2_kernel(Dot2Args a) {
   }
 
   // ---- K loop: LDS double-buffered, one barrier per step ---------------------------
-  const int64_t steps = (a.k_total + kStepK - 1) / kStepK;
+  const uint32_t steps = (k_total + kStepK - 1) / kStepK;
   uint32_t ra[4], rb[4];
 #pragma unroll
   for (int n = 0; n < 4; ++n) { ra[n] = load_a(n, 0); rb[n] = load_b(n, 0); }
 #pragma unroll
   for (int n = 0; n < 4; ++n) { lds_a[0][dst[n]] = ra[n]; lds_b[0][dst[n]] = rb[n]; }
   __syncthreads();
-  for (int64_t s = 0; s < steps; ++s) {
+  for (uint32_t s = 0; s < steps; ++s) {
     const int cur = (int)(s & 1);
     if (s + 1 < steps) {
 #pragma unroll
@@ -258,6 +259,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_dot2(const iree_uk_mmt4d_params_t* p
     a.col_scale = rowmajor->col_scale;
   }
   a.k_total = p->K * (int64_t)K0;
+  // 32-bit offsets inside a row panel (in elements) and a 32-bit K counter.
+  if (a.k_total >= (1ll << 31) - 64 || a.k_total * p->M0 >= (1ll << 31) || a.k_total * p->N0 >= (1ll << 31)) {
+    return -1;
+  }
   a.M0 = p->M0; a.N0 = p->N0; a.K0 = K0;
   while ((1 << a.lk0) < K0) ++a.lk0;
   a.accumulate = (p->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0;

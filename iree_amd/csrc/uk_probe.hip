@@ -152,7 +152,11 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(uint32_t type_flags, const vo
   const v4i* ops_ptr = (const v4i*)operands;
   const int n = (int)(operand_bytes / 16);
   hipEvent_t start, stop;
-  if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return (int)hipErrorUnknown;
+  if (hipEventCreate(&start) != hipSuccess) return (int)hipErrorUnknown;
+  if (hipEventCreate(&stop) != hipSuccess) {
+    (void)hipEventDestroy(start);
+    return (int)hipErrorUnknown;
+  }
   double ops = 0;
   int st = 0;
   auto run = [&](int it) {
@@ -207,7 +211,11 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(const void* src, int64_t src_pit
     return (int)hipErrorUnknown;
   }
   hipEvent_t start, stop;
-  if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return (int)hipErrorUnknown;
+  if (hipEventCreate(&start) != hipSuccess) return (int)hipErrorUnknown;
+  if (hipEventCreate(&stop) != hipSuccess) {
+    (void)hipEventDestroy(start);
+    return (int)hipErrorUnknown;
+  }
   // Four ways of writing the same copy; the fastest one is the ceiling.
   auto run = [&](int variant) {
     const char* s8 = (const char*)src;
