@@ -413,6 +413,9 @@ def main() -> int:
     peaks = {dt: round(R.measured_mfma_peak(dt), 1) for dt in ("s8", "f8", "f16", "bf16", "f32")}
     peaks["s8_zero_operands"] = round(R.measured_mfma_peak("s8", zeros=True), 1)
     result["measured_mfma_only_TOPS"] = peaks
+    if roof["bound"] == "mfma" and wl.dtype in peaks and peaks[wl.dtype] > 0:
+        # the same kernel against the ceiling measured in this run
+        roof["of_measured_mfma_only"] = round(roof["achieved"] / peaks[wl.dtype], 4)
 
     if not args.no_cpu and args.workload.startswith("c2_f16_chain"):
         base, cpu_out4, slab = cpu_baseline_c2(wl.keep)
