@@ -235,7 +235,7 @@ int launch_persistent(const Problem& p, int kt_count, bool force, hipStream_t st
 template <Elem E, int RBC, int TM, int WGM, int WGN>
 int launch_narrow(const Problem& p, int kt_count, hipStream_t stream) {
   constexpr int BM = WGM * TM * 16, BN = WGN * 64, KS = 64;
-  if (p.rb != RBC || p.N0 != 16 || p.M0 % 4 || p.M0 > BM || BM % p.M0) return -1;
+  if (p.rb != RBC || p.N0 != 16 || p.M0 % (16 / RBC) || p.M0 > BM || BM % p.M0) return -1;
   if (p.dequant) return -1;
   if (p.out_rows <= 0 || p.out_cols <= 0) return 0;
   if (p.out_cols < (int64_t)p.N1 * p.N0) return -1;   // a row-major matrix narrower than the tiles

@@ -21,17 +21,17 @@
 // 12 + j of panel q. Taking the same register of the four blocks gives four
 // CONSECUTIVE columns again, so accumulators still move 16 bytes per lane.
 // The LHS goes through LDS in the general kernel's image (chunk q of a step
-// holds K-tiles q, q + 4, ...: the K assignment of the RHS lanes), but its
-// loader lanes read the same four-row pieces as the RHS lanes do (8-byte
-// pieces for RB = 2) and regroup them the same way, four LDS rows per unit:
-// with whole 16-byte pieces a 2-byte-row unit would be 8 loads of 16 bytes,
-// and three register sets of those do not fit beside the accumulators. For
-// RB = 2 a loader unit is in fact half of that again (4 loads of 8 bytes: 8 of
-// an operand's 16 K bytes, stored as 8 bytes per row), so that all eight waves
-// load, each a little.
+// holds K-tiles q, q + 4, ...: the K assignment of the RHS lanes). Its loader
+// lanes read whole 16-byte pieces (4 rows for RB = 4, 8 rows for RB = 2: the
+// CU's address unit is the busiest part of this kernel, and a 16-byte load
+// costs it what an 8-byte one does) and regroup them as the RHS lanes do. For
+// RB = 2 a unit is a quarter of an operand's K (2 loads, 4 bytes per row, one
+// v_perm_b32 and one 4-byte LDS store per row): three register sets of whole
+// units would not fit beside the accumulators, and so all eight waves load,
+// each a little.
 //
-// Restrictions (launcher): RB in {2, 4}, N0 == 16, M0 a multiple of 4 that
-// divides the workgroup's rows,
+// Restrictions (launcher): RB in {2, 4}, N0 == 16, M0 a multiple of the rows
+// of an LHS piece (16 / RB) that divides the workgroup's rows,
 // K in whole 64-byte steps, 4-byte accumulators, no dequantizing store, output
 // columns complete (tiled output, or a row-major matrix as wide as the tiles).
 #ifndef IREE_UK_AMD_MMT4D_MFMA_NARROW_H_
@@ -58,9 +58,13 @@ void mmt4d_mfma_narrow_kernel(Args a) {
   constexpr int NCH = 4, KS = 64;           // 16-byte chunks / bytes of K per row per step
   constexpr int BM = WGM * TM * 16;
   constexpr int R = 16 / RBC;               // loads per lane operand set: K-tiles per 16 bytes of K
-  constexpr int RU = 4;                     // rows per piece (a piece: 4 rows x RB bytes, 16 or 8 bytes)
-  constexpr int LH = RBC == 2 ? 2 : 1;      // LHS loader units per 16-byte operand (halves of K)
-  constexpr int RL = R / LH;                // loads per LHS unit (4)
+  // The LHS loader moves 16-byte pieces: RU rows x RB bytes of one K-tile (the
+  // address unit of the CU is what this kernel is short of, and a 16-byte load
+  // costs it no more than an 8-byte one). RB = 2: 8 rows per piece, and a unit
+  // covers a quarter of an operand's K (two K-tiles, 4 bytes per row).
+  constexpr int RU = 16 / RBC;              // rows per LHS piece (8 or 4)
+  constexpr int LH = RBC == 2 ? 4 : 1;      // LHS loader units per 16-byte operand (parts of its K)
+  constexpr int RL = R / LH;                // loads per LHS unit (2 or 4)
   constexpr int UNITS = BM * NCH / RU * LH; // LHS loader units (RL loads, RU LDS stores each)
   constexpr int BLOCKS = (UNITS + 63) / 64; // in blocks of one unit per lane
   constexpr int NU = (BLOCKS + NW - 1) / NW;
@@ -68,7 +72,8 @@ void mmt4d_mfma_narrow_kernel(Args a) {
   constexpr int FR = 3;
   constexpr int NLD = NU * RL;              // LHS loads per thread per step
   constexpr int NST = NU * RU;              // LHS LDS stores per thread per step
-  using Raw = typename std::conditional<RBC == 4, v4i, v2i_n>::type;
+  using Raw = typename std::conditional<RBC == 4, v4i, v2i_n>::type;  // an RHS piece: 4 rows
+  using RawL = v4i;                                                     // an LHS piece: RU rows
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -85,17 +90,21 @@ void mmt4d_mfma_narrow_kernel(Args a) {
   const uint32_t kts_per_step = KS >> lrb;
   const uint32_t q = lane >> 4, r = lane & 15;
 
-  // Slot swizzle of the LDS image: row r of chunk (K-slice) g sits in slot
-  // r ^ g. A store instruction writes, per 16 lanes, the rows 4 mg + j of the
-  // four chunks (mg, g = 0 .. 3, one j): r ^ g sends them to 16 different
-  // slots, i.e. over all banks; a fragment read (one chunk, 16 rows) is a
+  // Slot swizzle of the LDS image: row r of chunk (K-slice) g of 16-row block b
+  // sits in slot r ^ piece_mask(g, b). A store instruction writes, for one j,
+  // row RU mg + j of every (row group mg, chunk g) pair (and, for 2-byte rows,
+  // of two neighbouring blocks and the four parts of K at their own offsets
+  // inside the slot): the mask sends the lanes of such a store to different
+  // bank groups. A fragment read (one chunk of one block, 16 rows) is a
   // permutation of the slots under any mask.
-  auto piece_mask = [](uint32_t g) { return g & 3u; };
+  auto piece_mask = [](uint32_t g, uint32_t blk) {
+    return RBC == 2 ? ((g & 3u) | ((blk & 1u) << 2)) : (g & 3u);
+  };
 
   // ---- LHS loader units ------------------------------------------------------------
-  // Unit u (lane `lane` of loader block `blk`) = (panel, half h, chunk g, row
-  // group mg): rows 4 mg .. + 3 of the panel, K-tiles g + 4 t of the step for
-  // t = RL h .. RL h + RL - 1 (all R of them when there is one half).
+  // Unit u (lane `lane` of loader block `blk`) = (panel, part h of K, chunk g,
+  // row group mg): rows RU mg .. + RU - 1 of the panel, K-tiles g + 4 t of the
+  // step for t = RL h .. RL h + RL - 1 (all R of them when there is one part).
   const char* sbase_a = a.lhs + (int64_t)pm0 * a.lhs_stride;
   const uint32_t kt_bytes_a = (uint32_t)a.M0 << lrb;
   const uint32_t sstep_a = kts_per_step * kt_bytes_a;
@@ -113,15 +122,18 @@ void mmt4d_mfma_narrow_kernel(Args a) {
     const uint32_t g = t1 - t2 * NCH;
     const int pl = (int)(t2 / LH);
     const uint32_t h = t2 - (uint32_t)pl * LH;
-    voff[i] = (uint32_t)pl * (uint32_t)a.lhs_stride + (g + h * RL * NCH) * kt_bytes_a + mg * (4u << lrb);
+    voff[i] = (uint32_t)pl * (uint32_t)a.lhs_stride + (g + h * RL * NCH) * kt_bytes_a + mg * (uint32_t)(RU * RBC);
     const uint32_t row = (uint32_t)pl * a.M0 + mg * RU;
     const uint32_t rr = row & 15;
-    // Row rr + j (j < 4, rr % 4 == 0) sits in slot (rr + j) ^ mask: the store
+    // Row rr + j (j < RU, rr % RU == 0) sits in slot (rr + j) ^ mask: the store
     // applies the j itself.
-    loff[i] = (((row >> 4) * 64 + g * 16) * 16) + ((rr & 8) | ((rr & 7) ^ piece_mask(g))) * 16 + h * 8;
+    loff[i] = (((row >> 4) * 64 + g * 16) * 16) + ((rr & 8) | ((rr & 7) ^ piece_mask(g, row >> 4))) * 16 +
+              h * (16 / LH);
     if (!(pl < a.bpm && pm0 + pl < a.M1) || blk >= BLOCKS) voff[i] = 0;
   }
-  const uint32_t rd_a = (uint32_t)(wm * TM) * 1024 + (q * 16 + (r ^ piece_mask(q))) * 16;
+  // (wm * TM is even: the parity of a wave's block is the parity of tm.)
+  const uint32_t rd_a0 = (uint32_t)(wm * TM) * 1024 + (q * 16 + (r ^ piece_mask(q, 0))) * 16;
+  const uint32_t rd_a1 = (uint32_t)(wm * TM) * 1024 + (q * 16 + (r ^ piece_mask(q, 1))) * 16;
 
   // ---- RHS: lane (q, r) reads rows 4 (r % 4) .. + 3 of panel r / 4 ---------------
   // N0 = 16 and the row width is a template parameter: the distances are
@@ -192,12 +204,11 @@ void mmt4d_mfma_narrow_kernel(Args a) {
   }
 
   // ---- pipeline (PIPE 3 of mmt4d_mfma_kernel.h) ------------------------------------
-  using RawG = typename std::conditional<RBC == 4, v4i_g, v2i_ng>::type;
-  auto load_a = [&](int i, int t, int step) -> Raw {
+  auto load_a = [&](int i, int t, int step) -> RawL {
     const char* sa = sbase_a + (uint64_t)((uint32_t)step * sstep_a + (uint32_t)t * skt_a);
-    return *reinterpret_cast<const RawG*>(sa + voff[i]);
+    return *reinterpret_cast<const v4i_g*>(sa + voff[i]);
   };
-  auto store_row = [&](uint32_t stage_off, int i, int j, const Raw (&in)[RL]) {
+  auto store_row = [&](uint32_t stage_off, int i, int j, const RawL (&in)[RL]) {
     if constexpr (BLOCKS % NW != 0) {
       if (wave + i * NW >= BLOCKS) return;  // wave-uniform
     }
@@ -205,20 +216,19 @@ void mmt4d_mfma_narrow_kernel(Args a) {
     if constexpr (LH == 1) {
       *reinterpret_cast<v4i*>(dst) = row_operand(in, j);
     } else {
-      // Half an operand: K-tiles x, x + 4, x + 8, x + 12 of row j, 2 bytes each.
+      // A quarter of an operand: K-tiles x and x + 4 of row j, 2 bytes each.
+      // Dword d of a piece holds rows 2d (low half) and 2d + 1 (high half).
+      static_assert(RL == 2, "two K-tiles per unit");
       const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-      v2i_n o;
-#pragma unroll
-      for (int w = 0; w < 2; ++w)
-        o[w] = (int)__builtin_amdgcn_perm((uint32_t)in[2 * w + 1][j >> 1], (uint32_t)in[2 * w][j >> 1], sel);
-      *reinterpret_cast<v2i_n*>(dst) = o;
+      *reinterpret_cast<uint32_t*>(dst) =
+          __builtin_amdgcn_perm((uint32_t)in[1][j >> 1], (uint32_t)in[0][j >> 1], sel);
     }
   };
   auto read_a = [&](uint32_t stage_off, int tm) {
-    return *reinterpret_cast<const v4i*>(lds + stage_off + rd_a + tm * 1024);
+    return *reinterpret_cast<const v4i*>(lds + stage_off + ((tm & 1) ? rd_a1 : rd_a0) + tm * 1024);
   };
   const int last = a.steps - 1;
-  Raw regs[3][NU][RL];
+  RawL regs[3][NU][RL];
   Raw raw[3][R];
   v4i fa[FR];
   // Steps 0 and 1 go to LDS stages 0 and 1 right away.
