@@ -38,8 +38,18 @@
 //   4  as 0 with the global loads three steps ahead through three register
 //      sets (any K): for M-thin problems, which are bound by memory latency
 //      and want as many bytes in flight per workgroup as registers allow.
-// Pipelines 1-3 need K in whole steps; the launcher gives a K remainder to a
-// second, accumulating launch of a PIPE 0 variant.
+//   5  both operands brought into LDS by LDS-direct global loads
+//      (global_load_lds, 16 bytes per lane: one instruction moves one 1 KiB
+//      fragment and touches no register), kStages5 stages deep; the eight
+//      waves form two groups of four (one wave of each group per SIMD) that
+//      alternate, half a step apart, between a memory phase (fragment reads,
+//      issue of the loads kStages5 - 1 steps ahead) and a compute phase (all MFMAs of
+//      the step back to back), with a workgroup barrier between phases: while
+//      one wave of a SIMD feeds the matrix pipe, the other one's memory
+//      instructions issue beside it instead of in between its MFMAs (row
+//      bytes >= 16, eight waves).
+// Pipelines 1-3 and 5 need K in whole steps; the launcher gives a K remainder
+// to a second, accumulating launch of a PIPE 0 variant.
 #ifndef IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
 #define IREE_UK_AMD_MMT4D_MFMA_KERNEL_H_
 
@@ -174,6 +184,21 @@ template <> struct ElemTraits<Elem::kF16F16> : ElemTraits<Elem::kF16> {
 template <> struct ElemTraits<Elem::kBF16BF16> : ElemTraits<Elem::kBF16> {
   using Out = Out16<8>;
 };
+
+// LDS-direct loads (PIPE 5): address-space-qualified pointers for the builtin,
+// and the wait for "at most N vector memory operations still in flight" (the
+// compiler does not track what these loads write, the kernel waits itself).
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+template <int N>
+__device__ __forceinline__ void wait_vmem_in_flight() {
+  static_assert(N >= 0 && N < 64, "the counter has six bits");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));  // expcnt, lgkmcnt: no wait
+}
+// Waits for the wave's LDS reads (and scalar loads), not for vector memory.
+__device__ __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+// LDS stages of PIPE 5.
+constexpr int kStages5 = 4;
 
 struct Args {
   const char* lhs;
@@ -338,6 +363,7 @@ void mmt4d_mfma_kernel(Args a) {
   uint32_t skt[NU];      // bytes between consecutive loads of a unit
   int32_t kt0[NU];       // K-tile index of the first load at step 0
   uint32_t loff[NU];     // LDS offset (within a stage) of the unit's first store
+  uint32_t ldma[NU];     // PIPE 5: LDS offset of the unit's 1 KiB block (uniform: lane 0's slot)
   // Regrouping loaders only: false for a unit whose rows lie beyond the
   // operand's LDS image. That happens when the tile height does not divide
   // the block (e.g. M0 = 24 in a 64-row block: the units of a third, partial
@@ -373,6 +399,7 @@ void mmt4d_mfma_kernel(Args a) {
       skt[i] = 0;
       lds_ok[i] = true;
       loff[i] = image + (uint32_t)xblk * 1024 + lane * 16;
+      ldma[i] = image + (uint32_t)xblk * 1024;
     } else {
       // Units in order [panel][chunk g][row group]; the unit's R loads read
       // K-tiles g, g + NCH, g + 2*NCH, ... so that one load instruction covers
@@ -393,6 +420,7 @@ void mmt4d_mfma_kernel(Args a) {
       // only touches the low bits and the store applies j ^ ... itself.
       loff[i] = image + (((row >> 4) * NCHB + (g >> 2)) * 64 + (g & 3) * 16) * 16 +
                 ((rr & 8) | ((rr & 7) ^ swizzle_mask(g, rr >> 3))) * 16;
+      ldma[i] = 0;
     }
     // Units outside the problem read from the start of the first panel.
     if (!(pl < bpx && px0 + pl < X1)) voff[i] = 0;
@@ -924,6 +952,72 @@ void mmt4d_mfma_kernel(Args a) {
     if (s < a.steps) iteration(s, std::integral_constant<int, 0>{});
     if (s + 1 < a.steps) iteration(s + 1, std::integral_constant<int, 1>{});
   }
+  else if constexpr (PIPE == 5) {
+    // Both operands through LDS by LDS-direct loads, two wave groups half a
+    // step apart. Phase k of the workgroup (a barrier ends each phase):
+    //   group 0: memory phase of step k/2 when k is even, compute phase when odd;
+    //   group 1: the same one phase later (it passes one extra barrier first,
+    //            group 0 one extra at the end).
+    // Memory phase of step s: read the step's fragments from stage s % NS,
+    // issue the loads of step s + NS - 1 into stage (s - 1) % NS, wait until the
+    // wave's own loads of step s + 1 have landed and its fragment reads have
+    // returned. The barrier that follows makes that true of every wave before
+    // anyone reads step s + 1 (its memory phase is at least one barrier away),
+    // and every wave has finished reading stage (s - 1) % NS before the first
+    // load into it is issued (their memory phases of step s - 1 ended at an
+    // earlier barrier). Past the last step the loads repeat the last step into
+    // a stage nobody reads any more, which keeps the in-flight count the waits
+    // assume.
+    static_assert(RBC >= 16 && HALVES == 1 && NKK == 1, "one 1 KiB block per loader unit and fragment");
+    static_assert(NW == 8 && EVEN, "two groups of four waves");
+    constexpr int NS = kStages5;
+    const int group = wave >> 2;
+    auto issue_dma = [&](uint32_t stage_off, int step) {
+#pragma unroll
+      for (int i = 0; i < NU; ++i) {
+        uint32_t o = voff[i] + (uint32_t)step * sstep[i];
+        // (kept as scalar base + 32-bit lane offset: see mmt4d_mfma_persistent.h)
+        asm volatile("" : "+v"(o));
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(sbase[i] + o),
+                                         (lds_ptr_t)(lds + stage_off + ldma[i]), 16, 0, 0);
+      }
+    };
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) issue_dma(s * STAGE, min(s, last));
+    wait_vmem_in_flight<NU*(NS - 2)>();
+    __builtin_amdgcn_s_barrier();
+    if (group == 1) __builtin_amdgcn_s_barrier();
+    v4i fa[TM][HALVES], fb[TN][HALVES];
+    auto step_body = [&](int s, auto stage_c) {
+      constexpr int ST = decltype(stage_c)::value;
+      read_frags(fa, fb, ST * STAGE, 0);
+      issue_dma(((ST + NS - 1) % NS) * STAGE, min(s + NS - 1, last));
+      wait_vmem_in_flight<NU*(NS - 2)>();
+      wait_lds_reads();
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      mfmas(fa, fb);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    static_assert(NS == 4, "the loop below is unrolled by the stage count");
+    int s = 0;
+    for (; s + 4 <= a.steps; s += 4) {
+      step_body(s, std::integral_constant<int, 0>{});
+      step_body(s + 1, std::integral_constant<int, 1>{});
+      step_body(s + 2, std::integral_constant<int, 2>{});
+      step_body(s + 3, std::integral_constant<int, 3>{});
+    }
+    if (s < a.steps) step_body(s, std::integral_constant<int, 0>{});
+    if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
+    if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
+    if (group == 0) __builtin_amdgcn_s_barrier();
+    // No LDS-direct load may still be on its way when the workgroup ends (its
+    // LDS goes to the next workgroup on the CU).
+    wait_vmem_in_flight<0>();
+  }
   // ---- epilogue -----------------------------------------------------------
   if constexpr (OB == 4) {
     if (a.dequant) {
@@ -975,7 +1069,8 @@ struct Shape {
   static constexpr int BM = WGM * TM * 16;
   static constexpr int BN = WGN * TN * 16;
   static constexpr size_t kLdsBytes =
-      (PIPE == 0 || PIPE == 4 ? 2 : 3) * (size_t)(PIPE == 2 || PIPE == 3 ? BM : BM + BN) * KS;
+      (PIPE == 5 ? kStages5 : PIPE == 0 || PIPE == 4 ? 2 : 3) *
+      (size_t)(PIPE == 2 || PIPE == 3 ? BM : BM + BN) * KS;
 };
 
 }  // namespace uk_mfma

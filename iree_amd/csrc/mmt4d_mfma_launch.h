@@ -409,7 +409,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 // 9 / 10 the persistent kernel in the 128x512 / 256x256 shape, 11 the 64x64
 // shape with 256-byte steps three steps ahead (tile rows under 16 bytes),
 // 12 .. 15 the narrow-row kernel (tile rows of 2 or 4 bytes, N0 = 16) in the
-// 256x256 / 128x512 / 128x128 / 64x64 shape;
+// 256x256 / 128x512 / 128x128 / 64x64 shape, 16 / 17 the LDS-direct ping-pong
+// pipeline in the 256x256 / 128x512 shape;
 // 0 = choose) overrides the
 // size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
@@ -437,6 +438,8 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 1;  // the narrow-row kernel in the 256x256 (12) or 128x512 (13) shape
   } else if (forced == 14) {
     choice = 2;  // the narrow-row kernel in the 128x128 shape
+  } else if (forced == 16 || forced == 17) {
+    choice = 1;  // the LDS-direct ping-pong pipeline in the 256x256 (16) or 128x512 (17) shape
   } else if (forced >= 8 && forced <= 10) {
     // The big variant in its 128x512 shape (8), the persistent kernel in that
     // shape (9) or in the square one (10); the plain square shape where the
@@ -597,6 +600,28 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         if (st < 0 && forced == 10) {
           st = launch_persistent<E, 8, 4, 2, 4>(p, kt_main, true, stream);
           if (st == 0) *name = "mmt4d_mfma_256x256_persistent";
+        }
+        if (st == 0) {
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
+      if constexpr (RBC >= 16 && H == 1) {
+        // Both operands through LDS-direct loads, two wave groups alternating
+        // between memory and compute phases (PIPE 5 of mmt4d_mfma_kernel.h): the
+        // default for the big problems of the 8- and 16-bit types (s8 8192^3
+        // 413 -> 388 us, bf16 8192^3 779 -> 718 us, f16 4096^3 102 -> 98 us
+        // against the register-direct-RHS pipeline in its best shape). f32
+        // keeps that pipeline (matrix-pipe bound there: 925 against 959 us).
+        constexpr bool kDefault = E != Elem::kF32;
+        if (forced == 17) {
+          st = launch_variant<E, RBC, 8, 4, 1, 8, 1, 5>(p, 0, kt_main, p.accumulate, stream);
+          if (st == 0) *name = "mmt4d_mfma_128x512_lds_direct";
+        }
+        if (st < 0 && (forced == 16 || forced == 17 || (forced == 0 && kDefault))) {
+          st = launch_variant<E, RBC, 8, 4, 2, 4, 1, 5>(p, 0, kt_main, p.accumulate, stream);
+          if (st == 0) *name = "mmt4d_mfma_256x256_lds_direct";
         }
         if (st == 0) {
           if (kt_main == p.K1) return 0;

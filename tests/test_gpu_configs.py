@@ -175,10 +175,12 @@ def test_c5_float_mmt4d_8192_sampled_tiles(runner, oracle, name, dtype):
 
 # The s8 8192^3 target: the reference's own x86 tile (16x16x2) and an
 # MFMA-friendly K0, bit-exact on the sampled tiles; the K0 = 16 case also under
-# every big workgroup shape (1 = 256x256, 8 = 128x512, 9 / 10 = persistent).
+# every big workgroup shape (1 = 256x256, 8 = 128x512, 9 / 10 = persistent,
+# 16 / 17 = the LDS-direct pipeline in the 256x256 / 128x512 shape).
 @pytest.mark.parametrize("name,variant", [("s8_mmt4d_8192_k2", 0), ("s8_mmt4d_8192_k16", 0),
                                           ("s8_mmt4d_8192_k16", 1), ("s8_mmt4d_8192_k16", 8),
                                           ("s8_mmt4d_8192_k16", 9), ("s8_mmt4d_8192_k16", 10),
+                                          ("s8_mmt4d_8192_k16", 16), ("s8_mmt4d_8192_k16", 17),
                                           ("s8_mmt4d_8192_k64", 0)])
 def test_target_s8_mmt4d_8192_bit_exact_on_sampled_tiles(runner, oracle, name, variant):
     wl = runner.workload(name)

@@ -31,7 +31,7 @@ def _want(oracle, c, lhs, rhs, acc_tiled, rows, cols, rs, cs, ok):
 
 MODES = [uk.KERNEL_MODE_AUTO, uk.KERNEL_MODE_GENERIC, uk.KERNEL_MODE_MFMA_VARIANT + 1,
          uk.KERNEL_MODE_MFMA_VARIANT + 4, uk.KERNEL_MODE_MFMA_VARIANT + 5,
-         uk.KERNEL_MODE_MFMA_VARIANT + 8]
+         uk.KERNEL_MODE_MFMA_VARIANT + 8, uk.KERNEL_MODE_MFMA_VARIANT + 16]
 
 
 @pytest.mark.gpu

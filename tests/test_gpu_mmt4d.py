@@ -87,9 +87,11 @@ def _mfma_shapes(M0, N0, K0, bits):
 # bytes wide, else the 32x64 kernel through LDS: the shapes below have both;
 # 5 is the thin kernel on the transposed problem and 6 the same kernel with
 # 64x64 blocks, under the same conditions; 7 is the 256x128 shape, 8 the
-# 128x512 shape; 11 is the 64x64 shape with the deep pipeline, and 12 .. 15 are
+# 128x512 shape; 11 is the 64x64 shape with the deep pipeline, 12 .. 15 are
 # the narrow-row kernels in the 256x256 / 128x512 / 128x128 / 64x64 shape, which
-# serve tile rows of 2 or 4 bytes with N0 = 16 and hand everything else on).
+# serve tile rows of 2 or 4 bytes with N0 = 16 and hand everything else on, and
+# 16 / 17 the LDS-direct ping-pong pipeline in the 256x256 / 128x512 shape, for
+# tile rows of 16 bytes and more).
 # Tile rows of one byte (s8, K0 = 1) have no MFMA kernel: iree_uk_mmt4d_info
 # says so and the reference grid above covers them on the scalar kernel. The
 # entry stays in the list, named for what it is, and is asserted unserved.
@@ -103,19 +105,23 @@ def _variant_applies(n, variant):
     """Forced shapes that a tile cannot take hand the call on to the choice by
     size, i.e. repeat variant 0: the deep 64x64 pipeline (11) exists for tile
     rows under 16 bytes, the narrow-row kernels (12 .. 15) for rows of 2 or 4
-    bytes with N0 = 16."""
+    bytes with N0 = 16, the LDS-direct pipeline (16, 17) for rows of 16 bytes
+    and more."""
     tf, M0, N0, K0 = MFMA_TILES[n]
     row_bytes = K0 * uk.MMT4D_TYPE_BITS[tf][0] // 8
     if variant == 11:
         return row_bytes < 16
     if variant in (12, 13, 14, 15):
         return row_bytes in (2, 4) and N0 == 16
+    if variant in (16, 17):
+        # the LDS-direct pipeline: rows of 16 bytes and more, one 16-byte piece per lane operand
+        return row_bytes >= 16 and tf != uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32
     return True
 
 
 _TILE_VARIANTS = [pytest.param(n, v, id=f"{_tile_id(n)}-{v}")
                   for n in range(len(MFMA_TILES))
-                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15) if _variant_applies(n, v)]
+                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15, 16, 17) if _variant_applies(n, v)]
 
 
 @pytest.mark.parametrize("n,variant", _TILE_VARIANTS)
@@ -165,7 +171,7 @@ def test_mmt4d_split_off_remainder_strips(gpu, oracle, shape):
 # single rounding at the end (SKIP_INTERMEDIATE_ROUNDINGS); on the reference
 # tests' small-integer inputs every f32 partial sum is exact, so the result must
 # equal the oracle's bit for bit, final rounding included.
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 8])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 8, 16])
 @pytest.mark.parametrize("tf,M0,N0,K0", [
     (uk.MMT4D_TYPE_F16F16F16, 16, 16, 8), (uk.MMT4D_TYPE_F16F16F16, 16, 16, 1),
     (uk.MMT4D_TYPE_BF16BF16BF16, 16, 16, 8), (uk.MMT4D_TYPE_BF16BF16BF16, 8, 32, 2)])
@@ -226,7 +232,7 @@ def _normal_operand(rng, kind, n, scale=1.0):
     (uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32, 16, 16, 32),
     (uk.MMT4D_TYPE_F32F32F32, 8, 8, 4), (uk.MMT4D_TYPE_F32F32F32, 16, 16, 1)])
 @pytest.mark.parametrize("accumulate", [0, 1])
-@pytest.mark.parametrize("variant", [0, 1, 8])
+@pytest.mark.parametrize("variant", [0, 1, 8, 16, 17])
 def test_mmt4d_float_tolerance_on_normal_inputs(gpu, oracle, tf, M0, N0, K0, accumulate, variant):
     lib, torch = gpu
     lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
@@ -274,7 +280,7 @@ def _pow2_bits(tf, exponent: int) -> int:
 
 @pytest.mark.parametrize("tf,sub_e,big_e", [(uk.MMT4D_TYPE_F16F16F32, -20, 10),
                                              (uk.MMT4D_TYPE_BF16BF16F32, -130, 100)])
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 8, 16])
 def test_mmt4d_subnormal_inputs_matrix_cores_keep_scalar_kernel_flushes(gpu, oracle, tf, sub_e, big_e, variant):
     """Pins how subnormal f16 / bf16 inputs are read. The reference's generic
     tile functions flush them to zero (common.h:664-700), and so do the oracle
@@ -562,8 +568,8 @@ def test_mmt4d_persistent_kernels(gpu, oracle, variant, tile, workgroups):
 
 
 def test_mmt4d_last_partial_round_runs_as_its_own_launch(gpu):
-    """A problem that the 128x512 shape tiles exactly into 1.25 rounds of
-    blocks (2 x 160 = 320 on 256 compute units) is split by columns: whole
+    """A problem that the 128x512 shape (and the 256x256 one) tiles exactly into
+    1.25 rounds of blocks (320 on 256 compute units) is split by columns: whole
     rounds in one launch, the last 32 block columns in another with a smaller
     shape. Results equal the single launch of a forced shape bit for bit, the
     column scales of the dequantizing store included."""
@@ -598,7 +604,7 @@ def test_mmt4d_last_partial_round_runs_as_its_own_launch(gpu):
             lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
         results[mode] = (out.cpu(), y.cpu(), name)
     auto, forced = results[uk.KERNEL_MODE_AUTO], results[uk.KERNEL_MODE_MFMA_VARIANT + 1]
-    assert auto[2] == "mmt4d_mfma_128x512_rhs_direct" and forced[2] == "mmt4d_mfma_256x256_rhs_direct"
+    assert auto[2] == "mmt4d_mfma_256x256_lds_direct" and forced[2] == "mmt4d_mfma_256x256_rhs_direct"
     assert torch.equal(auto[0], forced[0])
     assert torch.equal(auto[1], forced[1])
     # and against the integer product on a few rows and columns of both parts
