@@ -15,10 +15,16 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "obj")
 LIB = os.path.join(HERE, "libiree_uk_amd.so")
 
-HIP_SOURCES = ["mmt4d_mfma_s8.hip", "mmt4d_mfma_f16.hip", "mmt4d_mfma_bf16.hip",
-               "mmt4d_mfma_f8.hip", "mmt4d_mfma_f32.hip", "mmt4d_mfma_f16f16.hip", "mmt4d_mfma_bf16bf16.hip", "mmt4d_mfma_s8s4.hip",
+HIP_SOURCES = ["mmt4d_mfma_s8s4.hip",
                "uk_runtime.hip", "uk_probe.hip", "pack_unpack.hip",
                "mmt4d_generic.hip", "mmt4d_dot2.hip", "conv_nchwc.hip", "mmt4d_mfma.hip", "mmt4d_dispatch.hip"]
+# mmt4d_mfma_inst.hip once per (element type, class of tile row widths): the
+# kernel instantiations of one pair per object file, built in parallel.
+MFMA_TYPES = {"s8": "kS8", "f16": "kF16", "bf16": "kBF16", "f16f16": "kF16F16",
+              "bf16bf16": "kBF16BF16", "f32": "kF32", "f8": "kF8"}
+MFMA_ROW_CLASSES = {"f32": (4, 8, 16), "f8": (16,)}
+MFMA_INSTANCES = [(t, e, rb) for t, e in MFMA_TYPES.items()
+                  for rb in MFMA_ROW_CLASSES.get(t, (2, 4, 8, 16))]
 C_SOURCES = ["uk_host.c", "uk_plugin.c"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -56,6 +62,13 @@ def build(verbose: bool = False) -> str:
         o = os.path.join(OBJ, s + ".o")
         objs.append(o)
         jobs.append([HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, s), "-o", o])
+    for t, e, rb in MFMA_INSTANCES:
+        o = os.path.join(OBJ, f"mmt4d_mfma_inst_{t}_rb{rb}.o")
+        objs.append(o)
+        # the longest compilations first
+        jobs.insert(0, [HIPCC, *HIP_FLAGS, f"-DUK_INST_ELEM={e}", f"-DUK_INST_RBC={rb}",
+                        f"-DUK_INST_NAME=launch_{t}_rb{rb}", "-c",
+                        os.path.join(CSRC, "mmt4d_mfma_inst.hip"), "-o", o])
     for s in C_SOURCES:
         o = os.path.join(OBJ, s + ".o")
         objs.append(o)

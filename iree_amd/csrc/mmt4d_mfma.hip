@@ -1,18 +1,55 @@
 // mmt4d on the gfx950 matrix cores: shape checks and per-type dispatch. The
 // kernel template lives in mmt4d_mfma_kernel.h, variant selection in
-// mmt4d_mfma_launch.h; each element type is compiled in its own file.
+// mmt4d_mfma_launch.h; each element type and class of row widths is compiled on
+// its own (mmt4d_mfma_inst.hip).
 #include <hip/hip_runtime.h>
 
 #include "mmt4d_mfma_launch.h"
 
 namespace uk_mfma {
-int launch_s8(const Problem& p, int forced, hipStream_t stream, const char** name);
-int launch_f16(const Problem& p, int forced, hipStream_t stream, const char** name);
-int launch_bf16(const Problem& p, int forced, hipStream_t stream, const char** name);
-int launch_f8(const Problem& p, int forced, hipStream_t stream, const char** name);
-int launch_f32(const Problem& p, int forced, hipStream_t stream, const char** name);
-int launch_f16f16(const Problem& p, int forced, hipStream_t stream, const char** name);
-int launch_bf16bf16(const Problem& p, int forced, hipStream_t stream, const char** name);
+// One function per element type and class of tile row widths (2, 4, 8, and 16
+// bytes and more), each defined by its own compilation of mmt4d_mfma_inst.hip.
+#define UK_DECLARE_ROW_CLASSES(T)                                                         \
+  int launch_##T##_rb2(const Problem& p, int forced, hipStream_t stream, const char** name); \
+  int launch_##T##_rb4(const Problem& p, int forced, hipStream_t stream, const char** name); \
+  int launch_##T##_rb8(const Problem& p, int forced, hipStream_t stream, const char** name); \
+  int launch_##T##_rb16(const Problem& p, int forced, hipStream_t stream, const char** name);
+UK_DECLARE_ROW_CLASSES(s8)
+UK_DECLARE_ROW_CLASSES(f16)
+UK_DECLARE_ROW_CLASSES(bf16)
+UK_DECLARE_ROW_CLASSES(f16f16)
+UK_DECLARE_ROW_CLASSES(bf16bf16)
+int launch_f32_rb4(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_f32_rb8(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_f32_rb16(const Problem& p, int forced, hipStream_t stream, const char** name);
+int launch_f8_rb16(const Problem& p, int forced, hipStream_t stream, const char** name);
+#undef UK_DECLARE_ROW_CLASSES
+#define UK_DEFINE_BY_ROW_BYTES(T)                                                            \
+  inline int launch_##T(const Problem& p, int forced, hipStream_t stream, const char** name) { \
+    switch (p.rb) {                                                                          \
+      case 2: return launch_##T##_rb2(p, forced, stream, name);                              \
+      case 4: return launch_##T##_rb4(p, forced, stream, name);                              \
+      case 8: return launch_##T##_rb8(p, forced, stream, name);                              \
+      default: return launch_##T##_rb16(p, forced, stream, name);                            \
+    }                                                                                        \
+  }
+UK_DEFINE_BY_ROW_BYTES(s8)
+UK_DEFINE_BY_ROW_BYTES(f16)
+UK_DEFINE_BY_ROW_BYTES(bf16)
+UK_DEFINE_BY_ROW_BYTES(f16f16)
+UK_DEFINE_BY_ROW_BYTES(bf16bf16)
+#undef UK_DEFINE_BY_ROW_BYTES
+inline int launch_f32(const Problem& p, int forced, hipStream_t stream, const char** name) {
+  switch (p.rb) {
+    case 2: return -1;
+    case 4: return launch_f32_rb4(p, forced, stream, name);
+    case 8: return launch_f32_rb8(p, forced, stream, name);
+    default: return launch_f32_rb16(p, forced, stream, name);
+  }
+}
+inline int launch_f8(const Problem& p, int forced, hipStream_t stream, const char** name) {
+  return p.rb >= 16 ? launch_f8_rb16(p, forced, stream, name) : -1;
+}
 int launch_s8s4(const Problem& p, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 

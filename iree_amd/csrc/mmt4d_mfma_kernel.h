@@ -968,36 +968,134 @@ void mmt4d_mfma_kernel(Args a) {
     // earlier barrier). Past the last step the loads repeat the last step into
     // a stage nobody reads any more, which keeps the in-flight count the waits
     // assume.
-    static_assert(RBC >= 16 && HALVES == 1 && NKK == 1, "one 1 KiB block per loader unit and fragment");
-    static_assert(NW == 8 && EVEN, "two groups of four waves");
+    //
+    // Tile rows of 16 bytes and more: a 1 KiB block of the LDS image (16 rows x
+    // 64 bytes of K) is the MFMA fragment as it is. Tile rows of 2 or 4 bytes
+    // (the reference's x86 tiles 16x16x2 of s8 and bf16): the loads copy the
+    // K-tiles as they lie in memory, 16 rows x RB bytes each, one after the
+    // other ([K-tile][row][RB]: again 1 KiB per 16-row block and step, a
+    // 16-byte piece holding 16 / RB rows of one K-tile), and the fragment reads
+    // gather a row's pieces:
+    //   RB = 8  lane (q, r) reads the 8 bytes of row r in K-tiles q and q + 4
+    //           (one ds_read2_b64);
+    //   RB = 4  lane (q, r) reads the dwords of row r in K-tiles q, q + 4,
+    //           q + 8, q + 12 (two ds_read2st64_b32);
+    //   RB = 2  two transposing reads (ds_read_b64_tr_b16). Within a block of 16
+    //           lanes, lane i receives as element j the element i % 4 of what
+    //           lane 4 j + i / 4 addressed: lane (q, s) addresses rows
+    //           4 (s % 4) .. + 3 of K-tile 16 h + 4 q + s / 4 (eight contiguous
+    //           bytes) and lane (q, r) receives row r of K-tiles 16 h + 4 q .. + 3.
+    // Which K bytes of a step meet in which lane operand is the same for both
+    // operands, which is all the sum over K needs.
+    // A step of NKK x 64 bytes of K holds NKK such blocks per 16 rows, one
+    // after the other ([row block][64-byte chunk of K]).
+    static_assert((RBC >= 16 || RBC == 2 || RBC == 4 || RBC == 8) && HALVES == 1,
+                  "1 KiB blocks of 16 rows x 64 bytes of K");
+    static_assert(NW == 8, "two groups of four waves");
     constexpr int NS = kStages5;
+    constexpr int DB = (BM + BN) / 16 * NKK;  // 1 KiB blocks in a step's LDS image
+    static_assert(DB % NW == 0, "blocks split evenly over the waves");
+    constexpr int DU = DB / NW;
     const int group = wave >> 2;
+    const char* d_base[DU];
+    uint32_t d_voff[DU], d_step[DU], d_lds[DU];
+#pragma unroll
+    for (int i = 0; i < DU; ++i) {
+      if constexpr (RBC >= 16) {
+        static_assert(RBC < 16 || DU == NU, "the loader units are the 1 KiB blocks");
+        d_base[i] = sbase[i];
+        d_voff[i] = voff[i];
+        d_step[i] = sstep[i];
+        d_lds[i] = ldma[i];
+      } else {
+        constexpr int RP = 16 / RBC;   // rows of a K-tile in one 16-byte piece
+        constexpr int PPK = 16 / RP;   // pieces per K-tile of a 16-row block
+        const int blk = wave + i * NW;
+        const bool is_b = blk >= BM / 16 * NKK;
+        const int xblk = is_b ? blk - BM / 16 * NKK : blk;   // (row block, chunk) of the operand's image
+        const int rbk = xblk / NKK, chunk = xblk - rbk * NKK;
+        const int X0 = is_b ? a.N0 : a.M0;
+        const int X1 = is_b ? a.N1 : a.M1;
+        const int px0 = is_b ? pn0 : pm0;
+        const int bpx = is_b ? a.bpn : a.bpm;
+        const int64_t xstride = is_b ? a.rhs_stride : a.lhs_stride;
+        const uint32_t kt_bytes = (uint32_t)X0 * RBC;
+        const uint32_t row0 = (uint32_t)rbk * 16 + ((uint32_t)lane % PPK) * RP;
+        const uint32_t pl = row0 / (uint32_t)X0, x0 = row0 - pl * (uint32_t)X0;
+        const uint32_t kt_l = (uint32_t)chunk * (64 / RBC) + (uint32_t)lane / PPK;  // K-tile within the step
+        d_base[i] = (is_b ? a.rhs : a.lhs) + (int64_t)px0 * xstride;
+        d_voff[i] = pl * (uint32_t)xstride + kt_l * kt_bytes + x0 * RBC;
+        if (!((int)pl < bpx && px0 + (int)pl < X1)) d_voff[i] = 0;  // rows beyond the problem: valid bytes, never stored
+        d_step[i] = (uint32_t)(KS / RBC) * kt_bytes;
+        d_lds[i] = (is_b ? IMAGE_A : 0u) + (uint32_t)xblk * 1024;
+      }
+    }
     auto issue_dma = [&](uint32_t stage_off, int step) {
 #pragma unroll
-      for (int i = 0; i < NU; ++i) {
-        uint32_t o = voff[i] + (uint32_t)step * sstep[i];
+      for (int i = 0; i < DU; ++i) {
+        uint32_t o = d_voff[i] + (uint32_t)step * d_step[i];
         // (kept as scalar base + 32-bit lane offset: see mmt4d_mfma_persistent.h)
         asm volatile("" : "+v"(o));
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(sbase[i] + o),
-                                         (lds_ptr_t)(lds + stage_off + ldma[i]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(d_base[i] + o),
+                                         (lds_ptr_t)(lds + stage_off + d_lds[i]), 16, 0, 0);
+      }
+    };
+    // Lane offset of a fragment read within its 1 KiB block.
+    const uint32_t frag_lane = RBC >= 16 ? (uint32_t)lane * 16
+                               : RBC == 8 ? q * 128 + r * 8
+                               : RBC == 4 ? q * 64 + r * 4
+                                          : (4 * q + (r >> 2)) * 32 + (r & 3) * 8;
+    auto read_frag = [&](uint32_t block_off) -> v4i {
+      const char* p = lds + block_off + frag_lane;
+      if constexpr (RBC >= 16) {
+        return *reinterpret_cast<const v4i*>(p);
+      } else if constexpr (RBC == 8) {
+        typedef int v2i __attribute__((ext_vector_type(2)));
+        const v2i* w = reinterpret_cast<const v2i*>(p);
+        const v2i lo = w[0], hi = w[64];
+        return v4i{lo[0], lo[1], hi[0], hi[1]};
+      } else if constexpr (RBC == 4) {
+        const int* w = reinterpret_cast<const int*>(p);
+        return v4i{w[0], w[64], w[128], w[192]};
+      } else {
+        // Written as assembly: the compiler does not track what the LDS-direct
+        // loads write and would make the builtin form of this read wait for
+        // every load in flight. The kernel waits for these reads itself
+        // (wait_lds_reads before the phase's barrier; nothing uses the
+        // registers before it).
+        typedef int v2i __attribute__((ext_vector_type(2)));
+        v2i lo, hi;
+        const uint32_t addr = (uint32_t)(uintptr_t)p;  // LDS addresses are the low 32 bits
+        asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:512"
+                     : "=&v"(lo), "=&v"(hi) : "v"(addr) : "memory");
+        return v4i{lo[0], lo[1], hi[0], hi[1]};
       }
     };
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s) issue_dma(s * STAGE, min(s, last));
-    wait_vmem_in_flight<NU*(NS - 2)>();
+    wait_vmem_in_flight<DU*(NS - 2)>();
     __builtin_amdgcn_s_barrier();
     if (group == 1) __builtin_amdgcn_s_barrier();
-    v4i fa[TM][HALVES], fb[TN][HALVES];
+    v4i fa[NKK][TM][HALVES], fb[NKK][TN][HALVES];
     auto step_body = [&](int s, auto stage_c) {
       constexpr int ST = decltype(stage_c)::value;
-      read_frags(fa, fb, ST * STAGE, 0);
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          fa[kk][tm][0] = read_frag(ST * STAGE + (uint32_t)((wm * TM + tm) * NKK + kk) * 1024);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          fb[kk][tn][0] = read_frag(ST * STAGE + IMAGE_A + (uint32_t)((wn * TN + tn) * NKK + kk) * 1024);
+      }
       issue_dma(((ST + NS - 1) % NS) * STAGE, min(s + NS - 1, last));
-      wait_vmem_in_flight<NU*(NS - 2)>();
+      wait_vmem_in_flight<DU*(NS - 2)>();
       wait_lds_reads();
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      mfmas(fa, fb);
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) mfmas(fa[kk], fb[kk]);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);

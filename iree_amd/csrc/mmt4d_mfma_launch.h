@@ -409,8 +409,8 @@ inline int64_t workgroups(const Problem& p, int BM, int BN) {
 // 9 / 10 the persistent kernel in the 128x512 / 256x256 shape, 11 the 64x64
 // shape with 256-byte steps three steps ahead (tile rows under 16 bytes),
 // 12 .. 15 the narrow-row kernel (tile rows of 2 or 4 bytes, N0 = 16) in the
-// 256x256 / 128x512 / 128x128 / 64x64 shape, 16 / 17 the LDS-direct ping-pong
-// pipeline in the 256x256 / 128x512 shape;
+// 256x256 / 128x512 / 128x128 / 64x64 shape, 16 / 17 / 18 / 19 the LDS-direct
+// ping-pong pipeline in the 256x256 / 128x512 / 128x128 / 64x64 shape;
 // 0 = choose) overrides the
 // size heuristic for tests and tuning.
 //   thin  M-thin (decode-shaped) problems, up to 64 rows, which are bound by
@@ -440,6 +440,10 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 2;  // the narrow-row kernel in the 128x128 shape
   } else if (forced == 16 || forced == 17) {
     choice = 1;  // the LDS-direct ping-pong pipeline in the 256x256 (16) or 128x512 (17) shape
+  } else if (forced == 18) {
+    choice = 2;  // the same pipeline in the 128x128 shape
+  } else if (forced == 19) {
+    choice = 3;  // and in the 64x64 shape with 256-byte steps
   } else if (forced >= 8 && forced <= 10) {
     // The big variant in its 128x512 shape (8), the persistent kernel in that
     // shape (9) or in the square one (10); the plain square shape where the
@@ -553,9 +557,39 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   // of K (less than one step) to the two-stage variant of the same or a
   // smaller workgroup shape, as a second, accumulating launch.
   const int kts_per_step = BIG_KS >> p.lrb;
-  const int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
+  // 16-bit outputs are rounded once, after all of K (the reference's
+  // SKIP_INTERMEDIATE_ROUNDINGS semantics): a second launch would continue from
+  // a rounded value. With a K remainder they take the variants that run any K
+  // in one launch.
+  constexpr bool kOneLaunchOnly = ElemTraits<E>::Out::kOutBytes == 2;
+  int kt_main = kts_per_step > 0 ? (p.K1 / kts_per_step) * kts_per_step : 0;
+  if (kOneLaunchOnly && kt_main != p.K1) kt_main = 0;
   constexpr bool NARROW = (RBC == 2 || RBC == 4) && H == 1 && ElemTraits<E>::Out::kOutBytes == 4;
   if (choice == 1) {
+    if constexpr (RBC < 16 && H == 1) {
+      // Tile rows of 2, 4 or 8 bytes through the LDS-direct ping-pong pipeline
+      // (PIPE 5 of mmt4d_mfma_kernel.h: the loads copy the K-tiles as they lie
+      // in memory, the fragment reads gather each row's pieces).
+      // Measured against the register-regrouping kernels at 8192^3: s8 16x16x2
+      // 496 -> 382 us, bf16 16x16x2 932 -> 726 us, s8 16x16x8 486 -> 383 us; at
+      // 4096^3 s8 16x16x2 76 -> 57 us. (f32 keeps its kernels, as below.)
+      if (kt_main > 0 && (forced == 16 || forced == 17 || (forced == 0 && E != Elem::kF32))) {
+        int st = -1;
+        if (forced == 17) {
+          st = launch_variant<E, RBC, 8, 4, 1, 8, 1, 5>(p, 0, kt_main, p.accumulate, stream);
+          if (st == 0) *name = "mmt4d_mfma_128x512_lds_direct";
+        }
+        if (st < 0) {
+          st = launch_variant<E, RBC, 8, 4, 2, 4, 1, 5>(p, 0, kt_main, p.accumulate, stream);
+          if (st == 0) *name = "mmt4d_mfma_256x256_lds_direct";
+        }
+        if (st == 0) {
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
+    }
     if constexpr (NARROW) {
       // Tile rows of 2 or 4 bytes with N0 = 16 (the x86-style tiles): the RHS
       // goes straight to registers here too (mmt4d_mfma_narrow.h).
@@ -729,6 +763,20 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 3;
   }
   if (choice == 2) {
+    if constexpr (H == 1) {
+      // The LDS-direct ping-pong pipeline with 8 waves of 64x32 (measured against
+      // the kernels below: s8 2048^3 16x16x2 20.6 -> 14.7 us, 16x16x16 14.8 ->
+      // 14.5 us; 3072^3 40.5 -> 36.3 us; bf16 2048^3 23.4 -> 22.6 us).
+      if (kt_main > 0 && (forced == 18 || (forced == 0 && E != Elem::kF32))) {
+        int st = launch_variant<E, RBC, 4, 2, 2, 4, 1, 5>(p, 0, kt_main, p.accumulate, stream);
+        if (st == 0) {
+          *name = "mmt4d_mfma_128x128_lds_direct";
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
+    }
     if constexpr (NARROW) {
       // (Not chosen by size: measured level with or behind the 128x128 kernel
       // that sends both operands through LDS.)
@@ -755,6 +803,21 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     }
     int st = launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
     if (st >= 0) { *name = "mmt4d_mfma_128x128"; return st; }
+  }
+  if constexpr (H == 1) {
+    // 64x64 blocks, 8 waves of 32x16, 256 bytes of K per step (forced only).
+    const int kts256 = 256 >> p.lrb;
+    int kt_main256 = kts256 > 0 ? (p.K1 / kts256) * kts256 : 0;
+    if (kOneLaunchOnly && kt_main256 != p.K1) kt_main256 = 0;
+    if (kt_main256 > 0 && forced == 19) {
+      int st = launch_variant<E, RBC, 2, 1, 2, 4, 4, 5>(p, 0, kt_main256, p.accumulate, stream);
+      if (st == 0) {
+        *name = "mmt4d_mfma_64x64_lds_direct";
+        if (kt_main256 == p.K1) return 0;
+        return finish_k(launch_variant<E, RBC, 2, 2, 2, 2, NKK2, 0>(p, kt_main256, p.K1 - kt_main256, true, stream));
+      }
+      if (st > 0) return st;
+    }
   }
   if constexpr (RBC >= 16) {
     if (kt_main > 0) {
@@ -793,27 +856,6 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
   st = launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, 0, p.K1, p.accumulate, stream);
   if (st >= 0) *name = "mmt4d_mfma_128x128";
   return st;
-}
-
-template <Elem E>
-int launch_elem(const Problem& p, int forced, hipStream_t stream, const char** name) {
-  if constexpr (E == Elem::kF8) {
-    return p.rb >= 16 ? launch_class<E, 16>(p, forced, stream, name) : -1;
-  } else if constexpr (E == Elem::kF32) {
-    switch (p.rb) {
-      case 2: return -1;
-      case 4: return launch_class<E, 4>(p, forced, stream, name);
-      case 8: return launch_class<E, 8>(p, forced, stream, name);
-      default: return launch_class<E, 16>(p, forced, stream, name);
-    }
-  } else {
-    switch (p.rb) {
-      case 2: return launch_class<E, 2>(p, forced, stream, name);
-      case 4: return launch_class<E, 4>(p, forced, stream, name);
-      case 8: return launch_class<E, 8>(p, forced, stream, name);
-      default: return launch_class<E, 16>(p, forced, stream, name);
-    }
-  }
 }
 
 }  // namespace uk_mfma

@@ -90,8 +90,8 @@ def _mfma_shapes(M0, N0, K0, bits):
 # 128x512 shape; 11 is the 64x64 shape with the deep pipeline, 12 .. 15 are
 # the narrow-row kernels in the 256x256 / 128x512 / 128x128 / 64x64 shape, which
 # serve tile rows of 2 or 4 bytes with N0 = 16 and hand everything else on, and
-# 16 / 17 the LDS-direct ping-pong pipeline in the 256x256 / 128x512 shape, for
-# tile rows of 16 bytes and more).
+# 16 .. 19 the LDS-direct ping-pong pipeline in the 256x256 / 128x512 / 128x128 /
+# 64x64 shape).
 # Tile rows of one byte (s8, K0 = 1) have no MFMA kernel: iree_uk_mmt4d_info
 # says so and the reference grid above covers them on the scalar kernel. The
 # entry stays in the list, named for what it is, and is asserted unserved.
@@ -105,23 +105,23 @@ def _variant_applies(n, variant):
     """Forced shapes that a tile cannot take hand the call on to the choice by
     size, i.e. repeat variant 0: the deep 64x64 pipeline (11) exists for tile
     rows under 16 bytes, the narrow-row kernels (12 .. 15) for rows of 2 or 4
-    bytes with N0 = 16, the LDS-direct pipeline (16, 17) for rows of 16 bytes
-    and more."""
+    bytes with N0 = 16, the LDS-direct pipeline (16 .. 19) for every type but the
+    8-bit floats."""
     tf, M0, N0, K0 = MFMA_TILES[n]
     row_bytes = K0 * uk.MMT4D_TYPE_BITS[tf][0] // 8
     if variant == 11:
         return row_bytes < 16
     if variant in (12, 13, 14, 15):
         return row_bytes in (2, 4) and N0 == 16
-    if variant in (16, 17):
-        # the LDS-direct pipeline: rows of 16 bytes and more, one 16-byte piece per lane operand
-        return row_bytes >= 16 and tf != uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32
+    if variant in (16, 17, 18, 19):
+        # the LDS-direct pipeline: one 16-byte piece per lane operand (not the 8-bit floats)
+        return tf != uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32
     return True
 
 
 _TILE_VARIANTS = [pytest.param(n, v, id=f"{_tile_id(n)}-{v}")
                   for n in range(len(MFMA_TILES))
-                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15, 16, 17) if _variant_applies(n, v)]
+                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15, 16, 17, 18, 19) if _variant_applies(n, v)]
 
 
 @pytest.mark.parametrize("n,variant", _TILE_VARIANTS)
@@ -191,6 +191,29 @@ def test_mmt4d_16bit_outputs_single_rounding(gpu, oracle, tf, M0, N0, K0, varian
         assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
         if c.M and c.N and c.K:
             assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 8, 16, 17, 18, 19])
+@pytest.mark.parametrize("tf", [uk.MMT4D_TYPE_F16F16F16, uk.MMT4D_TYPE_BF16BF16BF16])
+def test_mmt4d_16bit_outputs_round_once_when_k_has_a_remainder(gpu, oracle, tf, variant):
+    """Sums that no longer fit a 16-bit float exactly (small-integer inputs, a
+    long K, ACCUMULATE) with K a few tiles past a whole number of pipeline
+    steps: the result is rounded once, after all of K, whatever kernel is
+    forced. A library that ran the remainder of K as a second launch on top of
+    the rounded result of the first would differ in some elements."""
+    lib, torch = gpu
+    M0, N0, K0 = 24, 64, 4
+    flags = tf | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS | uk.MMT4D_ACCUMULATE
+    lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + variant if variant else uk.KERNEL_MODE_AUTO)
+    for seed, (M, N, K) in enumerate(((12, 3, 130), (5, 9, 259), (11, 4, 33))):
+        c = T.Mmt4dCase(flags, M, N, K, M0, N0, K0, K * M0 * K0 + 16, K * N0 * K0, N * M0 * N0 + 16, 16, 0, 0)
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(99 + seed))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+        assert lib.last_kernel_name().startswith("mmt4d_mfma"), lib.last_kernel_name()
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
 
 
 def test_mmt4d_single_row_tiles_equal_row_major_matmul(gpu):
