@@ -363,7 +363,6 @@ void mmt4d_mfma_kernel(Args a) {
   uint32_t skt[NU];      // bytes between consecutive loads of a unit
   int32_t kt0[NU];       // K-tile index of the first load at step 0
   uint32_t loff[NU];     // LDS offset (within a stage) of the unit's first store
-  uint32_t ldma[NU];     // PIPE 5: LDS offset of the unit's 1 KiB block (uniform: lane 0's slot)
   // Regrouping loaders only: false for a unit whose rows lie beyond the
   // operand's LDS image. That happens when the tile height does not divide
   // the block (e.g. M0 = 24 in a 64-row block: the units of a third, partial
@@ -399,7 +398,6 @@ void mmt4d_mfma_kernel(Args a) {
       skt[i] = 0;
       lds_ok[i] = true;
       loff[i] = image + (uint32_t)xblk * 1024 + lane * 16;
-      ldma[i] = image + (uint32_t)xblk * 1024;
     } else {
       // Units in order [panel][chunk g][row group]; the unit's R loads read
       // K-tiles g, g + NCH, g + 2*NCH, ... so that one load instruction covers
@@ -420,7 +418,6 @@ void mmt4d_mfma_kernel(Args a) {
       // only touches the low bits and the store applies j ^ ... itself.
       loff[i] = image + (((row >> 4) * NCHB + (g >> 2)) * 64 + (g & 3) * 16) * 16 +
                 ((rr & 8) | ((rr & 7) ^ swizzle_mask(g, rr >> 3))) * 16;
-      ldma[i] = 0;
     }
     // Units outside the problem read from the start of the first panel.
     if (!(pl < bpx && px0 + pl < X1)) voff[i] = 0;
@@ -989,55 +986,68 @@ void mmt4d_mfma_kernel(Args a) {
     // operands, which is all the sum over K needs.
     // A step of NKK x 64 bytes of K holds NKK such blocks per 16 rows, one
     // after the other ([row block][64-byte chunk of K]).
-    static_assert((RBC >= 16 || RBC == 2 || RBC == 4 || RBC == 8) && HALVES == 1,
+    static_assert(RBC >= 16 || ((RBC == 2 || RBC == 4 || RBC == 8) && HALVES == 1),
                   "1 KiB blocks of 16 rows x 64 bytes of K");
     static_assert(NW == 8, "two groups of four waves");
+    // Lane operands of two 16-byte pieces (the 8-bit floats: 128 bytes of K per
+    // step, i.e. two 64-byte halves) do not leave room for four stages of whole
+    // steps: their LDS is a ring of five half-step slots instead (HALVES == 2
+    // below).
     constexpr int NS = kStages5;
-    constexpr int DB = (BM + BN) / 16 * NKK;  // 1 KiB blocks in a step's LDS image
-    static_assert(DB % NW == 0, "blocks split evenly over the waves");
-    constexpr int DU = DB / NW;
+    constexpr int IW = HALVES == 2 ? 4 : NW;          // waves that share one issue of loads
+    constexpr int DCH = HALVES == 2 ? 1 : NCHB;       // 64-byte chunks of K per issue
+    constexpr int DB = (BM + BN) / 16 * DCH;          // 1 KiB blocks per issue
+    static_assert(DB % IW == 0, "blocks split evenly over the issuing waves");
+    constexpr int DU = DB / IW;
     const int group = wave >> 2;
     const char* d_base[DU];
-    uint32_t d_voff[DU], d_step[DU], d_lds[DU];
+    uint32_t d_voff[DU], d_step[DU], d_half[DU], d_lds[DU];
 #pragma unroll
     for (int i = 0; i < DU; ++i) {
+      const int blk = (wave & (IW - 1)) + i * IW;
+      const bool is_b = blk >= BM / 16 * DCH;
+      const int xblk = is_b ? blk - BM / 16 * DCH : blk;   // (row block, 64-byte chunk) of the operand's image
+      const int rbk = xblk / DCH, chunk = xblk - rbk * DCH;
+      const int X0 = is_b ? a.N0 : a.M0;
+      const int X1 = is_b ? a.N1 : a.M1;
+      const int px0 = is_b ? pn0 : pm0;
+      const int bpx = is_b ? a.bpn : a.bpm;
+      const int64_t xstride = is_b ? a.rhs_stride : a.lhs_stride;
+      const uint32_t kt_bytes = (uint32_t)X0 << lrb;
+      uint32_t pl;
       if constexpr (RBC >= 16) {
-        static_assert(RBC < 16 || DU == NU, "the loader units are the 1 KiB blocks");
-        d_base[i] = sbase[i];
-        d_voff[i] = voff[i];
-        d_step[i] = sstep[i];
-        d_lds[i] = ldma[i];
+        // Lane (q, r): row r of the block, bytes 16 q .. 16 q + 15 of the chunk.
+        const uint32_t row = (uint32_t)rbk * 16 + r;
+        pl = row / (uint32_t)X0;
+        const uint32_t x0 = row - pl * (uint32_t)X0;
+        const uint32_t kb = (uint32_t)(chunk * 4 + q) * 16;
+        d_voff[i] = pl * (uint32_t)xstride + (kb >> lrb) * kt_bytes + (x0 << lrb) + (kb & ((1u << lrb) - 1));
       } else {
         constexpr int RP = 16 / RBC;   // rows of a K-tile in one 16-byte piece
         constexpr int PPK = 16 / RP;   // pieces per K-tile of a 16-row block
-        const int blk = wave + i * NW;
-        const bool is_b = blk >= BM / 16 * NKK;
-        const int xblk = is_b ? blk - BM / 16 * NKK : blk;   // (row block, chunk) of the operand's image
-        const int rbk = xblk / NKK, chunk = xblk - rbk * NKK;
-        const int X0 = is_b ? a.N0 : a.M0;
-        const int X1 = is_b ? a.N1 : a.M1;
-        const int px0 = is_b ? pn0 : pm0;
-        const int bpx = is_b ? a.bpn : a.bpm;
-        const int64_t xstride = is_b ? a.rhs_stride : a.lhs_stride;
-        const uint32_t kt_bytes = (uint32_t)X0 * RBC;
         const uint32_t row0 = (uint32_t)rbk * 16 + ((uint32_t)lane % PPK) * RP;
-        const uint32_t pl = row0 / (uint32_t)X0, x0 = row0 - pl * (uint32_t)X0;
+        pl = row0 / (uint32_t)X0;
+        const uint32_t x0 = row0 - pl * (uint32_t)X0;
         const uint32_t kt_l = (uint32_t)chunk * (64 / RBC) + (uint32_t)lane / PPK;  // K-tile within the step
-        d_base[i] = (is_b ? a.rhs : a.lhs) + (int64_t)px0 * xstride;
         d_voff[i] = pl * (uint32_t)xstride + kt_l * kt_bytes + x0 * RBC;
-        if (!((int)pl < bpx && px0 + (int)pl < X1)) d_voff[i] = 0;  // rows beyond the problem: valid bytes, never stored
-        d_step[i] = (uint32_t)(KS / RBC) * kt_bytes;
-        d_lds[i] = (is_b ? IMAGE_A : 0u) + (uint32_t)xblk * 1024;
       }
+      if (!((int)pl < bpx && px0 + (int)pl < X1)) d_voff[i] = 0;  // rows beyond the problem: valid bytes, never stored
+      d_base[i] = (is_b ? a.rhs : a.lhs) + (int64_t)px0 * xstride;
+      d_step[i] = (uint32_t)kts_per_step * kt_bytes;
+      // From the first to the second 64-byte half of a 128-byte step: further
+      // along the tile row when it holds both, else on to later K-tiles.
+      d_half[i] = a.rb >= 128 ? 64u : (uint32_t)(64 >> lrb) * kt_bytes;
+      d_lds[i] = (is_b ? (uint32_t)BM * 64 * DCH : 0u) + (uint32_t)xblk * 1024;
     }
-    auto issue_dma = [&](uint32_t stage_off, int step) {
+    // Loads of one issue: `step` and `half` (0 / 1, HALVES == 2 only) select the K bytes.
+    auto issue_dma = [&](uint32_t lds_off, int step, int half) {
 #pragma unroll
       for (int i = 0; i < DU; ++i) {
-        uint32_t o = d_voff[i] + (uint32_t)step * d_step[i];
+        uint32_t o = d_voff[i] + (uint32_t)step * d_step[i] + (half ? d_half[i] : 0u);
         // (kept as scalar base + 32-bit lane offset: see mmt4d_mfma_persistent.h)
         asm volatile("" : "+v"(o));
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(d_base[i] + o),
-                                         (lds_ptr_t)(lds + stage_off + d_lds[i]), 16, 0, 0);
+                                         (lds_ptr_t)(lds + lds_off + d_lds[i]), 16, 0, 0);
       }
     };
     // Lane offset of a fragment read within its 1 KiB block.
@@ -1071,46 +1081,113 @@ void mmt4d_mfma_kernel(Args a) {
         return v4i{lo[0], lo[1], hi[0], hi[1]};
       }
     };
-#pragma unroll
-    for (int s = 0; s < NS - 1; ++s) issue_dma(s * STAGE, min(s, last));
-    wait_vmem_in_flight<DU*(NS - 2)>();
-    __builtin_amdgcn_s_barrier();
-    if (group == 1) __builtin_amdgcn_s_barrier();
-    v4i fa[NKK][TM][HALVES], fb[NKK][TN][HALVES];
-    auto step_body = [&](int s, auto stage_c) {
-      constexpr int ST = decltype(stage_c)::value;
-#pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) {
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-          fa[kk][tm][0] = read_frag(ST * STAGE + (uint32_t)((wm * TM + tm) * NKK + kk) * 1024);
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn)
-          fb[kk][tn][0] = read_frag(ST * STAGE + IMAGE_A + (uint32_t)((wn * TN + tn) * NKK + kk) * 1024);
+    if constexpr (HALVES == 2) {
+      // Five slots of half a step (64 bytes of K: (BM + BN) * 64 bytes of LDS);
+      // half-step j (step j / 2, half j % 2) lives in slot j % 5. In its memory
+      // phase of step s a wave reads both halves of the step; group 0 then
+      // issues the whole half-step 2 s + 3 (the slot of half-step 2 s - 2, which
+      // group 1 finished reading a phase ago) and waits for it at the end of its
+      // compute phase, one barrier before its first read; group 1 issues
+      // half-step 2 s + 4 (the slot of 2 s - 1) and waits for it at the end of
+      // its next memory phase, again one barrier before the first read. Both
+      // groups thus bring half of every step, each in its own memory phase.
+      static_assert(NKK == 1, "one MFMA K-group per step");
+      constexpr uint32_t SLOT = (BM + BN) * 64;
+      constexpr uint32_t IMG_B = BM * 64;
+      // Half-steps 0, 1, 2 before the first phase: group 1 brings 0 and 2, group 0 brings 1.
+      if (group == 0) {
+        issue_dma(1 * SLOT, 0, 1);
+      } else {
+        issue_dma(0 * SLOT, 0, 0);
+        issue_dma(2 * SLOT, min(1, last), 0);
       }
-      issue_dma(((ST + NS - 1) % NS) * STAGE, min(s + NS - 1, last));
-      wait_vmem_in_flight<DU*(NS - 2)>();
-      wait_lds_reads();
-      __builtin_amdgcn_sched_barrier(0);
+      wait_vmem_in_flight<0>();
       __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
+      if (group == 1) __builtin_amdgcn_s_barrier();
+      v4i fa[TM][HALVES], fb[TN][HALVES];
+      auto step_body = [&](int s, auto phase_c) {
+        constexpr int P = decltype(phase_c)::value;  // s % 5
 #pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) mfmas(fa[kk], fb[kk]);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int h = 0; h < 2; ++h) {
+          constexpr uint32_t unused = 0; (void)unused;
+          const uint32_t slot = (uint32_t)((2 * P + h) % 5) * SLOT;
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm) fa[tm][h] = read_frag(slot + (uint32_t)(wm * TM + tm) * 1024);
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) fb[tn][h] = read_frag(slot + IMG_B + (uint32_t)(wn * TN + tn) * 1024);
+        }
+        if (group == 0) {
+          issue_dma((uint32_t)((2 * P + 3) % 5) * SLOT, min(s + 1, last), 1);
+        } else {
+          issue_dma((uint32_t)((2 * P + 4) % 5) * SLOT, min(s + 2, last), 0);
+          wait_vmem_in_flight<DU>();   // the half-step issued a step ago has landed
+        }
+        wait_lds_reads();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(fa, fb);
+        __builtin_amdgcn_sched_barrier(0);
+        if (group == 0) wait_vmem_in_flight<0>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      int s = 0;
+      for (; s + 5 <= a.steps; s += 5) {
+        step_body(s, std::integral_constant<int, 0>{});
+        step_body(s + 1, std::integral_constant<int, 1>{});
+        step_body(s + 2, std::integral_constant<int, 2>{});
+        step_body(s + 3, std::integral_constant<int, 3>{});
+        step_body(s + 4, std::integral_constant<int, 4>{});
+      }
+      if (s < a.steps) step_body(s, std::integral_constant<int, 0>{});
+      if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
+      if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
+      if (s + 3 < a.steps) step_body(s + 3, std::integral_constant<int, 3>{});
+    } else {
+#pragma unroll
+      for (int s = 0; s < NS - 1; ++s) issue_dma(s * STAGE, min(s, last), 0);
+      wait_vmem_in_flight<DU*(NS - 2)>();
       __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    static_assert(NS == 4, "the loop below is unrolled by the stage count");
-    int s = 0;
-    for (; s + 4 <= a.steps; s += 4) {
-      step_body(s, std::integral_constant<int, 0>{});
-      step_body(s + 1, std::integral_constant<int, 1>{});
-      step_body(s + 2, std::integral_constant<int, 2>{});
-      step_body(s + 3, std::integral_constant<int, 3>{});
+      if (group == 1) __builtin_amdgcn_s_barrier();
+      // Fragment (row block b, MFMA K-group kk) sits in block b * NKK + kk of its
+      // operand's image.
+      v4i fa[NKK][TM][HALVES], fb[NKK][TN][HALVES];
+      auto step_body = [&](int s, auto stage_c) {
+        constexpr int ST = decltype(stage_c)::value;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm)
+            fa[kk][tm][0] = read_frag(ST * STAGE + (uint32_t)((wm * TM + tm) * NKK + kk) * 1024);
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            fb[kk][tn][0] = read_frag(ST * STAGE + IMAGE_A + (uint32_t)((wn * TN + tn) * NKK + kk) * 1024);
+        }
+        issue_dma(((ST + NS - 1) % NS) * STAGE, min(s + NS - 1, last), 0);
+        wait_vmem_in_flight<DU*(NS - 2)>();
+        wait_lds_reads();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) mfmas(fa[kk], fb[kk]);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      static_assert(NS == 4, "the loop below is unrolled by the stage count");
+      int s = 0;
+      for (; s + 4 <= a.steps; s += 4) {
+        step_body(s, std::integral_constant<int, 0>{});
+        step_body(s + 1, std::integral_constant<int, 1>{});
+        step_body(s + 2, std::integral_constant<int, 2>{});
+        step_body(s + 3, std::integral_constant<int, 3>{});
+      }
+      if (s < a.steps) step_body(s, std::integral_constant<int, 0>{});
+      if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
+      if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
     }
-    if (s < a.steps) step_body(s, std::integral_constant<int, 0>{});
-    if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
-    if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
     if (group == 0) __builtin_amdgcn_s_barrier();
     // No LDS-direct load may still be on its way when the workgroup ends (its
     // LDS goes to the next workgroup on the CU).
@@ -1167,8 +1244,10 @@ struct Shape {
   static constexpr int BM = WGM * TM * 16;
   static constexpr int BN = WGN * TN * 16;
   static constexpr size_t kLdsBytes =
-      (PIPE == 5 ? kStages5 : PIPE == 0 || PIPE == 4 ? 2 : 3) *
-      (size_t)(PIPE == 2 || PIPE == 3 ? BM : BM + BN) * KS;
+      (PIPE == 5 && ElemTraits<E>::kHalves == 2)
+          ? 5 * (size_t)(BM + BN) * 64   // five slots of half a step
+          : (PIPE == 5 ? kStages5 : PIPE == 0 || PIPE == 4 ? 2 : 3) *
+                (size_t)(PIPE == 2 || PIPE == 3 ? BM : BM + BN) * KS;
 };
 
 }  // namespace uk_mfma

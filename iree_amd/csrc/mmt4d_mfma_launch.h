@@ -50,6 +50,7 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
                    hipStream_t stream) {
   using SH = Shape<E, TM, TN, WGM, WGN, NKK, PIPE>;
   constexpr int R = RBC >= 16 ? 1 : 16 / RBC;
+  if (SH::kLdsBytes > 160 * 1024) return -1;          // more LDS than a compute unit has
   if (p.rb > SH::KS) return -1;                       // a tile row must fit one step
   if (p.M0 > SH::BM || p.N0 > SH::BN) return -1;      // at least one whole panel
   if (p.M0 % R || p.N0 % R) return -1;                // pieces hold whole rows
@@ -440,6 +441,8 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     choice = 2;  // the narrow-row kernel in the 128x128 shape
   } else if (forced == 16 || forced == 17) {
     choice = 1;  // the LDS-direct ping-pong pipeline in the 256x256 (16) or 128x512 (17) shape
+  } else if (forced == 20) {
+    choice = 7;  // the same pipeline in the 256x128 shape
   } else if (forced == 18) {
     choice = 2;  // the same pipeline in the 128x128 shape
   } else if (forced == 19) {
@@ -641,12 +644,13 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
         }
         if (st > 0) return st;
       }
-      if constexpr (RBC >= 16 && H == 1) {
+      if constexpr (RBC >= 16) {
         // Both operands through LDS-direct loads, two wave groups alternating
         // between memory and compute phases (PIPE 5 of mmt4d_mfma_kernel.h): the
         // default for the big problems of the 8- and 16-bit types (s8 8192^3
-        // 413 -> 388 us, bf16 8192^3 779 -> 718 us, f16 4096^3 102 -> 98 us
-        // against the register-direct-RHS pipeline in its best shape). f32
+        // 413 -> 388 us, bf16 8192^3 779 -> 718 us, f16 4096^3 102 -> 98 us, f8
+        // 8192^3 415 -> 390 us against the register-direct-RHS pipeline in its
+        // best shape). f32
         // keeps that pipeline (matrix-pipe bound there: 925 against 959 us).
         constexpr bool kDefault = E != Elem::kF32;
         if (forced == 17) {
@@ -695,6 +699,15 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     // 256x256 blocks to fill the CUs; moves fewer L1 bytes per MFMA than the
     // 128x128 shape.
     if constexpr (RBC >= 16) {
+      if (kt_main > 0 && (forced == 20 || (forced == 0 && E != Elem::kF32))) {
+        int st = launch_variant<E, RBC, 8, 2, 2, 4, 1, 5>(p, 0, kt_main, p.accumulate, stream);
+        if (st == 0) {
+          *name = "mmt4d_mfma_256x128_lds_direct";
+          if (kt_main == p.K1) return 0;
+          return finish_k(launch_variant<E, RBC, 4, 4, 2, 2, NKK2, 0>(p, kt_main, p.K1 - kt_main, true, stream));
+        }
+        if (st > 0) return st;
+      }
       if (kt_main > 0) {
         int st = launch_variant<E, RBC, 8, 2, 2, 4, 1, 3>(p, 0, kt_main, p.accumulate, stream);
         if (st == 0) {

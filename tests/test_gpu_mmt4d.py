@@ -90,8 +90,8 @@ def _mfma_shapes(M0, N0, K0, bits):
 # 128x512 shape; 11 is the 64x64 shape with the deep pipeline, 12 .. 15 are
 # the narrow-row kernels in the 256x256 / 128x512 / 128x128 / 64x64 shape, which
 # serve tile rows of 2 or 4 bytes with N0 = 16 and hand everything else on, and
-# 16 .. 19 the LDS-direct ping-pong pipeline in the 256x256 / 128x512 / 128x128 /
-# 64x64 shape).
+# 16 .. 20 the LDS-direct ping-pong pipeline in the 256x256 / 128x512 / 128x128 /
+# 64x64 / 256x128 shape).
 # Tile rows of one byte (s8, K0 = 1) have no MFMA kernel: iree_uk_mmt4d_info
 # says so and the reference grid above covers them on the scalar kernel. The
 # entry stays in the list, named for what it is, and is asserted unserved.
@@ -105,23 +105,25 @@ def _variant_applies(n, variant):
     """Forced shapes that a tile cannot take hand the call on to the choice by
     size, i.e. repeat variant 0: the deep 64x64 pipeline (11) exists for tile
     rows under 16 bytes, the narrow-row kernels (12 .. 15) for rows of 2 or 4
-    bytes with N0 = 16, the LDS-direct pipeline (16 .. 19) for every type but the
-    8-bit floats."""
+    bytes with N0 = 16, the LDS-direct pipeline (16 .. 20): its small shapes (18,
+    19) not for the 8-bit floats, its 256x128 shape (20) for rows of 16 bytes and more."""
     tf, M0, N0, K0 = MFMA_TILES[n]
     row_bytes = K0 * uk.MMT4D_TYPE_BITS[tf][0] // 8
     if variant == 11:
         return row_bytes < 16
     if variant in (12, 13, 14, 15):
         return row_bytes in (2, 4) and N0 == 16
-    if variant in (16, 17, 18, 19):
-        # the LDS-direct pipeline: one 16-byte piece per lane operand (not the 8-bit floats)
+    if variant in (18, 19):
+        # the LDS-direct pipeline in its small shapes: one 16-byte piece per lane operand (not the 8-bit floats)
         return tf != uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32
+    if variant == 20:
+        return row_bytes >= 16
     return True
 
 
 _TILE_VARIANTS = [pytest.param(n, v, id=f"{_tile_id(n)}-{v}")
                   for n in range(len(MFMA_TILES))
-                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15, 16, 17, 18, 19) if _variant_applies(n, v)]
+                  for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20) if _variant_applies(n, v)]
 
 
 @pytest.mark.parametrize("n,variant", _TILE_VARIANTS)

@@ -162,17 +162,18 @@ def test_mmt4d_random_sweep_larger_shapes_and_forced_variants(gpu, oracle):
 
 
 def test_mmt4d_random_sweep_lds_direct_pipeline(gpu, oracle):
-    """The LDS-direct ping-pong pipeline (forced shapes 16 to 19): tile rows of
+    """The LDS-direct ping-pong pipeline (forced shapes 16 to 20): tile rows of
     2 to 64 bytes, random tiles incl. heights that straddle the 16-row MFMA
     blocks, tile counts ragged against the workgroup blocks, K with and
     without a remainder against the 64- or 256-byte step, loose strides, ACCUMULATE."""
     lib, torch = gpu
     rng = np.random.default_rng(2031)
     types = [uk.MMT4D_TYPE_S8S8S32, uk.MMT4D_TYPE_F16F16F32, uk.MMT4D_TYPE_BF16BF16F32,
-             uk.MMT4D_TYPE_F32F32F32, uk.MMT4D_TYPE_F16F16F16 | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS]
+             uk.MMT4D_TYPE_F32F32F32, uk.MMT4D_TYPE_F16F16F16 | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS,
+             uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32]
     names = set()
     done = 0
-    for ci in range(240):
+    for ci in range(300):
         tf = types[ci % len(types)]
         eb = uk.MMT4D_TYPE_BITS[tf & 0xFF][0] // 8
         M0, N0 = int(rng.choice([4, 8, 12, 16, 24, 32, 48, 64])), int(rng.choice([4, 8, 16, 20, 32, 64]))
@@ -187,7 +188,7 @@ def test_mmt4d_random_sweep_lds_direct_pipeline(gpu, oracle):
         lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
         want = out0.copy()
         G.run_mmt4d_case(oracle, c, lhs, rhs, want)
-        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + 16 + ci % 4)
+        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + 16 + (ci // len(types)) % 5)
         got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
         assert np.array_equal(got, want), (ci, c, lib.last_kernel_name())
         names.add(lib.last_kernel_name())
@@ -195,7 +196,8 @@ def test_mmt4d_random_sweep_lds_direct_pipeline(gpu, oracle):
     lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
     assert done >= 100, done
     assert {"mmt4d_mfma_256x256_lds_direct", "mmt4d_mfma_128x512_lds_direct",
-            "mmt4d_mfma_128x128_lds_direct", "mmt4d_mfma_64x64_lds_direct"} <= names, names
+            "mmt4d_mfma_128x128_lds_direct", "mmt4d_mfma_64x64_lds_direct",
+            "mmt4d_mfma_256x128_lds_direct"} <= names, names
 
 
 def test_mmt4d_random_sweep_thin_kernels(gpu, oracle):
