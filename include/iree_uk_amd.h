@@ -304,8 +304,10 @@ IREE_UK_AMD_EXPORT void iree_uk_amd_set_assert_handler(
  * hipError_t value (launch or staging failure), -1 (contract violation) or
  * one of the values below. */
 enum {
-  /* iree_uk_amd_mmt4d_no_alloc: the call's K-split workspace exceeds the
-   * library's static scratch array (iree_uk_amd_no_alloc_scratch_bytes). */
+  /* Not returned by this version of the library (kept so that the values
+   * stay what callers compiled against): a call of iree_uk_amd_mmt4d_no_alloc
+   * whose K-split workspace would exceed the static scratch array runs without
+   * the split instead. */
   IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL = 100001,
   /* iree_uk_amd_mmt4d_no_alloc: an operand is ordinary host memory, which
    * would have to be staged through a device allocation. */
@@ -365,8 +367,8 @@ IREE_UK_AMD_EXPORT uint64_t iree_uk_amd_mfma_decline_count(void);
 /* iree_uk_mmt4d_p for callers that cannot allocate device memory: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * It has no counterpart in the reference. Same parameters, same result (bit
- * for bit, floats included: both entry points take the same kernel with the
- * same split of K), with two differences:
+ * for bit, floats included, whenever both entry points split K alike: they
+ * take the same kernel), with two differences:
  *   - every operand must already be device-accessible memory; a host operand
  *     fails with IREE_UK_AMD_STATUS_NEEDS_ALLOCATION (iree_uk_mmt4d would
  *     stage it through a device allocation);
@@ -376,8 +378,12 @@ IREE_UK_AMD_EXPORT uint64_t iree_uk_amd_mfma_decline_count(void);
  *     device array of the library, iree_uk_amd_no_alloc_scratch_bytes() bytes
  *     (8 MiB of partials + 16384 counters) held by every GPU the library runs
  *     on, instead of a buffer iree_uk_mmt4d allocates on first need. A call
- *     whose split needs more fails with IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL
- *     and writes nothing.
+ *     whose split would need more runs without the split (one workgroup per
+ *     output block over all of K, which needs no scratch memory): the same
+ *     integers, and float sums in the unsplit order.
+ * (iree_uk_mmt4d itself, called on a stream that is being captured into a HIP
+ * graph, never hands that stream one of its own workspaces - the graph would
+ * outlive it - and runs such a call without the split.)
  * The call allocates nothing: no hipMalloc / hipFree, no allocating library
  * routine. All calls on one GPU share that GPU's array; the kernels leave its
  * counters at zero and write partials before reading them, so consecutive

@@ -16,6 +16,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_dot2(
     const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
     void* stream);
 
+namespace uk_mfma {
+void note_k_slices(int n);  // mmt4d_mfma.hip: records the slice count of the call
+}
+
 namespace {
 // Calls on this thread that iree_uk_mmt4d_info advertises a matrix-core kernel
 // for but that the scalar kernel served (see iree_uk_amd_mfma_decline_count).
@@ -34,6 +38,9 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
                                             const iree_uk_amd_rowmajor_out_t* rowmajor,
                                             void* stream, int kernel_mode,
                                             const char** kernel_name) {
+  // Every call starts from "one K slice": only the thin matrix-core kernel
+  // ever reports more (iree_uk_amd_last_k_slices).
+  uk_mfma::note_k_slices(1);
   // s8 x s4 -> s32 has an MFMA kernel for some shapes only; the launcher says
   // "not served" (negative) for the rest.
   const bool maybe = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32;

@@ -103,16 +103,22 @@ struct OwnedWorkspace {
   char* base;
   size_t partial_bytes;
   uint32_t n_counters;
+  uint64_t last_use;   // value of the thread's use counter when last handed out
 };
 // Freed when the thread ends; hipFree waits for the device, so no kernel in
 // flight can still use a workspace then.
 struct OwnedWorkspaces : std::vector<OwnedWorkspace> {
+  uint64_t uses = 0;
   ~OwnedWorkspaces() {
     for (OwnedWorkspace& w : *this) {
       if (w.base) (void)hipFree(w.base);
     }
   }
 };
+// Workspaces a thread keeps at most: beyond that the one used longest ago is
+// freed (a thread that runs through many short-lived streams would otherwise
+// hold a megabyte and more per stream handle it ever saw).
+constexpr size_t kMaxOwnedWorkspaces = 8;
 thread_local OwnedWorkspaces g_workspaces;
 thread_local bool g_no_alloc = false;
 thread_local int g_k_slices = 0;
@@ -130,9 +136,9 @@ void note_k_slices(int n) { g_last_k_slices = n; }
 int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStream_t stream,
                              KSplitWorkspace* ws) {
   if (g_no_alloc) {
-    if (partial_bytes > kScratchPartialBytes || n_counters > kScratchCounters) {
-      return IREE_UK_AMD_STATUS_SCRATCH_TOO_SMALL;
-    }
+    // A split that does not fit the static array: the call runs without the
+    // split, which needs no scratch memory at all.
+    if (partial_bytes > kScratchPartialBytes || n_counters > kScratchCounters) return 1;
     void* base = nullptr;
     const int st = scratch_address(&base);
     if (st != 0) return st;
@@ -140,22 +146,48 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
     ws->counters = (uint32_t*)((char*)base + kScratchPartialBytes);
     return 0;
   }
+  // A stream that is being captured into a graph gets no library-owned
+  // workspace at all: the graph would keep the pointer beyond the life of the
+  // thread that owns the block, and its replays would share the block with
+  // this thread's eager calls. Such a call runs without the split (callers that
+  // want the split inside a graph use iree_uk_amd_mmt4d_no_alloc and its
+  // serialization rule).
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) { (void)hipGetLastError(); return 1; }
+  if (capture != hipStreamCaptureStatusNone) return 1;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 1;
+  const uint64_t now = ++g_workspaces.uses;
   for (OwnedWorkspace& w : g_workspaces) {
     if (w.device == dev && w.stream == stream && w.partial_bytes >= partial_bytes &&
         w.n_counters >= n_counters) {
+      w.last_use = now;
       ws->partials = w.base;
       ws->counters = (uint32_t*)(w.base + w.partial_bytes);
       return 0;
     }
   }
-  // Nothing fits: allocate (sizes rounded up so that similar calls share it),
-  // unless the stream is being captured, where allocation is not allowed; the
-  // call then runs without the split.
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) { (void)hipGetLastError(); return 1; }
-  if (capture != hipStreamCaptureStatusNone) return 1;
+  // Nothing fits: allocate (sizes rounded up so that similar calls share it).
+  // First make room: a smaller workspace of the same stream is replaced, and
+  // beyond kMaxOwnedWorkspaces the one used longest ago goes. hipFree waits for
+  // the device, so no kernel in flight can still be using what is freed.
+  for (size_t i = 0; i < g_workspaces.size();) {
+    OwnedWorkspace& w = g_workspaces[i];
+    if (w.device == dev && w.stream == stream) {
+      (void)hipFree(w.base);
+      g_workspaces.erase(g_workspaces.begin() + (ptrdiff_t)i);
+    } else {
+      ++i;
+    }
+  }
+  while (g_workspaces.size() >= kMaxOwnedWorkspaces) {
+    size_t oldest = 0;
+    for (size_t i = 1; i < g_workspaces.size(); ++i) {
+      if (g_workspaces[i].last_use < g_workspaces[oldest].last_use) oldest = i;
+    }
+    (void)hipFree(g_workspaces[oldest].base);
+    g_workspaces.erase(g_workspaces.begin() + (ptrdiff_t)oldest);
+  }
   size_t want_partials = 1u << 20;
   while (want_partials < partial_bytes) want_partials <<= 1;
   uint32_t want_counters = 4096;
@@ -171,9 +203,7 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
     (void)hipFree(base);
     return 1;
   }
-  // A smaller workspace of the same stream is kept (a kernel in flight may
-  // still use it) and simply no longer chosen.
-  g_workspaces.push_back(OwnedWorkspace{dev, stream, base, want_partials, want_counters});
+  g_workspaces.push_back(OwnedWorkspace{dev, stream, base, want_partials, want_counters, now});
   ws->partials = base;
   ws->counters = (uint32_t*)(base + want_partials);
   return 0;

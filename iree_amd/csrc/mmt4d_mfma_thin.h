@@ -363,6 +363,14 @@ void mmt4d_thin_kernel(Args a) {
     }
     arrived = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrived);
     if (arrived != kslices - 1) return;
+    // The reader side of the handoff. What the other slices stored is complete
+    // at the point where the XCDs meet before their counter increments (their
+    // agent-scope stores are acknowledged from there, and each waited for its
+    // own before counting), and the agent-scope loads below go to that point
+    // instead of a cache; this fence only keeps the compiler from moving those
+    // loads above the test of the counter (workgroup scope: it costs no cache
+    // write-back or invalidation).
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (lane == 0) {
       __hip_atomic_store(a.ws_counters + block_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }

@@ -28,7 +28,7 @@ constexpr int kTM = 8, kTN = 4, kWaves = 8;
 
 template <Elem E>
 __global__ __launch_bounds__(kWaves * 64) void mfma_peak_kernel(const v4i* operands, int n_operands,
-                                                               int iters, int* sink) {
+                                                               int iters, int* sink, int sink_enable) {
   using TT = ElemTraits<E>;
   using Acc = typename TT::Acc;
   constexpr int H = TT::kHalves;
@@ -54,7 +54,10 @@ __global__ __launch_bounds__(kWaves * 64) void mfma_peak_kernel(const v4i* opera
 #pragma unroll
       for (int j = 0; j < kTN; ++j) acc[i][j] = TT::mfma(fb[j], fa[i], acc[i][j]);
   }
-  // Keep the accumulators alive without writing anything in practice.
+  // Keep the accumulators alive without writing anything in practice: the
+  // store depends on a kernel argument that the host always passes as zero,
+  // which the compiler cannot know (nothing about `iters` or the data lets it
+  // drop the loop).
   Acc s = acc[0][0];
 #pragma unroll
   for (int i = 0; i < kTM; ++i)
@@ -62,7 +65,7 @@ __global__ __launch_bounds__(kWaves * 64) void mfma_peak_kernel(const v4i* opera
     for (int j = 0; j < kTN; ++j)
       if (i || j) s = s + acc[i][j];
   const v4i bits = __builtin_bit_cast(v4i, s);
-  if ((bits[0] ^ bits[1] ^ bits[2] ^ bits[3]) == 0x5a17c0de && iters < 0) sink[t] = bits[0];
+  if (sink_enable) sink[t] = bits[0] ^ bits[1] ^ bits[2] ^ bits[3];
 }
 
 // K elements per MFMA instruction group issued by ElemTraits<E>::mfma.
@@ -74,7 +77,7 @@ template <Elem E>
 int run_mfma_peak(const v4i* operands, int n_operands, int iters, int workgroups, int* sink,
                   hipStream_t stream, double* ops) {
   hipLaunchKernelGGL(mfma_peak_kernel<E>, dim3(workgroups), dim3(kWaves * 64), 0, stream, operands,
-                     n_operands, iters, sink);
+                     n_operands, iters, sink, /*sink_enable=*/0);
   *ops = 2.0 * 16 * 16 * k_per_mfma<E>() * kTM * kTN * (double)iters * kWaves * workgroups;
   return (int)hipGetLastError();
 }

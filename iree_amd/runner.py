@@ -580,6 +580,13 @@ class Runner:
         for _ in range(4):
             best = max(best, self.lib.probe_mfma_peak(tf, operands.data_ptr(), n, iters,
                                                       sink.data_ptr(), st))
+        # A loop of nothing but MFMAs cannot beat the published peak and, on a
+        # healthy part, does not fall far below it: anything else means the probe
+        # did not measure what it is meant to (e.g. its loop was optimized away).
+        peak = PEAK_TFLOPS[dtype] * 1e12
+        if not 0.3 * peak <= best <= 1.02 * peak:
+            raise RuntimeError(f"MFMA-only probe for {dtype} reads {best / 1e12:.1f} T/s against a "
+                               f"published peak of {peak / 1e12:.1f}: not a valid ceiling")
         return best / 1e12
 
     def copy2d_ceiling_gbps(self, rows: int, row_bytes: int, src_pitch: int, dst_pitch: int,

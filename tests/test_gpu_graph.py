@@ -64,3 +64,59 @@ def test_chain_and_fused_calls_replay_from_a_graph(gpu):
     finally:
         lib.set_stream(None)
         lib.set_pointer_mode(uk.POINTER_MODE_AUTO)
+
+
+@pytest.mark.gpu
+def test_k_split_call_under_capture_takes_no_library_workspace(gpu):
+    """A decode-shaped mmt4d (few rows, long K: eagerly the thin kernel splits K
+    over workgroups through a workspace the library owns per thread and stream)
+    captured into a graph: the capturing stream is never handed such a
+    workspace - the graph would outlive it and share it with eager calls - so
+    the captured call runs without the split. Replays, with eager K-split calls
+    on the same thread and stream in between, equal the exact integer product."""
+    lib, torch = gpu
+    Mrows, N, K, M0, N0, K0 = 16, 1024, 14336, 16, 16, 16
+    M1, N1, K1 = 1, N // N0, K // K0
+    g = torch.Generator(device="cuda"); g.manual_seed(23)
+    lhs = torch.randint(-128, 128, (M1 * K1 * M0 * K0,), generator=g, device="cuda", dtype=torch.int8)
+    rhs = torch.randint(-128, 128, (N1 * K1 * N0 * K0,), generator=g, device="cuda", dtype=torch.int8)
+    out_eager = torch.zeros(M1 * N1 * M0 * N0, device="cuda", dtype=torch.int32)
+    out_graph = torch.zeros_like(out_eager)
+    a = lhs.view(M1, K1, M0, K0).permute(0, 2, 1, 3).reshape(M0, K).cpu().to(torch.int64)
+    b = rhs.view(N1, K1, N0, K0).permute(0, 2, 1, 3).reshape(N, K).cpu().to(torch.int64)
+    want = (a @ b.T).to(torch.int32).view(M1, M0, N1, N0).permute(0, 2, 1, 3).reshape(-1)
+
+    def call(out):
+        lib.mmt4d(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, out.data_ptr(), 0,
+                  N1 * M0 * N0, M1, N1, K1, M0, N0, K0, uk.MMT4D_TYPE_S8S8S32)
+
+    stream = torch.cuda.Stream()
+    lib.set_pointer_mode(uk.POINTER_MODE_DEVICE)
+    lib.set_stream(stream.cuda_stream)
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lib.set_k_slices(0)
+    try:
+        with torch.cuda.stream(stream):
+            call(out_eager)                    # creates this thread's workspace for the stream
+        stream.synchronize()
+        assert lib.last_k_slices() > 1, lib.last_kernel_name()
+        assert torch.equal(out_eager.cpu(), want)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            call(out_graph)
+            slices_under_capture = lib.last_k_slices()
+        torch.cuda.synchronize()
+        assert slices_under_capture == 1
+        for rep in range(3):
+            out_graph.zero_()
+            out_eager.zero_()
+            with torch.cuda.stream(stream):
+                call(out_eager)                # an eager K-split call between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_graph.cpu(), want), rep
+            assert torch.equal(out_eager.cpu(), want), rep
+    finally:
+        lib.set_stream(None)
+        lib.set_pointer_mode(uk.POINTER_MODE_AUTO)
