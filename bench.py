@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
                     [--no-extra] [--no-cpu]
+    python bench.py --sweep WORKLOAD     (T(K) table of a square mmt4d workload)
 
 A step is one pass of the workload's whole chain over one batch of seeded
 synthetic tensors that are already resident in HBM. The default workload is
@@ -32,7 +33,8 @@ EXTRA_WORKLOADS = [
     "s8_mmt4d_8192_k2", "s8_mmt4d_8192_k16", "s8_mmt4d_8192_k16_zeros", "s8_mmt4d_8192_k64",
     "s8_mmt4d_1024_k2",
     "c2_f16_chain_ragged", "c2_f16_fused_4096", "c2_f16_fused_ragged", "c3_s8_decode",
-    "c3_s8_decode_fused", "c3_s8_decode_down", "c4_f8_prefill",
+    "c3_s8_decode_fused", "c3_s8_decode_down", "c3_s8_decode_cold", "c3_s8_decode_fused_cold",
+    "c4_f8_prefill",
     "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "f32_mmt4d_4096_k1",
     "f32_mmt4d_4096_k4", "s16_mmt4d_4096_k2",
     "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288",
@@ -358,6 +360,9 @@ def main() -> int:
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--extra-iters", type=int, default=20)
+    ap.add_argument("--sweep", metavar="WORKLOAD", default=None,
+                    help="print T(K) of a square mmt4d workload (e.g. s8_mmt4d_8192_k16) under the "
+                         "big kernel variants, with a straight-line fit, instead of the JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards by tile rows with no "
@@ -370,6 +375,11 @@ def main() -> int:
 
     torch.cuda.set_device(0)
     R = rn.Runner(seed=0)
+    if args.sweep:
+        print("command: python bench.py --sweep " + args.sweep)
+        print(R.k_sweep(args.sweep))
+        R.close()
+        return 0
     wl = R.workload(args.workload)
     dominant = "mmt4d" if any(o.name == "mmt4d" for o in wl.ops) else wl.ops[0].name
     sec_per_step, sec_per_step_events, dom_us = R.run_steps(wl, args.steps, args.warmup, dominant)
@@ -413,6 +423,10 @@ def main() -> int:
     peaks = {dt: round(R.measured_mfma_peak(dt), 1) for dt in ("s8", "f8", "f16", "bf16", "f32")}
     peaks["s8_zero_operands"] = round(R.measured_mfma_peak("s8", zeros=True), 1)
     result["measured_mfma_only_TOPS"] = peaks
+    # The shader clock those rates imply: rate / (1024 SIMDs x operations per SIMD
+    # and clock), the published peak being that product at 2.4 GHz.
+    result["measured_mfma_only_clock_GHz"] = {
+        dt: round(2.4 * v / rn.PEAK_TFLOPS["s8" if dt.startswith("s8") else dt], 3) for dt, v in peaks.items()}
     if roof["bound"] == "mfma" and wl.dtype in peaks and peaks[wl.dtype] > 0:
         # the same kernel against the ceiling measured in this run
         roof["of_measured_mfma_only"] = round(roof["achieved"] / peaks[wl.dtype], 4)
@@ -483,9 +497,15 @@ def main() -> int:
                 continue
             kk = e["kernels"]["mmt4d"]
             dt = name.split("_")[0] if not name.startswith("c4") else "f8"
+            traffic, traffic_source = recorded_traffic(name, "mmt4d", kk["kernel"])
             t = {"kernel": kk["kernel"].replace("mmt4d_mfma_", ""), "us": kk["avg_us"],
                  "TOPS": round(kk["achieved"], 1), "frac": round(kk["frac"], 3),
-                 "of_mfma_only": round(kk["achieved"] / peaks[dt], 3)}
+                 "of_mfma_only": round(kk["achieved"] / peaks[dt], 3),
+                 # the same object as the headline's `roofline`, for this workload's mmt4d kernel
+                 "roofline": {"bound": kk["bound"], "achieved": kk["achieved"],
+                              "peak": rn.PEAK_TFLOPS[dt], "unit": kk["unit"], "frac": kk["frac"],
+                              "traffic": traffic, "traffic_source": traffic_source,
+                              "of_measured_mfma_only": round(kk["achieved"] / peaks[dt], 4)}}
             if "parity" in e:
                 par = e["parity"]
                 t["parity"] = ("bit-exact on %d sampled tiles" % par["tiles"] if par.get("bit_exact")
@@ -501,6 +521,34 @@ def main() -> int:
             if "copy2d_ceiling" in e:
                 t["copy2d_frac"] = round(e["copy2d_ceiling"]["frac"], 3)
             targets[name] = t
+        # The decode layer (HBM-bound: its weights stream once per launch). `warm`:
+        # the benchmark's repeated launches find the 58.7 MB of weights in the 256 MB
+        # memory-side cache; `cold`: launches rotate over eight copies of the weights,
+        # so every launch streams them from HBM - the figure a serving loop sees.
+        for name, label in (("c3_s8_decode", "warm"), ("c3_s8_decode_cold", "cold"),
+                            ("c3_s8_decode_fused", "warm"), ("c3_s8_decode_fused_cold", "cold"),
+                            ("c3_s8_decode_down", "warm")):
+            e = extra.get(name)
+            if not e:
+                continue
+            kk = e["kernels"]["mmt4d"]
+            traffic, traffic_source = recorded_traffic(name, "mmt4d", kk["kernel"])
+            targets[name] = {"kernel": kk["kernel"].replace("mmt4d_mfma_", ""), "weights": label,
+                             "us": kk["avg_us"], "GBps": round(kk["achieved"], 1),
+                             "frac": round(kk["frac"], 3),
+                             "roofline": {"bound": "hbm", "achieved": kk["achieved"],
+                                          "peak": rn.PEAK_HBM_GBPS, "unit": "GB/s", "frac": kk["frac"],
+                                          "traffic": traffic, "traffic_source": traffic_source}}
+        e = extra.get("s16_mmt4d_4096_k2")
+        if e:
+            kk = e["kernels"]["mmt4d"]
+            targets["s16_mmt4d_4096_k2"] = {
+                "kernel": kk["kernel"], "us": kk["avg_us"], "TOPS": round(kk["achieved"], 1),
+                "frac": round(kk["frac"], 3),
+                "roofline": {"bound": "vdot2", "achieved": kk["achieved"], "peak": rn.PEAK_TFLOPS["s16"],
+                             "unit": kk["unit"], "frac": kk["frac"], "traffic": None,
+                             "what": "no 16-bit integer matrix instruction: the peak is that of "
+                                     "v_dot2_i32_i16 on the vector ALUs"}}
         for name in TARGET_PACK:
             e = extra.get(name)
             if not e or "pack" not in e["kernels"]:
