@@ -818,11 +818,15 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     if (st >= 0) { *name = "mmt4d_mfma_128x128"; return st; }
   }
   if constexpr (H == 1) {
-    // 64x64 blocks, 8 waves of 32x16, 256 bytes of K per step (forced only).
+    // 64x64 blocks, 8 waves of 32x16, 256 bytes of K per step.
     const int kts256 = 256 >> p.lrb;
     int kt_main256 = kts256 > 0 ? (p.K1 / kts256) * kts256 : 0;
     if (kOneLaunchOnly && kt_main256 != p.K1) kt_main256 = 0;
-    if (kt_main256 > 0 && forced == 19) {
+    // Chosen for narrow tile rows when the 64x64 blocks fill the compute units
+    // (s8 1024^3 16x16x2: 7.0 -> 6.4 us; with rows of 16 bytes and more the
+    // register-direct kernel below is level or ahead: 5.7 against 5.9 us).
+    const bool small_narrow = forced == 0 && RBC < 16 && E != Elem::kF32 && workgroups(p, 64, 64) >= 192;
+    if (kt_main256 > 0 && (forced == 19 || small_narrow)) {
       int st = launch_variant<E, RBC, 2, 1, 2, 4, 4, 5>(p, 0, kt_main256, p.accumulate, stream);
       if (st == 0) {
         *name = "mmt4d_mfma_64x64_lds_direct";

@@ -1202,6 +1202,88 @@ bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
   return false;
 }
 
+//===----------------------------------------------------------------------===//
+// Direct pack: untransposed tiles whose rows are whole 16-byte pieces, matrix
+// tiled exactly (no padding). A 16-byte piece of a matrix row is a 16-byte
+// piece of a tile row, so the data needs no regrouping in LDS: every thread
+// moves kDirectPieces pieces from register to register. A workgroup takes 16
+// matrix rows x 1 KiB: a wave reads 256 contiguous bytes of each of 4 rows and
+// writes, per tile, 4 x (tile row bytes) contiguous bytes; the four waves
+// together fill whole tiles when the tile height divides 16. No LDS round
+// trip, no barrier: for problems of a few tens of megabytes, which are bound by
+// the latency of one pass (launch, one load, one store) rather than by HBM.
+//===----------------------------------------------------------------------===//
+struct DirectArgs {
+  const char* src;
+  char* dst;
+  int64_t src_pitch;     // bytes between matrix rows
+  int64_t dst_stride0;   // bytes between rows of tiles
+  uint32_t rows, row_bytes;
+  uint32_t tile_rows, tile_row_bytes, log2_tile_row_bytes;
+  uint32_t col_groups;   // 1 KiB column groups per matrix row
+};
+constexpr int kDirectPieces = 4;
+
+__global__ __launch_bounds__(kThreads) void pack_direct_kernel(DirectArgs a) {
+  const uint32_t rg = blockIdx.x / a.col_groups, cg = blockIdx.x - rg * a.col_groups;
+  const uint32_t lane16 = threadIdx.x & 15;            // 16-byte piece within a 256-byte segment
+  const uint32_t row = rg * 16 + (threadIdx.x >> 4);
+  if (row >= a.rows) return;
+  const uint32_t o0 = row / a.tile_rows, m0 = row - o0 * a.tile_rows;
+  const char* srow = a.src + (int64_t)row * a.src_pitch;
+  char* drow = a.dst + (int64_t)o0 * a.dst_stride0 + (int64_t)m0 * a.tile_row_bytes;
+  const uint32_t tile_bytes = a.tile_rows * a.tile_row_bytes;
+  v4u v[kDirectPieces];
+  uint32_t col[kDirectPieces];
+#pragma unroll
+  for (int i = 0; i < kDirectPieces; ++i) {
+    col[i] = cg * 1024 + (uint32_t)i * 256 + lane16 * 16;
+    if (col[i] < a.row_bytes) v[i] = gload<16>(srow + col[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < kDirectPieces; ++i) {
+    if (col[i] < a.row_bytes) {
+      const uint32_t o1 = col[i] >> a.log2_tile_row_bytes;
+      gstore<16>(drow + (int64_t)o1 * tile_bytes + (col[i] & (a.tile_row_bytes - 1)), v[i]);
+    }
+  }
+}
+
+// Launches the direct pack when the call is of that form (see above) and
+// small enough to be latency-bound; false otherwise.
+bool launch_pack_direct(const iree_uk_pack_params_t* p, int es, const char* src, char* dst,
+                        bool transposed, hipStream_t stream) {
+  if (transposed || p->in_stride1 != 1) return false;
+  const int64_t trb = p->out_size3 * es;   // tile row bytes
+  if (trb < 16 || trb > 4096 || (trb & (trb - 1))) return false;
+  if (p->in_size0 != p->out_size0 * p->out_size2 || p->in_size1 != p->out_size1 * p->out_size3) return false;
+  if (p->in_size0 <= 0 || p->in_size1 <= 0) return false;
+  const int64_t row_bytes = p->in_size1 * es, pitch = p->in_stride0 * es;
+  if (pitch < 0 || ((uintptr_t)src | (uintptr_t)dst | (uint64_t)pitch | (uint64_t)(p->out_stride0 * es)) & 15) return false;
+  // Above a few tens of megabytes the streaming kernels (loads two blocks ahead,
+  // larger blocks) are level or ahead (f16 4096 x 4096, 33.5 MB: 11.9 against
+  // 11.6 us); below, one pass of latency is what counts (s8 2048 x 8192 in
+  // 16x32 tiles, 16.8 MB: 8.4 -> 5.7 us).
+  const int64_t total = p->in_size0 * row_bytes;
+  if (total > (24ll << 20) || p->in_size0 >= (1ll << 31) || row_bytes >= (1ll << 31) ||
+      p->out_size2 >= (1 << 20)) {
+    return false;
+  }
+  DirectArgs a;
+  a.src = src; a.dst = dst;
+  a.src_pitch = pitch;
+  a.dst_stride0 = p->out_stride0 * es;
+  a.rows = (uint32_t)p->in_size0; a.row_bytes = (uint32_t)row_bytes;
+  a.tile_rows = (uint32_t)p->out_size2; a.tile_row_bytes = (uint32_t)trb;
+  a.log2_tile_row_bytes = 0;
+  while ((1u << a.log2_tile_row_bytes) < a.tile_row_bytes) ++a.log2_tile_row_bytes;
+  a.col_groups = (uint32_t)((row_bytes + 1023) / 1024);
+  const int64_t grid = ((p->in_size0 + 15) / 16) * a.col_groups;
+  if (grid >= (1ll << 31)) return false;
+  uk::launch(0, pack_direct_kernel, dim3((uint32_t)grid), dim3(kThreads), 0, stream, a);
+  return true;
+}
+
 uint32_t replicate_pad(uint64_t pad, int es) {
   if (es == 1) return (uint32_t)(pad & 0xFF) * 0x01010101u;
   if (es == 2) return (uint32_t)(pad & 0xFFFF) * 0x00010001u;
@@ -1234,6 +1316,13 @@ extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
   const char* src = (const char*)p->in_buffer + p->in_offset * es;
   char* dst = (char*)p->out_buffer + p->out_offset * es;
 
+  // (Any forced mmt4d variant mode keeps pack on the LDS-staged kernels, so that
+  // tests and timings can reach both.)
+  if (kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO &&
+      launch_pack_direct(p, es, src, dst, ti || to, stream)) {
+    *kernel_name = "pack_direct";
+    return (int)hipGetLastError();
+  }
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC) {
     TiledPlan plan = plan_tiled(v, es, src, p->in_stride0, p->in_stride1,
                                 p->in_size0, p->in_size1, dst, ti, to, false);

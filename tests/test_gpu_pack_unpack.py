@@ -102,7 +102,7 @@ def test_pack_block_spanning_shapes(gpu, oracle, mode):
         G.run_pack_case(oracle, c, inp, want)
         got = T.gpu_pack(lib, torch, c, inp, out0)
         assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
-        tiled += lib.last_kernel_name() in ("pack_tiled", "pack_stream")
+        tiled += lib.last_kernel_name() in ("pack_tiled", "pack_stream", "pack_direct")
     if mode == uk.KERNEL_MODE_AUTO:
         assert tiled >= 60, tiled  # the LDS-staged kernel is the one under test
     else:
@@ -131,6 +131,40 @@ def test_unpack_block_spanning_shapes(gpu, oracle, mode):
         assert tiled >= 40, tiled
 
 
+@pytest.mark.parametrize("tf,t0,t1", [
+    (uk.PACK_TYPE_I8I8, 16, 16), (uk.PACK_TYPE_I8I8, 16, 32), (uk.PACK_TYPE_I8I8, 32, 64),
+    (uk.PACK_TYPE_I8I8, 1, 128), (uk.PACK_TYPE_F16F16, 16, 16), (uk.PACK_TYPE_BF16BF16, 24, 8),
+    (uk.PACK_TYPE_F32F32, 8, 4), (uk.PACK_TYPE_I32I32, 5, 16)])
+def test_pack_direct_kernel_exact_untransposed_tilings(gpu, oracle, tf, t0, t1):
+    """Untransposed packs of a matrix that the tiles cover exactly, tile rows of
+    whole 16-byte pieces, 16-byte aligned rows: the register-to-register kernel
+    (no LDS staging) serves them up to a few tens of megabytes. Whole output
+    buffers against the oracle, loose pitches and offsets included, and the
+    LDS-staged kernels on the same call give the same bytes."""
+    lib, torch = gpu
+    es = uk.PACK_TYPE_BYTES[tf]
+    align = 16 // es
+    for ci, (o0, o1) in enumerate(((1, 1), (3, 5), (17, 9), (40, 33), (2, 130))):
+        in0, in1 = o0 * t0, o1 * t1
+        c = T.PackCase(tf, in0, in1, o0, o1, t0, t1, in1 + (ci % 3) * align, 1,
+                       o1 * t0 * t1 + (ci % 2) * align, (ci % 2) * align, (ci % 3) * align, 0x1234)
+        rng = np.random.default_rng(7000 + ci)
+        inp, out0 = T.make_pack_buffers(c, rng)
+        want = out0.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+        got = T.gpu_pack(lib, torch, c, inp, out0)
+        assert lib.last_kernel_name() == "pack_direct", (c.label(), lib.last_kernel_name())
+        assert np.array_equal(got, want), c.label()
+        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + 1)   # keeps pack on the LDS-staged kernels
+        try:
+            staged = T.gpu_pack(lib, torch, c, inp, out0)
+            assert lib.last_kernel_name() in ("pack_stream", "pack_tiled"), lib.last_kernel_name()
+        finally:
+            lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+        assert np.array_equal(staged, want), c.label()
+
+
 def test_pack_unpack_round_trip_and_numpy_identity(gpu):
     """Size-independent properties at a size the oracle would be slow on:
     pack == pad+reshape+transpose, unpack(pack(x)) == x."""
@@ -153,7 +187,7 @@ def test_pack_unpack_round_trip_and_numpy_identity(gpu):
         flags = tf | (0x100 if ti else 0) | (0x200 if to else 0)
         lib.pack(d_x.data_ptr(), 0, shape[1], 1, d_p.data_ptr(), 0, o1 * o2 * o3,
                  o2 * o3, shape[0], shape[1], o0, o1, o2, o3, pad_bits, flags)
-        assert lib.last_kernel_name() in ("pack_stream", "pack_tiled")
+        assert lib.last_kernel_name() in ("pack_stream", "pack_tiled", "pack_direct")
         got4 = d_p.cpu().numpy().view(dtype).reshape(want4.shape)
         assert np.array_equal(got4, want4)
         d_y = torch.full((x.size * x.itemsize,), 0x5A, dtype=torch.uint8, device="cuda")
