@@ -41,9 +41,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
   // Every call starts from "one K slice": only the thin matrix-core kernel
   // ever reports more (iree_uk_amd_last_k_slices).
   uk_mfma::note_k_slices(1);
-  // s8 x s4 -> s32 has an MFMA kernel for some shapes only; the launcher says
-  // "not served" (negative) for the rest.
-  const bool maybe = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32;
+  // s8 x s4 -> s32 and s16 x s16 -> s32 have an MFMA kernel for some shapes
+  // only; the launcher says "not served" (negative) for the rest.
+  const uint32_t type = p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK;
+  const bool maybe = type == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32 || type == IREE_UK_FLAG_MMT4D_TYPE_S16S16S32;
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC &&
       (maybe || iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags))) {
     const int forced = kernel_mode >= IREE_UK_AMD_KERNEL_MODE_MFMA_VARIANT

@@ -51,6 +51,7 @@ inline int launch_f8(const Problem& p, int forced, hipStream_t stream, const cha
   return p.rb >= 16 ? launch_f8_rb16(p, forced, stream, name) : -1;
 }
 int launch_s8s4(const Problem& p, hipStream_t stream, const char** name);
+int launch_s16(const Problem& p, int forced, hipStream_t stream, const char** name);
 }  // namespace uk_mfma
 
 #include <mutex>
@@ -257,7 +258,7 @@ bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 
 // 1 when an MFMA kernel serves (type, M0, N0, K0) for every M, N, K: the row
 // width K0*sizeof(elem) is a power of two in [2, 128] bytes (f8: [16, 128]),
-// tiles are at most 128 rows, and for rows narrower than 16 bytes the tile
+// tiles are at most 64 rows, and for rows narrower than 16 bytes the tile
 // height is a multiple of the 16/RB rows that share a 16-byte piece.
 extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
                                                     int32_t K0, uint32_t flags) {
@@ -287,6 +288,10 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
   // [16, 64], K in whole 64-element steps): it does not count as "supported"
   // for iree_uk_mmt4d_info, but is tried before the generic kernel.
   const bool s8s4 = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32;
+  // s16 x s16 -> s32 likewise: four 8-bit products per element pair in the
+  // LDS-direct pipeline, for K in whole steps of 64 elements (forced variant 18
+  // is that kernel's 128x128 shape).
+  const bool s16 = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S16S16S32;
   if (s8s4) {
     e = Elem::kS8S4;
     eb = 1;
@@ -294,6 +299,15 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     if (p->K0 != 16 && p->K0 != 32 && p->K0 != 64) return -1;
     if (p->M0 < 1 || p->N0 < 1 || p->M0 > 64 || p->N0 > 64) return -1;
     if (forced_variant != 0 && forced_variant != 4) return -1;
+  } else if (s16) {
+    e = Elem::kS16;
+    eb = 2;
+    ob = 4;
+    const int64_t rb = (int64_t)p->K0 * eb;
+    if (!is_pow2(rb) || rb < 2 || rb > 128) return -1;
+    if (p->M0 < 1 || p->N0 < 1 || p->M0 > 64 || p->N0 > 64) return -1;
+    if (rb < 16 && (p->M0 % (16 / rb) || p->N0 % (16 / rb))) return -1;
+    if (forced_variant != 0 && forced_variant != 18) return -1;
   } else {
     if (!elem_of(p->flags, &e, &eb, &ob)) return -1;
     if (!iree_uk_amd_hip_mmt4d_mfma_supported(p->M0, p->N0, p->K0, p->flags)) return -1;
@@ -362,6 +376,7 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
   pr.accumulate = (p->flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   switch (e) {
     case Elem::kS8S4: return uk_mfma::launch_s8s4(pr, stream, kernel_name);
+    case Elem::kS16: return uk_mfma::launch_s16(pr, forced_variant, stream, kernel_name);
     case Elem::kS8: return uk_mfma::launch_s8(pr, forced_variant, stream, kernel_name);
     case Elem::kF16: return uk_mfma::launch_f16(pr, forced_variant, stream, kernel_name);
     case Elem::kBF16: return uk_mfma::launch_bf16(pr, forced_variant, stream, kernel_name);

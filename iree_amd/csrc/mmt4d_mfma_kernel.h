@@ -79,7 +79,10 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 // kS8S4: s8 x s4 -> s32 (two 4-bit RHS values per byte, low nibble first,
 // runtime/src/iree/builtins/ukernel/mmt4d_tile_generic.c:11-51); served by
 // the thin kernel only (mmt4d_mfma_thin.h).
-enum class Elem { kS8, kF16, kBF16, kF8, kF32, kF16F16, kBF16BF16, kS8S4 };
+// kS16: s16 x s16 -> s32 as four 8-bit integer products per element pair (the
+// hardware has no 16-bit integer matrix instruction); served by the LDS-direct
+// pipeline only (PIPE 5 below, which describes the arithmetic).
+enum class Elem { kS8, kF16, kBF16, kF8, kF32, kF16F16, kBF16BF16, kS8S4, kS16 };
 
 typedef uint16_t v4u16 __attribute__((ext_vector_type(4)));
 
@@ -157,6 +160,19 @@ template <> struct ElemTraits<Elem::kF8> {
     // form with 2^0 block scales computes the same but is a two-part
     // instruction (scale load + MFMA) and issues more slowly.
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+
+// Sixteen 16-bit elements per lane operand (two 16-byte pieces, 128 bytes of K
+// per step as for the 8-bit floats). The pipeline splits them into a register
+// quad of high bytes and one of low bytes and issues the four byte products
+// itself; `mfma` here is the low x low product, which accumulates unscaled.
+template <> struct ElemTraits<Elem::kS16> {
+  using Acc = v4i;
+  using Out = Out32<v4i, int32_t>;
+  static constexpr int kHalves = 2;
+  static __device__ __forceinline__ Acc mfma(const v4i* a, const v4i* b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a[1], b[1], c, 0, 0, 0);
   }
 };
 
@@ -986,7 +1002,7 @@ void mmt4d_mfma_kernel(Args a) {
     // operands, which is all the sum over K needs.
     // A step of NKK x 64 bytes of K holds NKK such blocks per 16 rows, one
     // after the other ([row block][64-byte chunk of K]).
-    static_assert(RBC >= 16 || ((RBC == 2 || RBC == 4 || RBC == 8) && HALVES == 1),
+    static_assert(RBC >= 16 || RBC == 2 || RBC == 4 || RBC == 8,
                   "1 KiB blocks of 16 rows x 64 bytes of K");
     static_assert(NW == 8, "two groups of four waves");
     // Lane operands of two 16-byte pieces (the 8-bit floats: 128 bytes of K per
@@ -1105,6 +1121,83 @@ void mmt4d_mfma_kernel(Args a) {
       __builtin_amdgcn_s_barrier();
       if (group == 1) __builtin_amdgcn_s_barrier();
       v4i fa[TM][HALVES], fb[TN][HALVES];
+      // ---- 16-bit integers -------------------------------------------------
+      // With a = 256 ah + al + 128 (ah the signed high byte, al the low byte
+      // minus 128, both in [-128, 127]) and b likewise,
+      //   sum a b = 65536 sum ah bh + 256 sum (ah bl + al bh) + sum al bl
+      //             + 128 (sum a + sum b) - 16384 K,
+      // all of it modulo 2^32: three accumulator sets fed by four 8-bit integer
+      // MFMAs per block and step (the low x low products go to `acc`, on top of
+      // the caller's accumulators), and the row sums of both operands, which
+      // the vector ALUs add up with v_dot2_i32_i16 against (1, 1) in the memory
+      // phase. A fragment is shared by the waves of a block row (column); each
+      // of them sums one fragment in WGN (WGM) and the sums are exchanged
+      // through LDS once the K loop is done.
+      constexpr bool S16 = E == Elem::kS16;
+      v4i hh[S16 ? TM : 1][S16 ? TN : 1], mid[S16 ? TM : 1][S16 ? TN : 1];
+      int rsa[S16 ? TM : 1], rsb[S16 ? TN : 1];
+      if constexpr (S16) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+          rsa[tm] = 0;
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) hh[tm][tn] = mid[tm][tn] = v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) rsb[tn] = 0;
+      }
+      auto row_sum16 = [&](const v4i (&f)[HALVES], int sum) {
+        typedef short v2s __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            // (a copy first: a bit cast applied to the vector element itself
+            // reads element 0 whatever the index)
+            const int word = f[h][w];
+            sum = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, word), v2s{1, 1}, sum, false);
+          }
+        return sum;
+      };
+      // f[0], f[1] (sixteen elements of one row) -> f[0]: their high bytes,
+      // f[1]: their low bytes minus 128. The order of the sixteen is the same
+      // for both operands, which is all the sum over K needs.
+      auto split16 = [&](v4i (&f)[HALVES]) {
+        v4i hi, lo;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            const uint32_t d0 = (uint32_t)f[h][2 * w], d1 = (uint32_t)f[h][2 * w + 1];
+            hi[2 * h + w] = (int)__builtin_amdgcn_perm(d1, d0, 0x07050301u);
+            lo[2 * h + w] = (int)(__builtin_amdgcn_perm(d1, d0, 0x06040200u) ^ 0x80808080u);
+          }
+        f[0] = hi;
+        f[1] = lo;
+      };
+      auto mfmas16 = [&]() {
+        // Products that share an accumulator are a whole sweep of the blocks apart.
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            hh[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][0], fa[tm][0], hh[tm][tn], 0, 0, 0);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            mid[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][0], fa[tm][1], mid[tm][tn], 0, 0, 0);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            acc[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][1], fa[tm][1], acc[tm][tn], 0, 0, 0);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            mid[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][1], fa[tm][0], mid[tm][tn], 0, 0, 0);
+      };
       auto step_body = [&](int s, auto phase_c) {
         constexpr int P = decltype(phase_c)::value;  // s % 5
 #pragma unroll
@@ -1123,10 +1216,24 @@ void mmt4d_mfma_kernel(Args a) {
           wait_vmem_in_flight<DU>();   // the half-step issued a step ago has landed
         }
         wait_lds_reads();
+        if constexpr (S16) {
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm) {
+            if (tm % WGN == wn) rsa[tm] = row_sum16(fa[tm], rsa[tm]);
+            split16(fa[tm]);
+          }
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) {
+            if (tn % WGM == wm) rsb[tn] = row_sum16(fb[tn], rsb[tn]);
+            split16(fb[tn]);
+          }
+        }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        mfmas(fa, fb);
+        if constexpr (S16) mfmas16();
+        else mfmas(fa, fb);
         __builtin_amdgcn_sched_barrier(0);
         if (group == 0) wait_vmem_in_flight<0>();
         __builtin_amdgcn_s_barrier();
@@ -1144,6 +1251,39 @@ void mmt4d_mfma_kernel(Args a) {
       if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
       if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
       if (s + 3 < a.steps) step_body(s + 3, std::integral_constant<int, 3>{});
+      if constexpr (S16) {
+        // Row sums through LDS (every load has landed and every fragment has
+        // been read once all waves are past the barrier below): per row the
+        // four K-slice partials of the wave that summed that fragment.
+        static_assert(TM % WGN == 0 && TN % WGM == 0, "every fragment is summed by one wave");
+        if (group == 0) __builtin_amdgcn_s_barrier();
+        wait_vmem_in_flight<0>();
+        __syncthreads();
+        int* sums = reinterpret_cast<int*>(lds);   // [BM + BN rows][4 slices]
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          if (tm % WGN == wn) sums[((wm * TM + tm) * 16 + r) * 4 + q] = rsa[tm];
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          if (tn % WGM == wm) sums[(BM + (wn * TN + tn) * 16 + r) * 4 + q] = rsb[tn];
+        __syncthreads();
+        const uint32_t k_term = 16384u * 64u * (uint32_t)a.steps;   // 64 elements of K per step
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+          const v4i pa = *reinterpret_cast<const v4i*>(sums + ((wm * TM + tm) * 16 + r) * 4);
+          const uint32_t sa = (uint32_t)pa[0] + (uint32_t)pa[1] + (uint32_t)pa[2] + (uint32_t)pa[3];
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const v4i pb = *reinterpret_cast<const v4i*>(sums + (BM + (wn * TN + tn) * 16 + 4 * q + e) * 4);
+              const uint32_t sb = (uint32_t)pb[0] + (uint32_t)pb[1] + (uint32_t)pb[2] + (uint32_t)pb[3];
+              acc[tm][tn][e] = (int)((uint32_t)acc[tm][tn][e] + ((uint32_t)hh[tm][tn][e] << 16) +
+                                     ((uint32_t)mid[tm][tn][e] << 8) + 128u * (sa + sb) - k_term);
+            }
+          }
+        }
+      }
     } else {
 #pragma unroll
       for (int s = 0; s < NS - 1; ++s) issue_dma(s * STAGE, min(s, last), 0);
@@ -1188,7 +1328,8 @@ void mmt4d_mfma_kernel(Args a) {
       if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
       if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
     }
-    if (group == 0) __builtin_amdgcn_s_barrier();
+    // (the 16-bit integers have done both already, before their exchange through LDS)
+    if (group == 0 && E != Elem::kS16) __builtin_amdgcn_s_barrier();
     // No LDS-direct load may still be on its way when the workgroup ends (its
     // LDS goes to the next workgroup on the CU).
     wait_vmem_in_flight<0>();

@@ -56,7 +56,7 @@ def test_dequant_unpack_equals_mmt4d_unpack_scale(gpu, oracle, tf, M0, N0, K0, m
     lk, rk, ok = T.MMT4D_KINDS[tf]
     k_whole = max(1, 3 * 128 * 8 // (K0 * uk.MMT4D_TYPE_BITS[tf][0]))  # whole 64/128-byte K steps
     shapes = [(3, 2, 5, 0, 0), (17, 18, 9, 5, 3), (1, 1, 1, 0, 15), (1, 40, 33, 15, 0),
-              (2, 5, k_whole, 3, 2), (21, 1, k_whole, 0, 7)]
+              (2, 5, k_whole, 3, 2), (21, 1, k_whole, 0, 7), (5, 6, k_whole, 3, 2)]
     for si, (M1, N1, K1, cut0, cut1) in enumerate(shapes):
         for acc in (0, 1):
             rows, cols = M1 * M0 - min(cut0, M0 - 1), N1 * N0 - min(cut1, N0 - 1)
