@@ -215,6 +215,22 @@ __device__ __forceinline__ void wait_vmem_in_flight() {
 __device__ __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 // LDS stages of PIPE 5.
 constexpr int kStages5 = 4;
+// Half-step slots of PIPE 5's ring for lane operands of two 16-byte pieces. The
+// 16-bit integers finish a step in half the time of the 8-bit floats (same
+// instruction count, instructions half as long), so the same distance in time
+// between a load's issue and its use takes a ring twice as deep, where it fits.
+template <Elem E, int BM, int BN>
+constexpr int ring_slots() {
+  return (E == Elem::kS16 && 9 * (BM + BN) * 64 <= 160 * 1024) ? 9 : 5;
+}
+// f(integral_constant<int, I>) for I = BEGIN .. END - 1.
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (BEGIN < END) {
+    f(std::integral_constant<int, BEGIN>{});
+    static_for<BEGIN + 1, END>(f);
+  }
+}
 
 struct Args {
   const char* lhs;
@@ -1007,7 +1023,7 @@ void mmt4d_mfma_kernel(Args a) {
     static_assert(NW == 8, "two groups of four waves");
     // Lane operands of two 16-byte pieces (the 8-bit floats: 128 bytes of K per
     // step, i.e. two 64-byte halves) do not leave room for four stages of whole
-    // steps: their LDS is a ring of five half-step slots instead (HALVES == 2
+    // steps: their LDS is a ring of half-step slots instead (HALVES == 2
     // below).
     constexpr int NS = kStages5;
     constexpr int IW = HALVES == 2 ? 4 : NW;          // waves that share one issue of loads
@@ -1098,29 +1114,50 @@ void mmt4d_mfma_kernel(Args a) {
       }
     };
     if constexpr (HALVES == 2) {
-      // Five slots of half a step (64 bytes of K: (BM + BN) * 64 bytes of LDS);
-      // half-step j (step j / 2, half j % 2) lives in slot j % 5. In its memory
-      // phase of step s a wave reads both halves of the step; group 0 then
-      // issues the whole half-step 2 s + 3 (the slot of half-step 2 s - 2, which
-      // group 1 finished reading a phase ago) and waits for it at the end of its
-      // compute phase, one barrier before its first read; group 1 issues
-      // half-step 2 s + 4 (the slot of 2 s - 1) and waits for it at the end of
-      // its next memory phase, again one barrier before the first read. Both
-      // groups thus bring half of every step, each in its own memory phase.
+      // A ring of RING = 2 D + 1 slots of half a step (64 bytes of K: (BM + BN) *
+      // 64 bytes of LDS); half-step j (step j / 2, half j % 2) lives in slot
+      // j % RING. In its memory phase of step s a wave reads both halves of the
+      // step; group 0 then issues the whole half-step 2 s + RING - 2 (the slot of
+      // half-step 2 s - 2, which group 1 finished reading a phase ago), group 1
+      // the half-step 2 s + RING - 1 (the slot of 2 s - 1). Both groups thus bring
+      // half of every step (group 0 the second halves, group 1 the first), each
+      // in its own memory phase, D - 1 and D steps ahead; each waits, one barrier
+      // before the first read of the half-step its group brought for step s + 1,
+      // until only what it issued later is still in flight: group 0 at the end
+      // of its compute phase (D - 2 issues), group 1 at the end of its memory
+      // phase (D - 1 issues).
       static_assert(NKK == 1, "one MFMA K-group per step");
+      constexpr int RING = ring_slots<E, BM, BN>();
+      constexpr int D = (RING - 1) / 2;
       constexpr uint32_t SLOT = (BM + BN) * 64;
       constexpr uint32_t IMG_B = BM * 64;
-      // Half-steps 0, 1, 2 before the first phase: group 1 brings 0 and 2, group 0 brings 1.
+      // Half-steps 0 .. RING - 3 before the first phase: group 1 brings the even
+      // ones, group 0 the odd ones.
       if (group == 0) {
-        issue_dma(1 * SLOT, 0, 1);
+#pragma unroll
+        for (int j = 1; j <= RING - 4; j += 2) issue_dma((uint32_t)j * SLOT, min(j / 2, last), 1);
       } else {
-        issue_dma(0 * SLOT, 0, 0);
-        issue_dma(2 * SLOT, min(1, last), 0);
+#pragma unroll
+        for (int j = 0; j <= RING - 3; j += 2) issue_dma((uint32_t)j * SLOT, min(j / 2, last), 0);
       }
       wait_vmem_in_flight<0>();
       __builtin_amdgcn_s_barrier();
-      if (group == 1) __builtin_amdgcn_s_barrier();
       v4i fa[TM][HALVES], fb[TN][HALVES];
+      if constexpr (E == Elem::kS16) {
+        // The 16-bit integers read the fragments of a step a phase ahead of its
+        // memory phase (see their step below): those of step 0 here.
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+          fa[tm][0] = read_frag((uint32_t)(wm * TM + tm) * 1024);
+          fa[tm][1] = read_frag(SLOT + (uint32_t)(wm * TM + tm) * 1024);
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+          fb[tn][0] = read_frag(IMG_B + (uint32_t)(wn * TN + tn) * 1024);
+          fb[tn][1] = read_frag(SLOT + IMG_B + (uint32_t)(wn * TN + tn) * 1024);
+        }
+      }
+      if (group == 1) __builtin_amdgcn_s_barrier();
       // ---- 16-bit integers -------------------------------------------------
       // With a = 256 ah + al + 128 (ah the signed high byte, al the low byte
       // minus 128, both in [-128, 127]) and b likewise,
@@ -1159,98 +1196,179 @@ void mmt4d_mfma_kernel(Args a) {
           }
         return sum;
       };
-      // f[0], f[1] (sixteen elements of one row) -> f[0]: their high bytes,
-      // f[1]: their low bytes minus 128. The order of the sixteen is the same
-      // for both operands, which is all the sum over K needs.
-      auto split16 = [&](v4i (&f)[HALVES]) {
-        v4i hi, lo;
+      // The sixteen elements of one row in f[0], f[1] -> their high bytes, or
+      // their low bytes minus 128. The order of the sixteen is the same in both
+      // and for both operands, which is all the sum over K needs.
+      auto high_bytes = [&](const v4i (&f)[HALVES]) {
+        v4i hi;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-          for (int w = 0; w < 2; ++w) {
-            const uint32_t d0 = (uint32_t)f[h][2 * w], d1 = (uint32_t)f[h][2 * w + 1];
-            hi[2 * h + w] = (int)__builtin_amdgcn_perm(d1, d0, 0x07050301u);
-            lo[2 * h + w] = (int)(__builtin_amdgcn_perm(d1, d0, 0x06040200u) ^ 0x80808080u);
+          for (int w = 0; w < 2; ++w)
+            hi[2 * h + w] = (int)__builtin_amdgcn_perm((uint32_t)f[h][2 * w + 1], (uint32_t)f[h][2 * w], 0x07050301u);
+        return hi;
+      };
+      auto low_bytes = [&](const v4i (&f)[HALVES]) {
+        v4i lo;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int w = 0; w < 2; ++w)
+            lo[2 * h + w] = (int)(__builtin_amdgcn_perm((uint32_t)f[h][2 * w + 1], (uint32_t)f[h][2 * w], 0x06040200u) ^
+                                  0x80808080u);
+        return lo;
+      };
+      v4i ha[S16 ? TM : 1], hb[S16 ? TN : 1];
+      // The fragment reads of a step, both halves of each fragment.
+      auto read_frags16 = [&](uint32_t slot0, uint32_t slot1) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+          fa[tm][0] = read_frag(slot0 + (uint32_t)(wm * TM + tm) * 1024);
+          fa[tm][1] = read_frag(slot1 + (uint32_t)(wm * TM + tm) * 1024);
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+          fb[tn][0] = read_frag(slot0 + IMG_B + (uint32_t)(wn * TN + tn) * 1024);
+          fb[tn][1] = read_frag(slot1 + IMG_B + (uint32_t)(wn * TN + tn) * 1024);
+        }
+      };
+      // A step of the 16-bit integers. A wave issues one instruction per turn of
+      // its SIMD (every fourth cycle), and this kernel has some 200 of them per
+      // wave and step (32 MFMAs, 100 vector ALU instructions for the byte split
+      // and the row sums, 24 LDS reads, the loads, scalar bookkeeping) against
+      // 128 turns in the 512 cycles its MFMAs take: it is bound by instruction
+      // issue, not by the matrix pipe. What helps is to spread the instructions
+      // evenly over the two phases. A memory phase made of reads, then permutes,
+      // is the longer one by far, so the reads move: a wave issues the reads of step s + 1
+      // in the middle of its compute phase of step s, once the low bytes of
+      // step s are out of the raw fragments (the same registers take the new
+      // ones), and they return under the second half of its MFMAs. The memory
+      // phase is then: issue of the loads, high bytes, row sums.
+      //   compute phase: high x high and high x low products (need what the
+      //   memory phase prepared, and the low bytes of the LHS) with the low
+      //   bytes worked out beside them, three vector ALU instructions under each
+      //   MFMA; then the fragment reads beside the low x low and low x high
+      //   products. Products that share an accumulator are a whole sweep of the
+      //   blocks apart.
+      // Reading step s + 1 a phase early asks for its loads a phase early: every
+      // wave waits at the end of both of its phases until at most D - 2 of its
+      // issues are in flight, which covers group 0's half of step s + 1 at the end
+      // of its memory phase of step s and group 1's half at the end of its
+      // compute phase of step s - 1, both one barrier before group 0's reads.
+      static_assert(!S16 || D >= 3, "the early fragment reads need a ring of seven slots or more");
+      auto step_body16 = [&](int s, auto phase_c) __attribute__((always_inline)) {
+        constexpr int P = decltype(phase_c)::value;  // s % RING
+        // ---- memory phase ----
+        // (no branch on the group: it would end the basic block and with it the
+        // compiler's count of the fragment reads still in flight)
+        const uint32_t dma_slot = group == 0 ? (uint32_t)((2 * P + RING - 2) % RING) * SLOT
+                                             : (uint32_t)((2 * P + RING - 1) % RING) * SLOT;
+        issue_dma(dma_slot, min(s + D - 1 + group, last), 1 - group);
+        if constexpr (RBC == 2) wait_lds_reads();   // (the transposing reads: the compiler does not see them)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) ha[tm] = high_bytes(fa[tm]);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) hb[tn] = high_bytes(fb[tn]);
+        __builtin_amdgcn_sched_barrier(0);
+        // Row sums of the fragments this wave is responsible for.
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+          if (tm % WGN == wn) rsa[tm] = row_sum16(fa[tm], rsa[tm]);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          if (tn % WGM == wm) rsb[tn] = row_sum16(fb[tn], rsb[tn]);
+        wait_vmem_in_flight<DU*(D - 2)>();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- compute phase ----
+        v4i la[TM], lb[TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) la[tm] = low_bytes(fa[tm]);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) lb[tn] = low_bytes(fb[tn]);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            hh[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hb[tn], ha[tm], hh[tm][tn], 0, 0, 0);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            mid[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hb[tn], la[tm], mid[tm][tn], 0, 0, 0);
+        constexpr int kLowOps = 2 * 4 * (TM + TN);        // a permute and an exclusive-or per word
+        constexpr int kBeside = 2 * TM * TN;              // the first two sweeps
+        constexpr int kPer = (kLowOps + kBeside - 1) / kBeside;
+        // (masks: 0x008 matrix instructions, 0x002 vector ALU, 0x100 LDS reads)
+#pragma unroll
+        for (int i = 0; i < kBeside; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, kPer, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags16((uint32_t)((2 * P + 2) % RING) * SLOT, (uint32_t)((2 * P + 3) % RING) * SLOT);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            acc[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lb[tn], la[tm], acc[tm][tn], 0, 0, 0);
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            mid[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lb[tn], ha[tm], mid[tm][tn], 0, 0, 0);
+        if constexpr (RBC != 2) {
+          // Two read instructions per 16-byte piece for tile rows under 16 bytes.
+          constexpr int kReads = (RBC >= 16 ? 1 : 2) * 2 * (TM + TN);
+          constexpr int kPerR = (kReads + kBeside - 1) / kBeside;
+#pragma unroll
+          for (int i = 0; i < kBeside; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+            __builtin_amdgcn_sched_group_barrier(0x100, kPerR, 1);
           }
-        f[0] = hi;
-        f[1] = lo;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmem_in_flight<DU*(D - 2)>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
       };
-      auto mfmas16 = [&]() {
-        // Products that share an accumulator are a whole sweep of the blocks apart.
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-          for (int tn = 0; tn < TN; ++tn)
-            hh[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][0], fa[tm][0], hh[tm][tn], 0, 0, 0);
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-          for (int tn = 0; tn < TN; ++tn)
-            mid[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][0], fa[tm][1], mid[tm][tn], 0, 0, 0);
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-          for (int tn = 0; tn < TN; ++tn)
-            acc[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][1], fa[tm][1], acc[tm][tn], 0, 0, 0);
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-          for (int tn = 0; tn < TN; ++tn)
-            mid[tm][tn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[tn][1], fa[tm][0], mid[tm][tn], 0, 0, 0);
-      };
-      auto step_body = [&](int s, auto phase_c) {
-        constexpr int P = decltype(phase_c)::value;  // s % 5
+      auto step_body = [&](int s, auto phase_c) __attribute__((always_inline)) {
+        constexpr int P = decltype(phase_c)::value;  // s % RING
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          constexpr uint32_t unused = 0; (void)unused;
-          const uint32_t slot = (uint32_t)((2 * P + h) % 5) * SLOT;
+          const uint32_t slot = (uint32_t)((2 * P + h) % RING) * SLOT;
 #pragma unroll
           for (int tm = 0; tm < TM; ++tm) fa[tm][h] = read_frag(slot + (uint32_t)(wm * TM + tm) * 1024);
 #pragma unroll
           for (int tn = 0; tn < TN; ++tn) fb[tn][h] = read_frag(slot + IMG_B + (uint32_t)(wn * TN + tn) * 1024);
         }
         if (group == 0) {
-          issue_dma((uint32_t)((2 * P + 3) % 5) * SLOT, min(s + 1, last), 1);
+          issue_dma((uint32_t)((2 * P + RING - 2) % RING) * SLOT, min(s + D - 1, last), 1);
         } else {
-          issue_dma((uint32_t)((2 * P + 4) % 5) * SLOT, min(s + 2, last), 0);
-          wait_vmem_in_flight<DU>();   // the half-step issued a step ago has landed
+          issue_dma((uint32_t)((2 * P + RING - 1) % RING) * SLOT, min(s + D, last), 0);
+          wait_vmem_in_flight<DU*(D - 1)>();   // the first half of step s + 1 has landed
         }
         wait_lds_reads();
-        if constexpr (S16) {
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int tm = 0; tm < TM; ++tm) {
-            if (tm % WGN == wn) rsa[tm] = row_sum16(fa[tm], rsa[tm]);
-            split16(fa[tm]);
-          }
-#pragma unroll
-          for (int tn = 0; tn < TN; ++tn) {
-            if (tn % WGM == wm) rsb[tn] = row_sum16(fb[tn], rsb[tn]);
-            split16(fb[tn]);
-          }
-        }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (S16) mfmas16();
-        else mfmas(fa, fb);
+        mfmas(fa, fb);
         __builtin_amdgcn_sched_barrier(0);
-        if (group == 0) wait_vmem_in_flight<0>();
+        if (group == 0) wait_vmem_in_flight<DU*(D - 2)>();   // the second half of step s + 1 has landed
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       };
+      auto step = [&](int s, auto phase_c) __attribute__((always_inline)) {
+        if constexpr (S16) step_body16(s, phase_c);
+        else step_body(s, phase_c);
+      };
       int s = 0;
-      for (; s + 5 <= a.steps; s += 5) {
-        step_body(s, std::integral_constant<int, 0>{});
-        step_body(s + 1, std::integral_constant<int, 1>{});
-        step_body(s + 2, std::integral_constant<int, 2>{});
-        step_body(s + 3, std::integral_constant<int, 3>{});
-        step_body(s + 4, std::integral_constant<int, 4>{});
-      }
-      if (s < a.steps) step_body(s, std::integral_constant<int, 0>{});
-      if (s + 1 < a.steps) step_body(s + 1, std::integral_constant<int, 1>{});
-      if (s + 2 < a.steps) step_body(s + 2, std::integral_constant<int, 2>{});
-      if (s + 3 < a.steps) step_body(s + 3, std::integral_constant<int, 3>{});
+      for (; s + RING <= a.steps; s += RING)
+        static_for<0, RING>([&](auto p) __attribute__((always_inline)) { step(s + decltype(p)::value, p); });
+      static_for<0, RING - 1>([&](auto p) __attribute__((always_inline)) {
+        if (s + decltype(p)::value < a.steps) step(s + decltype(p)::value, p);
+      });
       if constexpr (S16) {
         // Row sums through LDS (every load has landed and every fragment has
         // been read once all waves are past the barrier below): per row the
@@ -1386,7 +1504,7 @@ struct Shape {
   static constexpr int BN = WGN * TN * 16;
   static constexpr size_t kLdsBytes =
       (PIPE == 5 && ElemTraits<E>::kHalves == 2)
-          ? 5 * (size_t)(BM + BN) * 64   // five slots of half a step
+          ? ring_slots<E, BM, BN>() * (size_t)(BM + BN) * 64   // a ring of half-step slots
           : (PIPE == 5 ? kStages5 : PIPE == 0 || PIPE == 4 ? 2 : 3) *
                 (size_t)(PIPE == 2 || PIPE == 3 ? BM : BM + BN) * KS;
 };
