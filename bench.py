@@ -545,10 +545,10 @@ def main() -> int:
             targets["s16_mmt4d_4096_k2"] = {
                 "kernel": kk["kernel"], "us": kk["avg_us"], "TOPS": round(kk["achieved"], 1),
                 "frac": round(kk["frac"], 3),
-                "roofline": {"bound": "vdot2", "achieved": kk["achieved"], "peak": rn.PEAK_TFLOPS["s16"],
+                "roofline": {"bound": "mfma", "achieved": kk["achieved"], "peak": rn.PEAK_TFLOPS["s16"],
                              "unit": kk["unit"], "frac": kk["frac"], "traffic": None,
-                             "what": "no 16-bit integer matrix instruction: the peak is that of "
-                                     "v_dot2_i32_i16 on the vector ALUs"}}
+                             "what": "no 16-bit integer matrix instruction: a 16 x 16-bit product runs as four "
+                                     "8 x 8-bit products, so the peak is a quarter of the int8 one"}}
         for name in TARGET_PACK:
             e = extra.get(name)
             if not e or "pack" not in e["kernels"]:

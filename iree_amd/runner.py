@@ -23,9 +23,9 @@ from . import ukernel as uk
 # Published MI355X peaks (dense).
 PEAK_HBM_GBPS = 8000.0
 PEAK_TFLOPS = {"s8": 5000.0, "f8": 5000.0, "f16": 2500.0, "bf16": 2500.0, "f32": 157.3,
-               # s16 has no matrix instruction: the rate of the vector dot product
-               # v_dot2_i32_i16 (256 CUs x 4 SIMDs x 16 lanes x 2 multiply-adds at 2.4 GHz).
-               "s16": 157.3}
+               # s16 has no matrix instruction of its own: a 16 x 16-bit product is four
+               # 8 x 8-bit products on the int8 matrix instruction, so a quarter of its peak.
+               "s16": 1250.0}
 
 
 @dataclasses.dataclass
@@ -240,8 +240,8 @@ class Runner:
                             op.bytes, "s8", dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1,
                                                  N1=N1, K1=K1, M0=M0, N0=N0, K0=K0))
         if name.startswith("s16_mmt4d_"):
-            # s16 x s16 -> s32 (no 16-bit integer matrix instruction: the vector
-            # dot-product kernel), e.g. the reference's AVX-512 VNNI tile 16x16x2
+            # s16 x s16 -> s32 (no 16-bit integer matrix instruction: four 8-bit
+            # products per element pair), e.g. the reference's AVX-512 VNNI tile 16x16x2
             _, _, size, k0 = name.split("_")
             S, K0 = int(size), int(k0[1:])
             M0 = N0 = 16
@@ -255,8 +255,7 @@ class Runner:
             op = self._mmt4d_op(lhs4, rhs4, out4, M1, N1, K1, M0, N0, K0,
                                 uk.MMT4D_TYPE_S16S16S32 | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION,
                                 "s16", 2)
-            op.bound = "vdot2"   # no 16-bit integer matrix instruction: bound by the vector dot product's rate
-            return Workload(name, f"mmt4d s16xs16->s32 {S}^3 tiles 16x16x{K0} (vector dot products)", [op],
+            return Workload(name, f"mmt4d s16xs16->s32 {S}^3 tiles 16x16x{K0} (four s8 products per element pair)", [op],
                             op.flops, op.bytes, "s16",
                             dict(lhs4=lhs4, rhs4=rhs4, out4=out4, M1=M1, N1=N1, K1=K1,
                                  M0=M0, N0=N0, K0=K0))
