@@ -83,10 +83,14 @@ enum {
 /* iree_uk_mmt4d_info result bits (exported_bits.h:49). On this target the bit
  * means "an MFMA kernel (not the scalar fallback kernel) serves this case".
  * It is not set for the 16-bit integer LHS types (S16S16S32, S16U4S32,
- * S16S8S32): the hardware has no 16-bit integer matrix instruction. With the
- * fallback flag and K0 a power of two >= 2 they run on a vector dot-product
- * kernel (v_dot2_i32_i16 fed from LDS, bit-exact), about twenty times the
- * scalar kernel's rate; other K0 on the scalar kernel. */
+ * S16S8S32): the hardware has no 16-bit integer matrix instruction, and no
+ * kernel serves every shape of a tile. With the fallback flag, S16S16S32
+ * runs on the matrix cores as four 8-bit products per element pair (exact
+ * modulo 2^32) when K is a whole number of 64-element steps and the result has
+ * more than 32 rows and columns; otherwise, with K0 a power of two >= 2, these
+ * types run on a vector dot-product kernel (v_dot2_i32_i16 fed from LDS,
+ * bit-exact), about twenty times the scalar kernel's rate; other K0 on the
+ * scalar kernel. */
 enum {
   IREE_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION = 0x1,
 };
