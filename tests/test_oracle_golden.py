@@ -145,7 +145,7 @@ def test_f8_decode_closed_form(oracle):
 
 
 def test_f8_decode_known_values(oracle):
-    # runtime/src/iree/base/internal/math_test.cc:483-589 and the survey KATs.
+    # runtime/src/iree/base/internal/math_test.cc:483-589 and further known-answer values.
     kv = {0x01: 2.0 ** -9, 0x07: 7 * 2.0 ** -9, 0x08: 2.0 ** -6,
           0x0F: 0.029296875, 0x28: 0.25, 0x38: 1.0, 0x40: 2.0, 0x77: 240.0,
           0x78: 256.0, 0x7E: 448.0, 0xB8: -1.0, 0xFE: -448.0, 0xED: -104.0}
