@@ -472,6 +472,7 @@ def main() -> int:
                 gbps = R.copy2d_ceiling_gbps(rows, row_bytes, sp, dp)
                 entry["copy2d_ceiling"] = {
                     "GBps": round(gbps, 1), "frac": round(gbps / rn.PEAK_HBM_GBPS, 4),
+                    "whole_lines_only_frac": round(R.last_copy2d_whole_lines_gbps / rn.PEAK_HBM_GBPS, 4),
                     "what": f"plain copy of {rows} rows x {row_bytes} B, pitch {sp} -> {dp} B"}
                 if "unpack" in w.ops[-1].name:
                     # unpack moves the matrix the other way: its ceiling is
@@ -479,6 +480,7 @@ def main() -> int:
                     back = R.copy2d_ceiling_gbps(rows, row_bytes, dp, sp)
                     entry["copy2d_ceiling_unpack"] = {
                         "GBps": round(back, 1), "frac": round(back / rn.PEAK_HBM_GBPS, 4),
+                        "whole_lines_only_frac": round(R.last_copy2d_whole_lines_gbps / rn.PEAK_HBM_GBPS, 4),
                         "what": f"plain copy of {rows} rows x {row_bytes} B, pitch {dp} -> {sp} B"}
                 keep = w.keep
                 if "back" in keep:

@@ -433,7 +433,13 @@ IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_kernel_name(void);
  * iree_uk_amd_probe_copy2d: `iters` plain copies of `rows` rows of `row_bytes`
  * bytes between two pitches (everything 4-byte aligned): the ceiling of a
  * pack / unpack that moves the same matrix between the same pitches.
- * *seconds_per_copy receives the average. */
+ * *seconds_per_copy receives the average of the fastest of five ways of
+ * writing the copy (1, 4 or 8 vectors in flight per lane, ordinary or
+ * non-temporal stores, and one whose stores cover only whole 128-byte lines
+ * of the destination whatever its pitch).
+ * iree_uk_amd_probe_copy2d_variants: the same, and seconds_per_variant[0..4]
+ * (when not NULL) receive the average of every variant, the whole-line one
+ * last. */
 IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(
     uint32_t type_flags, const void* operands, int64_t operand_bytes, int iters,
     int workgroups, void* sink, void* stream, double* ops_per_second);
@@ -441,6 +447,10 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(
     const void* src, int64_t src_pitch, void* dst, int64_t dst_pitch,
     int64_t row_bytes, int64_t rows, int iters, void* stream,
     double* seconds_per_copy);
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d_variants(
+    const void* src, int64_t src_pitch, void* dst, int64_t dst_pitch,
+    int64_t row_bytes, int64_t rows, int iters, void* stream,
+    double* seconds_per_copy, double* seconds_per_variant);
 
 /* Per-kernel device timing for the calling thread. Between begin and end,
  * every kernel an entry point launches carries its own start/stop event pair

@@ -85,26 +85,36 @@ int run_mfma_peak(const v4i* operands, int n_operands, int iters, int workgroups
 // A workgroup copies 4 KiB pieces of rows (16 bytes per lane, 4-byte aligned
 // like the pack kernels' 2-D side), walking pieces grid-stride, DEPTH pieces
 // per turn: all loads of a turn are issued before its stores. NT: non-temporal
-// stores (the destination is not read again).
-template <int DEPTH, bool NT>
+// stores (the destination is not read again). LINES: the pieces of a row are
+// shifted so that every store of a wave covers whole 128-byte lines of the
+// destination whatever the pitch (one more, partial piece per row; the loads
+// are then the unaligned side).
+template <int DEPTH, bool NT, bool LINES = false>
 __global__ __launch_bounds__(256) void copy2d_kernel(const char* src, int64_t src_pitch, char* dst,
                                                      int64_t dst_pitch, int64_t row_bytes,
                                                      int64_t rows) {
   typedef uk_mfma::v4i v4i_a4 __attribute__((aligned(4)));
-  const int64_t pieces_per_row = (row_bytes + 4095) / 4096;
+  const int64_t pieces_per_row = (row_bytes + 4095) / 4096 + (LINES ? 1 : 0);
   const int64_t total = pieces_per_row * rows;
+  // Byte offset of lane's vector of piece p inside its row (may start before the
+  // row or end after it: such a vector moves word by word, or not at all).
+  auto offset_of = [&](int64_t p, int64_t* row) {
+    *row = p / pieces_per_row;
+    int64_t off = (p - *row * pieces_per_row) * 4096 + (int64_t)threadIdx.x * 16;
+    if (LINES) off -= (int64_t)(((uintptr_t)dst + (uint64_t)(*row * dst_pitch)) & 127);
+    return off;
+  };
   for (int64_t p0 = (int64_t)blockIdx.x * DEPTH; p0 < total; p0 += (int64_t)gridDim.x * DEPTH) {
     uk_mfma::v4i v[DEPTH];
     int64_t so[DEPTH], dof[DEPTH];
     bool whole[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      const int64_t p = p0 + d;
-      const int64_t row = p / pieces_per_row, piece = p - row * pieces_per_row;
-      const int64_t off = piece * 4096 + (int64_t)threadIdx.x * 16;
+      int64_t row;
+      const int64_t off = offset_of(p0 + d, &row);
       so[d] = row * src_pitch + off;
       dof[d] = row * dst_pitch + off;
-      whole[d] = p < total && off + 16 <= row_bytes;
+      whole[d] = p0 + d < total && off >= 0 && off + 16 <= row_bytes;
       if (whole[d]) v[d] = *reinterpret_cast<const v4i_a4*>(src + so[d]);
     }
 #pragma unroll
@@ -113,13 +123,13 @@ __global__ __launch_bounds__(256) void copy2d_kernel(const char* src, int64_t sr
         if (NT) __builtin_nontemporal_store(v[d], reinterpret_cast<v4i_a4*>(dst + dof[d]));
         else *reinterpret_cast<v4i_a4*>(dst + dof[d]) = v[d];
       } else if (p0 + d < total) {
-        // the last, partial vector of a row: word by word
-        const int64_t p = p0 + d;
-        const int64_t row = p / pieces_per_row, piece = p - row * pieces_per_row;
-        const int64_t off = piece * 4096 + (int64_t)threadIdx.x * 16;
-        for (int64_t b = off; b < row_bytes && b < off + 16; b += 4)
-          *reinterpret_cast<int*>(dst + row * dst_pitch + b) =
-              *reinterpret_cast<const int*>(src + row * src_pitch + b);
+        // a vector that straddles an end of its row: word by word
+        int64_t row;
+        const int64_t off = offset_of(p0 + d, &row);
+        for (int64_t b = off; b < off + 16; b += 4)
+          if (b >= 0 && b < row_bytes)
+            *reinterpret_cast<int*>(dst + row * dst_pitch + b) =
+                *reinterpret_cast<const int*>(src + row * src_pitch + b);
       }
     }
   }
@@ -194,15 +204,26 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(uint32_t type_flags, const vo
 
 // Copies `rows` rows of `row_bytes` bytes (a multiple of 4) from `src` (rows
 // `src_pitch` bytes apart) to `dst` (`dst_pitch`) `iters` times on `stream`,
-// in four variants of the copy kernel (1, 4 or 8 vectors in flight per lane,
-// ordinary or non-temporal stores), and returns the average seconds per copy
-// of the fastest variant: the ceiling of a pack / unpack
-// that moves the same matrix between the same two pitches. All pointers and
-// pitches 4-byte aligned.
+// in five variants of the copy kernel (1, 4 or 8 vectors in flight per lane,
+// ordinary or non-temporal stores, pieces shifted row by row so that only
+// whole 128-byte lines of the destination are written), and returns the
+// average seconds per copy of the fastest variant: the ceiling of a pack /
+// unpack that moves the same matrix between the same two pitches. When
+// `seconds_per_variant` is not null it receives the five averages (the last
+// one is the whole-line variant). All pointers and pitches 4-byte aligned.
 IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(const void* src, int64_t src_pitch, void* dst,
                                                 int64_t dst_pitch, int64_t row_bytes,
                                                 int64_t rows, int iters, void* stream_v,
                                                 double* seconds_per_copy) {
+  return iree_uk_amd_probe_copy2d_variants(src, src_pitch, dst, dst_pitch, row_bytes, rows, iters,
+                                           stream_v, seconds_per_copy, nullptr);
+}
+
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d_variants(const void* src, int64_t src_pitch, void* dst,
+                                                         int64_t dst_pitch, int64_t row_bytes,
+                                                         int64_t rows, int iters, void* stream_v,
+                                                         double* seconds_per_copy,
+                                                         double* seconds_per_variant) {
   hipStream_t stream = (hipStream_t)stream_v;
   if (!src || !dst || !seconds_per_copy || iters < 1 || row_bytes < 4 || (row_bytes & 3) || rows < 1 ||
       (((uintptr_t)src | (uintptr_t)dst | (uint64_t)src_pitch | (uint64_t)dst_pitch) & 3)) {
@@ -219,7 +240,7 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(const void* src, int64_t src_pit
     (void)hipEventDestroy(start);
     return (int)hipErrorUnknown;
   }
-  // Four ways of writing the same copy; the fastest one is the ceiling.
+  // Five ways of writing the same copy; the fastest one is the ceiling.
   auto run = [&](int variant) {
     const char* s8 = (const char*)src;
     char* d8 = (char*)dst;
@@ -227,12 +248,13 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(const void* src, int64_t src_pit
       case 0: hipLaunchKernelGGL((copy2d_kernel<1, false>), dim3(cus * 8), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
       case 1: hipLaunchKernelGGL((copy2d_kernel<4, false>), dim3(cus * 4), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
       case 2: hipLaunchKernelGGL((copy2d_kernel<4, true>), dim3(cus * 4), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
-      default: hipLaunchKernelGGL((copy2d_kernel<8, true>), dim3(cus * 2), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
+      case 3: hipLaunchKernelGGL((copy2d_kernel<8, true>), dim3(cus * 2), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
+      default: hipLaunchKernelGGL((copy2d_kernel<4, true, true>), dim3(cus * 4), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
     }
   };
   int st = 0;
   double best = 0.0;
-  for (int variant = 0; variant < 4 && st == 0; ++variant) {
+  for (int variant = 0; variant < 5 && st == 0; ++variant) {
     run(variant);
     run(variant);
     st = (int)hipEventRecord(start, stream);
@@ -244,6 +266,7 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(const void* src, int64_t src_pit
     if (st == 0) st = (int)hipEventElapsedTime(&ms, start, stop);
     const double sec = (double)ms * 1e-3 / iters;
     if (st == 0 && (best == 0.0 || sec < best)) best = sec;
+    if (st == 0 && seconds_per_variant) seconds_per_variant[variant] = sec;
   }
   (void)hipEventDestroy(start);
   (void)hipEventDestroy(stop);

@@ -702,8 +702,10 @@ class Runner:
         src = torch.empty(rows * src_pitch, dtype=torch.uint8, device="cuda")
         dst = torch.empty(rows * dst_pitch, dtype=torch.uint8, device="cuda")
         self.stream.synchronize()
-        sec = self.lib.probe_copy2d(src.data_ptr(), src_pitch, dst.data_ptr(), dst_pitch, row_bytes,
-                                    rows, iters, self.stream.cuda_stream)
+        sec, per = self.lib.probe_copy2d_variants(src.data_ptr(), src_pitch, dst.data_ptr(), dst_pitch,
+                                                  row_bytes, rows, iters, self.stream.cuda_stream)
+        # (the last variant writes whole 128-byte lines only, whatever the pitch)
+        self.last_copy2d_whole_lines_gbps = 2.0 * rows * row_bytes / per[4] / 1e9
         return 2.0 * rows * row_bytes / sec / 1e9
 
     def measured_copy_gbps(self, nbytes: int = 1 << 30, iters: int = 10) -> float:

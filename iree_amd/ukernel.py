@@ -195,6 +195,10 @@ class UKernelLibrary:
         L.iree_uk_amd_probe_copy2d.argtypes = [_vp, _i64, _vp, _i64, _i64, _i64, ctypes.c_int, _vp,
                                                ctypes.POINTER(ctypes.c_double)]
         L.iree_uk_amd_probe_copy2d.restype = ctypes.c_int
+        L.iree_uk_amd_probe_copy2d_variants.argtypes = [_vp, _i64, _vp, _i64, _i64, _i64, ctypes.c_int, _vp,
+                                                        ctypes.POINTER(ctypes.c_double),
+                                                        ctypes.POINTER(ctypes.c_double)]
+        L.iree_uk_amd_probe_copy2d_variants.restype = ctypes.c_int
         self._handler_ref = None
         self._violations: list[str] = []
 
@@ -310,6 +314,17 @@ class UKernelLibrary:
         if st != 0:
             raise RuntimeError(f"iree_uk_amd_probe_copy2d: status {st}")
         return sec.value
+
+    def probe_copy2d_variants(self, src, src_pitch, dst, dst_pitch, row_bytes, rows, iters, stream):
+        """(seconds of the fastest copy variant, [seconds of each of the five
+        variants]); the last variant writes whole 128-byte lines only."""
+        sec = ctypes.c_double(0.0)
+        per = (ctypes.c_double * 5)()
+        st = self.lib.iree_uk_amd_probe_copy2d_variants(src, src_pitch, dst, dst_pitch, row_bytes, rows,
+                                                        iters, stream, ctypes.byref(sec), per)
+        if st != 0:
+            raise RuntimeError(f"iree_uk_amd_probe_copy2d_variants: status {st}")
+        return sec.value, list(per)
 
     # --------------------------------------------------------------- control
     def _check(self):
