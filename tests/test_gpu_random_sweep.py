@@ -136,7 +136,7 @@ def test_mmt4d_random_sweep_larger_shapes_and_forced_variants(gpu, oracle):
     types = [uk.MMT4D_TYPE_S8S8S32, uk.MMT4D_TYPE_F16F16F32, uk.MMT4D_TYPE_BF16BF16F32,
              uk.MMT4D_TYPE_F32F32F32, uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32]
     done = 0
-    for ci in range(400):
+    for ci in range(300):
         tf = types[ci % len(types)]
         eb = uk.MMT4D_TYPE_BITS[tf][0] // 8
         M0, N0 = int(rng.choice([4, 8, 12, 16, 24, 32, 48, 64])), int(rng.choice([4, 8, 16, 20, 32, 64]))
@@ -158,7 +158,7 @@ def test_mmt4d_random_sweep_larger_shapes_and_forced_variants(gpu, oracle):
         assert lib.last_kernel_name().startswith("mmt4d_mfma"), (ci, c, lib.last_kernel_name())
         done += 1
     lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
-    assert done >= 120, done
+    assert done >= 90, done
 
 
 def test_mmt4d_random_sweep_lds_direct_pipeline(gpu, oracle):
@@ -173,7 +173,7 @@ def test_mmt4d_random_sweep_lds_direct_pipeline(gpu, oracle):
              uk.MMT4D_TYPE_F8E4M3FNF8E4M3FNF32]
     names = set()
     done = 0
-    for ci in range(300):
+    for ci in range(210):
         tf = types[ci % len(types)]
         eb = uk.MMT4D_TYPE_BITS[tf & 0xFF][0] // 8
         M0, N0 = int(rng.choice([4, 8, 12, 16, 24, 32, 48, 64])), int(rng.choice([4, 8, 16, 20, 32, 64]))
@@ -194,7 +194,7 @@ def test_mmt4d_random_sweep_lds_direct_pipeline(gpu, oracle):
         names.add(lib.last_kernel_name())
         done += 1
     lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
-    assert done >= 100, done
+    assert done >= 70, done
     assert {"mmt4d_mfma_256x256_lds_direct", "mmt4d_mfma_128x512_lds_direct",
             "mmt4d_mfma_128x128_lds_direct", "mmt4d_mfma_64x64_lds_direct",
             "mmt4d_mfma_256x128_lds_direct"} <= names, names
@@ -298,7 +298,7 @@ def test_mmt4d_random_sweep_narrow_row_kernels(gpu, oracle):
              (uk.MMT4D_TYPE_F16F16F32, 2), (uk.MMT4D_TYPE_BF16BF16F32, 2), (uk.MMT4D_TYPE_BF16BF16F32, 1),
              (uk.MMT4D_TYPE_F32F32F32, 1)]
     served = set()
-    for ci in range(280):
+    for ci in range(196):
         tf, K0 = tiles[ci % len(tiles)]
         rb = K0 * uk.MMT4D_TYPE_BITS[tf][0] // 8
         M0 = int(rng.choice([8, 16, 24, 32, 64]))
