@@ -447,6 +447,15 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d(
     const void* src, int64_t src_pitch, void* dst, int64_t dst_pitch,
     int64_t row_bytes, int64_t rows, int iters, void* stream,
     double* seconds_per_copy);
+/* iree_uk_amd_probe_ds_read_tr16: one wave executes ds_read_b64_tr_b16, every
+ * lane at the 16-bit index `lane_index[lane]` (device memory, 64 ints,
+ * multiples of 4 below `lds_values` <= 16384) of an LDS image whose 16-bit
+ * values equal their own indices; `out` (device memory, 256 shorts) receives
+ * each lane's four values. Waits for `stream`. The fragment reads of the
+ * mmt4d kernels for 2-byte tile rows rest on this instruction's lane mapping;
+ * the test suite pins it through this call. No counterpart in the reference. */
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_ds_read_tr16(
+    const int* lane_index, short* out, int lds_values, void* stream);
 IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d_variants(
     const void* src, int64_t src_pitch, void* dst, int64_t dst_pitch,
     int64_t row_bytes, int64_t rows, int iters, void* stream,

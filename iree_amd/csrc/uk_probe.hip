@@ -135,9 +135,44 @@ __global__ __launch_bounds__(256) void copy2d_kernel(const char* src, int64_t sr
   }
 }
 
+// One wave: LDS holds 16-bit values equal to their own index; lane l reads the
+// eight bytes at 16-bit index lane_index[l] with ds_read_b64_tr_b16 and stores
+// the four values it receives.
+__global__ __launch_bounds__(64) void ds_read_tr16_kernel(const int* lane_index, short* out, int lds_values) {
+  extern __shared__ __attribute__((aligned(16))) short tr16_lds[];
+  for (int i = threadIdx.x; i < lds_values; i += 64) tr16_lds[i] = (short)i;
+  __syncthreads();
+  typedef int v2i __attribute__((ext_vector_type(2)));
+  v2i v;
+  const uint32_t addr = (uint32_t)(uintptr_t)(tr16_lds + lane_index[threadIdx.x]);   // LDS addresses are the low 32 bits
+  asm volatile("ds_read_b64_tr_b16 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+  out[threadIdx.x * 4 + 0] = (short)(v[0] & 0xFFFF);
+  out[threadIdx.x * 4 + 1] = (short)((uint32_t)v[0] >> 16);
+  out[threadIdx.x * 4 + 2] = (short)(v[1] & 0xFFFF);
+  out[threadIdx.x * 4 + 3] = (short)((uint32_t)v[1] >> 16);
+}
+
 }  // namespace
 
 extern "C" {
+
+// Runs ds_read_b64_tr_b16 in one wave for the lane addresses in `lane_index`
+// (64 ints of device memory: the 16-bit index each lane addresses, a multiple
+// of 4, below `lds_values` <= 16384) on an LDS image whose 16-bit values are
+// their own indices; `out` (256 shorts of device memory) receives the four
+// values of every lane. The mmt4d kernels' fragment reads for 2-byte tile rows
+// rest on this instruction's lane mapping; tests/test_gpu_probe.py pins it.
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_ds_read_tr16(const int* lane_index, short* out,
+                                                      int lds_values, void* stream_v) {
+  hipStream_t stream = (hipStream_t)stream_v;
+  if (!lane_index || !out || lds_values < 4 || lds_values > 16384) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(ds_read_tr16_kernel, dim3(1), dim3(64), (size_t)lds_values * 2, stream, lane_index,
+                     out, lds_values);
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return (int)err;
+  return (int)hipStreamSynchronize(stream);
+}
+
 
 // Runs the MFMA-only loop of the element type in `type_flags` (an
 // IREE_UK_FLAG_MMT4D_TYPE_* value: S8S8S32, F16F16F32, BF16BF16F32, F32F32F32

@@ -199,6 +199,8 @@ class UKernelLibrary:
                                                         ctypes.POINTER(ctypes.c_double),
                                                         ctypes.POINTER(ctypes.c_double)]
         L.iree_uk_amd_probe_copy2d_variants.restype = ctypes.c_int
+        L.iree_uk_amd_probe_ds_read_tr16.argtypes = [_vp, _vp, ctypes.c_int, _vp]
+        L.iree_uk_amd_probe_ds_read_tr16.restype = ctypes.c_int
         self._handler_ref = None
         self._violations: list[str] = []
 
@@ -325,6 +327,11 @@ class UKernelLibrary:
         if st != 0:
             raise RuntimeError(f"iree_uk_amd_probe_copy2d_variants: status {st}")
         return sec.value, list(per)
+
+    def probe_ds_read_tr16(self, lane_index_ptr, out_ptr, lds_values, stream) -> None:
+        st = self.lib.iree_uk_amd_probe_ds_read_tr16(lane_index_ptr, out_ptr, lds_values, stream)
+        if st != 0:
+            raise RuntimeError(f"iree_uk_amd_probe_ds_read_tr16: status {st}")
 
     # --------------------------------------------------------------- control
     def _check(self):
