@@ -419,17 +419,17 @@ def test_thread_local_device_memory_is_released_when_the_thread_ends(gpu):
             t.join()
         torch.cuda.synchronize()
 
-    # A first batch lets the HIP runtime settle (it takes device memory in
-    # chunks of its own, 64 MiB at a time, the first time threads come and go);
-    # the second batch is the one that is measured: what each of its threads
-    # staged (24 MiB and more) must all have gone back.
-    run_threads(3)
+    # The HIP runtime takes and returns device memory in chunks of its own (64 MiB
+    # at a time, whenever it pleases on a fresh machine), so the check is made
+    # against what a leak would cost: sixteen threads that each stage 24 MiB and
+    # more would leave 384 MiB behind; a quarter of that is the limit.
+    run_threads(2)
     free_before = torch.cuda.mem_get_info()[0]
-    run_threads(4)
+    run_threads(16)
     free_after = torch.cuda.mem_get_info()[0]
     assert all(h[0] >= 24 << 20 for h in held), held          # each thread staged its own copy
     assert len({h[1] for h in held}) == 1
-    assert free_before - free_after < (8 << 20), (free_before, free_after)
+    assert free_before - free_after < (96 << 20), (free_before, free_after)
 
 
 def test_entry_points_from_concurrent_threads(gpu, oracle):
