@@ -483,6 +483,13 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_timing_end(double* elapsed_us, int* kinds,
 IREE_UK_AMD_EXPORT int64_t iree_uk_amd_staging_bytes(void);
 IREE_UK_AMD_EXPORT int iree_uk_amd_release_staging(void);
 
+/* Device allocations (hipMalloc calls) the library has made in this process so
+ * far, over all threads: the staging arenas above and the K-split workspaces
+ * of iree_uk_mmt4d. A caller, or a test, can see with it that a call
+ * allocated nothing (iree_uk_amd_mmt4d_no_alloc never does). No counterpart
+ * in the reference. */
+IREE_UK_AMD_EXPORT int64_t iree_uk_amd_device_alloc_count(void);
+
 /* Number of devices visible to HIP (0 when there is none or no driver). */
 IREE_UK_AMD_EXPORT int iree_uk_amd_device_count(void);
 

@@ -196,6 +196,7 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
   char* base = nullptr;
   const size_t bytes = want_partials + (size_t)want_counters * sizeof(uint32_t);
   if (hipMalloc((void**)&base, bytes) != hipSuccess) { (void)hipGetLastError(); return 1; }
+  iree_uk_amd_hip_note_device_alloc();
   // The counters start at zero; the kernels keep them there. The fill is
   // ordered before the launch that follows on the same stream.
   if (hipMemsetAsync(base + want_partials, 0, (size_t)want_counters * sizeof(uint32_t), stream) !=

@@ -87,6 +87,9 @@ int iree_uk_amd_hip_copy2d_to_host(void* dst, int64_t dst_pitch,
                                    int64_t width, int64_t height, void* stream);
 int iree_uk_amd_hip_stream_synchronize(void* stream);
 const char* iree_uk_amd_hip_error_string(int status);
+/* Counts one device allocation of the library (see
+ * iree_uk_amd_device_alloc_count). */
+void iree_uk_amd_hip_note_device_alloc(void);
 
 #ifdef __cplusplus
 }

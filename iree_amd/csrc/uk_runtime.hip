@@ -1,6 +1,7 @@
 // Thin C-ABI wrappers over the HIP runtime for the plain-C host layer.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <vector>
 
 #include "uk_hip_abi.h"
@@ -128,10 +129,19 @@ int iree_uk_amd_hip_staging_reserve(void** base, int64_t bytes) {
       arena->base = nullptr;
       return (int)err;
     }
+    iree_uk_amd_hip_note_device_alloc();
     arena->bytes = want;
   }
   *base = arena->base;
   return 0;
+}
+
+// Device allocations (hipMalloc calls) the library has made in this process:
+// the staging arenas here and the K-split workspaces of mmt4d_mfma.hip.
+static std::atomic<int64_t> g_device_allocs{0};
+extern "C" void iree_uk_amd_hip_note_device_alloc(void) { g_device_allocs.fetch_add(1, std::memory_order_relaxed); }
+extern "C" IREE_UK_AMD_EXPORT int64_t iree_uk_amd_device_alloc_count(void) {
+  return g_device_allocs.load(std::memory_order_relaxed);
 }
 
 extern "C" IREE_UK_AMD_EXPORT int64_t iree_uk_amd_staging_bytes(void) {

@@ -186,6 +186,7 @@ class UKernelLibrary:
         L.iree_uk_amd_set_assert_handler.argtypes = [_vp]
         L.iree_uk_amd_timing_begin.restype = None
         L.iree_uk_amd_staging_bytes.restype = _i64
+        L.iree_uk_amd_device_alloc_count.restype = _i64
         L.iree_uk_amd_release_staging.restype = ctypes.c_int
         L.iree_uk_amd_timing_end.argtypes = [_vp, _vp, ctypes.c_int]
         L.iree_uk_amd_timing_end.restype = ctypes.c_int
@@ -404,6 +405,10 @@ class UKernelLibrary:
     def staging_bytes(self) -> int:
         """Device bytes the calling thread's host-operand staging arena holds."""
         return int(self.lib.iree_uk_amd_staging_bytes())
+
+    def device_alloc_count(self) -> int:
+        """hipMalloc calls the library has made in this process so far."""
+        return int(self.lib.iree_uk_amd_device_alloc_count())
 
     def release_staging(self) -> int:
         """Frees the calling thread's staging arena; 0 or a hipError_t value."""
