@@ -16,7 +16,7 @@ OBJ = os.path.join(CSRC, "obj")
 LIB = os.path.join(HERE, "libiree_uk_amd.so")
 
 HIP_SOURCES = ["mmt4d_mfma_s16.hip", "mmt4d_mfma_s8s4.hip",
-               "uk_runtime.hip", "uk_probe.hip", "pack_unpack.hip",
+               "uk_runtime.hip", "uk_probe.hip", "pack_unpack.hip", "pack_tr.hip",
                "mmt4d_generic.hip", "mmt4d_dot2.hip", "conv_nchwc.hip", "mmt4d_mfma.hip", "mmt4d_dispatch.hip"]
 # mmt4d_mfma_inst.hip once per (element type, class of tile row widths): the
 # kernel instantiations of one pair per object file, built in parallel.

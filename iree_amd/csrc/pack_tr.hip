@@ -1,0 +1,329 @@
+// pack with an element-granular transposition inside the tile, for 1- and
+// 2-byte elements, on the LDS transposing reads of gfx950.
+//
+// TRANSPOSE_INNER stores a tile as [b1][b0] (b0 the position along the rows of
+// the source matrix, b1 along its columns; index algebra of
+// runtime/src/iree/builtins/ukernel/tools/pack_test.c:13-71): what is
+// contiguous in the destination runs down a column of the source. That is the
+// form a row-major [K][N] right-hand side takes on its way to [N1][K1][N0][K0]
+// (tests/e2e/linalg/pack_i8.mlir:48-68). An untransposed tile whose rows hold
+// one or two bytes is the same problem with the tile row as the element: the
+// reference's x86 tiles for s8, 16x2 (arch/x86_64/mmt4d_x86_64_tiles.inl),
+// are 16 two-byte elements that run down the source column.
+//
+// A workgroup stages a block of 64 rows x 256 bytes of the matrix in LDS, row
+// major, and reads it back with ds_read_b64_tr_b16 / ds_read_b64_tr_b8. Within
+// a block of 16 lanes these hand lane i, as element j of its eight bytes,
+// element i % E of what lane (16 / E) j + i / E addressed (E = 4 two-byte or 8
+// one-byte elements per lane): when lane l addresses row r0 + l / (16 / E),
+// columns c0 + E (l % (16 / E)) ..., lane i receives column c0 + i of rows
+// r0 .. r0 + E - 1, i.e. eight bytes that are contiguous in the destination.
+// Two reads give a lane 16 such bytes where the tile is that tall. The walk over
+// the blocks is the streaming pack kernels': persistent workgroups, the global
+// loads of the next block issued before the barrier of the current one, two
+// LDS buffers, one barrier per block.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "uk_device_common.h"
+#include "uk_hip_abi.h"
+#include "uk_launch.h"
+
+namespace {
+
+// A block is 64 rows x 256 bytes of the matrix: 16 KB, 256 threads, four
+// workgroups per CU. (64 KB blocks of 1024 threads, 256 x 256 or 64 x 1024,
+// were measured on operands of 64 to 470 MB and were no faster.)
+constexpr int kBlockRows = 64, kBlockRowBytes = 256;
+
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+struct TrArgs {
+  const char* src;
+  char* dst;
+  int64_t src_pitch;        // bytes between matrix rows
+  int64_t s0, s1;           // tiled side: bytes from one row tile / column tile to the next
+  uint32_t rows;            // matrix rows
+  uint32_t row_bytes;       // matrix row length, bytes
+  uint32_t outer0, outer1;  // tiles along rows / columns
+  uint32_t lt0, lt1;        // log2 of the tile's extent along rows / columns, elements
+  uint32_t nblk0, nblk1;    // blocks along rows / columns
+  uint32_t strip;           // block columns per strip of the walk
+  uint32_t lds_pitch;       // bytes per LDS row
+  uint32_t lds_buf_bytes;
+  uint32_t pad32;           // the padding element replicated over 32 bits
+};
+
+template <int EB>
+__device__ __forceinline__ v2u read_tr(uint32_t lds_addr) {
+  v2u v;
+  if constexpr (EB == 2) {
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=&v"(v) : "v"(lds_addr) : "memory");
+  } else {
+    asm volatile("ds_read_b64_tr_b8 %0, %1" : "=&v"(v) : "v"(lds_addr) : "memory");
+  }
+  return v;
+}
+
+// EB: bytes per transposed element. V: bytes a lane stores at once (16 where
+// the tile's extent along the rows is a multiple of 16 bytes, else 8).
+template <int EB, int V>
+__global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kernel(TrArgs a) {
+  constexpr int kThreads = kBlockRows * kBlockRowBytes / 64;  // 64 bytes of the block per thread
+  constexpr int kBlockBytes = kBlockRows * kBlockRowBytes;
+  constexpr int VPR = kBlockRowBytes / 16;     // 16-byte vectors per block row
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  constexpr int E = 8 / EB;                    // elements per lane and read
+  constexpr int CH = 16 / E;                   // 8-byte column chunks per 16 columns
+  constexpr int BC = kBlockRowBytes / EB;      // block columns, elements
+  constexpr int NCG = BC / 16;                 // groups of 16 columns
+  constexpr int RPI = V / EB;                  // rows per item
+  constexpr int N1 = kBlockBytes / 16 / kThreads;  // 16-byte source vectors per thread
+  constexpr int N2 = kBlockBytes / V / kThreads;   // destination vectors per thread
+  constexpr int R = V / 8;                     // reads per destination vector
+  typedef v4u v4u_a4 __attribute__((aligned(4)));
+
+  const uint32_t tid = threadIdx.x;
+  // Row groups of one tile (its extent along the rows over what an item takes).
+  const uint32_t lht = a.lt0 - (RPI == 16 ? 4 : RPI == 8 ? 3 : 2);  // log2
+
+  // ---- per-thread tables (the same for every block) ----
+  uint32_t g1off[N1], l1off[N1];
+#pragma unroll
+  for (int i = 0; i < N1; ++i) {
+    const uint32_t idx = tid + i * kThreads;
+    const uint32_t r = idx / VPR, v = idx % VPR;
+    g1off[i] = r * (uint32_t)a.src_pitch + v * 16;
+    l1off[i] = r * a.lds_pitch + v * 16;
+  }
+  uint32_t l2addr[N2], g2off[N2], tl0[N2], tl1[N2];
+#pragma unroll
+  for (int i = 0; i < N2; ++i) {
+    const uint32_t idx = tid + i * kThreads;
+    const uint32_t l = idx & 15, item = idx >> 4;
+    // Items in the order (row group within the tile, column group, tile along
+    // the rows): the four items of a wave's instruction then store bytes that
+    // are neighbours in the destination wherever the tile shape allows.
+    const uint32_t h = item & ((1u << lht) - 1);
+    const uint32_t cg = (item >> lht) & (NCG - 1);
+    const uint32_t rgt = (item >> lht) / NCG;
+    const uint32_t r0 = ((rgt << lht) + h) * RPI;
+    // What this lane addresses for the item's reads.
+    l2addr[i] = (r0 + l / CH) * a.lds_pitch + (cg * 16 + (l % CH) * E) * EB;
+    // What it receives: column cg * 16 + l of rows r0 .. r0 + RPI - 1.
+    const uint32_t c = cg * 16 + l;
+    tl0[i] = r0 >> a.lt0;
+    tl1[i] = c >> a.lt1;
+    const uint32_t b0 = r0 & ((1u << a.lt0) - 1), b1 = c & ((1u << a.lt1) - 1);
+    g2off[i] = tl0[i] * (uint32_t)a.s0 + tl1[i] * (uint32_t)a.s1 + ((b1 << a.lt0) + b0) * EB;
+  }
+  const uint32_t tiles0 = kBlockRows >> a.lt0, tiles1 = BC >> a.lt1;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;  // LDS addresses are the low 32 bits
+
+  struct Block {
+    uint32_t blk0, blk1, row_base, col_base_bytes;
+    const char* src;
+    char* dst;
+    bool interior;
+  };
+  auto block_at = [&](uint32_t blk) {
+    Block b;
+    // Strips of `strip` block columns, each walked block row by block row.
+    const uint32_t per_strip = a.strip * a.nblk0;
+    const uint32_t st = blk / per_strip, rem = blk - st * per_strip;
+    const uint32_t width = min(a.strip, a.nblk1 - st * a.strip);
+    b.blk0 = rem / width;
+    b.blk1 = st * a.strip + (rem - b.blk0 * width);
+    b.row_base = b.blk0 * kBlockRows;
+    b.col_base_bytes = b.blk1 * kBlockRowBytes;
+    b.src = a.src + (int64_t)b.row_base * a.src_pitch + b.col_base_bytes;
+    b.dst = a.dst + (int64_t)(b.blk0 * tiles0) * a.s0 + (int64_t)(b.blk1 * tiles1) * a.s1;
+    b.interior = b.row_base + kBlockRows <= a.rows && b.col_base_bytes + kBlockRowBytes <= a.row_bytes &&
+                 (b.blk0 + 1) * tiles0 <= a.outer0 && (b.blk1 + 1) * tiles1 <= a.outer1;
+    return b;
+  };
+  v4u pre[N1];
+  auto prefetch = [&](const Block& b) {
+    if (b.interior) {
+#pragma unroll
+      for (int i = 0; i < N1; ++i) pre[i] = *reinterpret_cast<const v4u_a4*>(b.src + g1off[i]);
+      return;
+    }
+    // Edge block: vectors that lie wholly inside the matrix; the rest is dealt
+    // with when the block goes to LDS.
+#pragma unroll
+    for (int i = 0; i < N1; ++i) {
+      const uint32_t idx = tid + i * kThreads;
+      const uint32_t r = idx / VPR, cb = (idx % VPR) * 16;
+      if (b.row_base + r < a.rows && b.col_base_bytes + cb + 16 <= a.row_bytes)
+        pre[i] = *reinterpret_cast<const v4u_a4*>(b.src + g1off[i]);
+    }
+  };
+
+  const uint32_t nblocks = a.nblk0 * a.nblk1;
+  // Workgroups go to the eight XCDs round-robin; the workgroups of one XCD
+  // take consecutive blocks.
+  const uint32_t first_blk = (gridDim.x & 7) ? blockIdx.x
+                                             : (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (first_blk < nblocks) prefetch(block_at(first_blk));
+  uint32_t buf = 0;
+  for (uint32_t blk = first_blk; blk < nblocks; blk += gridDim.x, buf ^= 1) {
+    const Block b = block_at(blk);
+    char* lbuf = lds + buf * a.lds_buf_bytes;
+    // ---- matrix rows -> LDS ----
+    if (b.interior) {
+#pragma unroll
+      for (int i = 0; i < N1; ++i) *reinterpret_cast<v4u*>(lbuf + l1off[i]) = pre[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < N1; ++i) {
+        const uint32_t idx = tid + i * kThreads;
+        const uint32_t r = idx / VPR, cb = (idx % VPR) * 16;
+        const bool row_ok = b.row_base + r < a.rows;
+        v4u val;
+        if (row_ok && b.col_base_bytes + cb + 16 <= a.row_bytes) {
+          val = pre[i];
+        } else {
+          val = v4u{a.pad32, a.pad32, a.pad32, a.pad32};
+          if (row_ok && b.col_base_bytes + cb < a.row_bytes) {
+            // The row ends inside this vector: element by element.
+            __attribute__((aligned(16))) char reg[16];
+            *reinterpret_cast<v4u*>(reg) = val;
+            const char* gp = b.src + g1off[i];
+            const uint32_t left = a.row_bytes - (b.col_base_bytes + cb);
+            for (uint32_t bb = 0; bb + EB <= left && bb < 16; bb += EB) {
+              if constexpr (EB == 2) *reinterpret_cast<uint16_t*>(reg + bb) = *reinterpret_cast<const uint16_t*>(gp + bb);
+              else reg[bb] = gp[bb];
+            }
+            val = *reinterpret_cast<const v4u*>(reg);
+          }
+        }
+        *reinterpret_cast<v4u*>(lbuf + l1off[i]) = val;
+      }
+    }
+    if (blk + gridDim.x < nblocks) prefetch(block_at(blk + gridDim.x));
+    __syncthreads();
+
+    // ---- LDS, transposed -> tiles ----
+    const uint32_t lb = lds_base + buf * a.lds_buf_bytes;
+    v2u got[N2][R];
+#pragma unroll
+    for (int i = 0; i < N2; ++i)
+#pragma unroll
+      for (int h = 0; h < R; ++h) got[i][h] = read_tr<EB>(lb + l2addr[i] + (uint32_t)h * E * a.lds_pitch);
+    // The compiler does not count these reads: wait for them here, and tie the
+    // registers to the wait so that nothing uses them before it.
+#define UK_GOT(k) "+v"(got[(k) % N2][(k) / N2 % R])
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : UK_GOT(0), UK_GOT(1), UK_GOT(2), UK_GOT(3), UK_GOT(4), UK_GOT(5), UK_GOT(6), UK_GOT(7)
+                 :
+                 : "memory");
+#undef UK_GOT
+    static_assert(N2 * R == 8, "eight reads per thread and block");
+#pragma unroll
+    for (int i = 0; i < N2; ++i) {
+      if (!b.interior && !(b.blk0 * tiles0 + tl0[i] < a.outer0 && b.blk1 * tiles1 + tl1[i] < a.outer1)) continue;
+      char* gp = b.dst + g2off[i];
+      // Non-temporal stores: the tiles are written once, in whole lines over a
+      // few instructions, and not read again by this kernel (f16 4096 x 4096:
+      // 11.4 -> 9.4 us; s8 8192 x 28672: 97 -> 67 us).
+      if constexpr (V == 16) {
+        const v4u val = v4u{got[i][0][0], got[i][0][1], got[i][1][0], got[i][1][1]};
+        __builtin_nontemporal_store(val, reinterpret_cast<v4u*>(gp));
+      } else {
+        __builtin_nontemporal_store(got[i][0], reinterpret_cast<v2u*>(gp));
+      }
+    }
+    // No second barrier: the next block uses the other buffer, and its barrier
+    // orders this block's reads before that buffer is written again.
+  }
+}
+
+uint32_t log2_exact(int64_t x) {
+  uint32_t l = 0;
+  while ((1ll << l) < x) ++l;
+  return l;
+}
+bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+
+
+}  // namespace
+
+// Launches the transposing pack when it serves the call (true), else launches
+// nothing. `es`: bytes per element of the pack's type; src / dst with their
+// offsets applied.
+bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const char* src, char* dst,
+                                hipStream_t stream) {
+  const bool ti = p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
+  const bool to = p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_OUTER;
+  if (p->in_stride1 != 1 || p->in_stride0 < 0) return false;
+  // Element of the transposition and the tile's extents in such elements:
+  // t0 along the matrix rows, t1 along its columns.
+  int eb;
+  int64_t t0, t1, size1;
+  if (ti) {
+    if (es > 2) return false;
+    eb = es; t0 = p->out_size3; t1 = p->out_size2; size1 = p->in_size1;
+  } else {
+    // Tile rows of one or two bytes: the row is the element.
+    eb = (int)(p->out_size3 * es);
+    if (eb != 1 && eb != 2) return false;
+    if (p->in_size1 % p->out_size3 != 0) return false;  // (a last row of half padding)
+    t0 = p->out_size2; t1 = 1; size1 = p->in_size1 / p->out_size3;
+  }
+  const int64_t tile_bytes = t0 * t1 * eb;
+  const int64_t outer0 = to ? p->out_size1 : p->out_size0;  // tiles along the matrix rows
+  const int64_t outer1 = to ? p->out_size0 : p->out_size1;
+  const int64_t bc = kBlockRowBytes / eb;
+  if (!is_pow2(t0) || !is_pow2(t1) || t0 > kBlockRows || t1 > bc || (t0 * eb) % 8 != 0) return false;
+  const int V = (t0 * eb) % 16 == 0 ? 16 : 8;
+  const int64_t s_outer = p->out_stride0 * es;
+  const int64_t s0 = to ? tile_bytes : s_outer;
+  const int64_t s1 = to ? s_outer : tile_bytes;
+  const int64_t pitch = p->in_stride0 * es;
+  if (s_outer < 0) return false;
+  // Alignment: 4 bytes on the matrix side, the store width on the tiled side.
+  if (((uintptr_t)src | (uint64_t)pitch) & 3) return false;
+  if (((uintptr_t)dst | (uint64_t)s0 | (uint64_t)s1) & (uint64_t)(V - 1)) return false;
+  const int64_t tiles0 = kBlockRows / t0, tiles1 = bc / t1;
+  // 32-bit offsets inside a block, 32-bit sizes.
+  if (pitch * kBlockRows >= (1ll << 31) || tiles0 * s0 + tiles1 * s1 >= (1ll << 31)) return false;
+  if (p->in_size0 >= (1ll << 31) || size1 * eb >= (1ll << 31) || outer0 >= (1ll << 24) || outer1 >= (1ll << 24)) return false;
+  const int64_t nblk0 = uk::ceil_div(outer0, tiles0), nblk1 = uk::ceil_div(outer1, tiles1);
+  if (nblk0 * nblk1 >= (1ll << 31) || nblk0 * nblk1 == 0) return false;
+
+  TrArgs a;
+  a.src = src;
+  a.dst = dst;
+  a.src_pitch = pitch;
+  a.s0 = s0;
+  a.s1 = s1;
+  a.rows = (uint32_t)p->in_size0;
+  a.row_bytes = (uint32_t)(size1 * eb);
+  a.outer0 = (uint32_t)outer0;
+  a.outer1 = (uint32_t)outer1;
+  a.lt0 = log2_exact(t0);
+  a.lt1 = log2_exact(t1);
+  a.nblk0 = (uint32_t)nblk0;
+  a.nblk1 = (uint32_t)nblk1;
+  // Under TRANSPOSE_OUTER the tiles of one block column follow each other in
+  // the destination: the walk goes down the block columns.
+  a.strip = to ? 1u : (uint32_t)nblk1;
+  // Rows that the lanes of one read touch lie 16 (one-byte elements: 16 rows
+  // of 16 bytes per half wave) or 32 bytes apart modulo the 256 bytes of the banks.
+  a.lds_pitch = kBlockRowBytes + 16 * eb;
+  a.lds_buf_bytes = kBlockRows * a.lds_pitch;
+  uint64_t pad = p->padding_value & (es == 1 ? 0xFFull : 0xFFFFull);
+  a.pad32 = es == 1 ? (uint32_t)(pad * 0x01010101ull) : (uint32_t)(pad * 0x00010001ull);
+  const uint32_t nblocks = (uint32_t)(nblk0 * nblk1);
+  const size_t lds = 2 * (size_t)a.lds_buf_bytes;
+  const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
+  const dim3 block(kBlockRows * kBlockRowBytes / 64);
+  if (eb == 2 && V == 16) uk::launch(0, pack_tr_kernel<2, 16>, dim3(grid), block, lds, stream, a);
+  else if (eb == 2) uk::launch(0, pack_tr_kernel<2, 8>, dim3(grid), block, lds, stream, a);
+  else if (V == 16) uk::launch(0, pack_tr_kernel<1, 16>, dim3(grid), block, lds, stream, a);
+  else uk::launch(0, pack_tr_kernel<1, 8>, dim3(grid), block, lds, stream, a);
+  return true;
+}

@@ -1303,6 +1303,10 @@ int elem_bytes_of(uint32_t flags) {
 
 }  // namespace
 
+// pack_tr.hip: tiles transposed element by element, 1- and 2-byte elements.
+bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const char* src, char* dst,
+                                hipStream_t stream);
+
 extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
                                            void* stream_v, int kernel_mode,
                                            const char** kernel_name) {
@@ -1321,6 +1325,10 @@ extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
   if (kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO &&
       launch_pack_direct(p, es, src, dst, ti || to, stream)) {
     *kernel_name = "pack_direct";
+    return (int)hipGetLastError();
+  }
+  if (kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO && iree_uk_amd_launch_pack_tr(p, es, src, dst, stream)) {
+    *kernel_name = "pack_transposing";
     return (int)hipGetLastError();
   }
   if (kernel_mode != IREE_UK_AMD_KERNEL_MODE_GENERIC) {

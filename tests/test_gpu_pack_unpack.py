@@ -102,7 +102,7 @@ def test_pack_block_spanning_shapes(gpu, oracle, mode):
         G.run_pack_case(oracle, c, inp, want)
         got = T.gpu_pack(lib, torch, c, inp, out0)
         assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
-        tiled += lib.last_kernel_name() in ("pack_tiled", "pack_stream", "pack_direct")
+        tiled += lib.last_kernel_name() in ("pack_tiled", "pack_stream", "pack_direct", "pack_transposing")
     if mode == uk.KERNEL_MODE_AUTO:
         assert tiled >= 60, tiled  # the LDS-staged kernel is the one under test
     else:
@@ -165,6 +165,89 @@ def test_pack_direct_kernel_exact_untransposed_tilings(gpu, oracle, tf, t0, t1):
         assert np.array_equal(staged, want), c.label()
 
 
+# (type, stored tile shape out_size2 x out_size3, TRANSPOSE_INNER): element-wise
+# transpositions of 1- and 2-byte elements, and untransposed tiles whose rows
+# are one or two bytes (the reference's 16x2 s8 tile,
+# arch/x86_64/mmt4d_x86_64_tiles.inl).
+TRANSPOSING_TILES = [
+    (uk.PACK_TYPE_F16F16, 16, 16, True), (uk.PACK_TYPE_BF16BF16, 16, 8, True), (uk.PACK_TYPE_F16F16, 16, 4, True),
+    (uk.PACK_TYPE_F16F16, 32, 64, True), (uk.PACK_TYPE_F16F16, 1, 16, True), (uk.PACK_TYPE_BF16BF16, 128, 16, True),
+    (uk.PACK_TYPE_I8I8, 16, 8, True), (uk.PACK_TYPE_I8I8, 16, 16, True), (uk.PACK_TYPE_I8I8, 16, 32, True),
+    (uk.PACK_TYPE_I8I8, 8, 64, True), (uk.PACK_TYPE_I8I8, 256, 8, True), (uk.PACK_TYPE_I8I8, 2, 16, True),
+    (uk.PACK_TYPE_I8I8, 16, 2, False), (uk.PACK_TYPE_I8I8, 8, 2, False), (uk.PACK_TYPE_I8I8, 64, 2, False),
+    (uk.PACK_TYPE_I8I8, 16, 1, False), (uk.PACK_TYPE_I8I8, 8, 1, False),
+    (uk.PACK_TYPE_F16F16, 16, 1, False), (uk.PACK_TYPE_BF16BF16, 4, 1, False),
+]
+
+
+def _transposing_cases(tf, s2, s3, ti):
+    """Matrix shapes around the kernel's 64-row x 256-byte blocks: one block and
+    less, several with ragged edges in both directions, tile grids larger than
+    the matrix (tiles of nothing but padding), both outer orders, loose pitches
+    and offsets that keep the alignment the kernel asks for (4 bytes on the
+    matrix side, 16 on the tiled side)."""
+    es = uk.PACK_TYPE_BYTES[tf]
+    a0, a1 = (s3, s2) if ti else (s2, s3)    # tile extent along matrix rows / columns
+    g = T.Lcg(1234 + s2 * 7 + s3)
+    even = 2 if (not ti and s3 == 2) else 1  # (whole two-byte tile rows)
+    for (in0, in1, extra) in ((5, 6, 0), (64, 256 // es, 0), (67, 2 * (256 // es) + 10, 0), (200, 130, 1),
+                              (129, 700, 0), (3 * 64, 3 * (256 // es), 2)):
+        in1 = -(-in1 // even) * even
+        for to in (0, 1):
+            for variant in range(2):
+                o0 = -(-in0 // a0) + extra
+                o1 = -(-in1 // a1) + (extra + 1) // 2
+                os0, os1 = (o1, o0) if to else (o0, o1)
+                flags = tf | (0x100 if ti else 0) | (0x200 if to else 0)
+                unit = 16 // es
+                yield T.PackCase(flags, in0, in1, os0, os1, s2, s3,
+                                 -(-in1 // 4) * 4 + (0, 4 * 3)[variant], 1,
+                                 os1 * s2 * s3 + (0, unit * 3)[variant],
+                                 (0, 4 * 5)[variant], (0, unit * 2)[variant], g.u64())
+
+
+@pytest.mark.parametrize("tile", TRANSPOSING_TILES, ids=lambda t: f"type{t[0]}_{t[1]}x{t[2]}_{'ti' if t[3] else 'rows'}")
+def test_pack_transposing_kernel(gpu, oracle, tile):
+    """The kernel built on the LDS transposing reads: whole output buffers
+    against the oracle, and the LDS-staged kernels on the same calls."""
+    lib, torch = gpu
+    tf, s2, s3, ti = tile
+    for ci, c in enumerate(_transposing_cases(tf, s2, s3, ti)):
+        rng = np.random.default_rng(8000 + ci)
+        inp, out0 = T.make_pack_buffers(c, rng)
+        want = out0.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+        got = T.gpu_pack(lib, torch, c, inp, out0)
+        assert lib.last_kernel_name() == "pack_transposing", (c.label(), lib.last_kernel_name())
+        assert np.array_equal(got, want), c.label()
+        lib.set_kernel_mode(uk.KERNEL_MODE_MFMA_VARIANT + 1)   # keeps pack on the LDS-staged kernels
+        try:
+            staged = T.gpu_pack(lib, torch, c, inp, out0)
+            assert lib.last_kernel_name() in ("pack_stream", "pack_tiled"), lib.last_kernel_name()
+        finally:
+            lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+        assert np.array_equal(staged, want), c.label()
+
+
+def test_pack_transposing_kernel_declines_what_it_does_not_serve(gpu, oracle):
+    """Rows that are only 2-byte aligned, tile extents that are not powers of
+    two, an odd number of columns under two-byte tile rows: other kernels, same
+    bytes."""
+    lib, torch = gpu
+    cases = [T.PackCase(uk.PACK_TYPE_F16F16 | 0x100, 70, 131, 5, 9, 16, 16, 131, 1, 9 * 256, 0, 0, 7),
+             T.PackCase(uk.PACK_TYPE_I8I8 | 0x100, 70, 130, 6, 6, 24, 12, 132, 1, 6 * 288, 0, 0, 7),
+             T.PackCase(uk.PACK_TYPE_I8I8, 70, 131, 5, 66, 16, 2, 132, 1, 66 * 32, 0, 0, 7),
+             T.PackCase(uk.PACK_TYPE_F32F32 | 0x100, 70, 130, 9, 9, 16, 8, 132, 1, 9 * 128, 0, 0, 7)]
+    for ci, c in enumerate(cases):
+        inp, out0 = T.make_pack_buffers(c, np.random.default_rng(ci))
+        want = out0.copy()
+        G.run_pack_case(oracle, c, inp, want)
+        got = T.gpu_pack(lib, torch, c, inp, out0)
+        assert lib.last_kernel_name() != "pack_transposing", c.label()
+        assert np.array_equal(got, want), c.label()
+
+
 def test_pack_unpack_round_trip_and_numpy_identity(gpu):
     """Size-independent properties at a size the oracle would be slow on:
     pack == pad+reshape+transpose, unpack(pack(x)) == x."""
@@ -187,7 +270,7 @@ def test_pack_unpack_round_trip_and_numpy_identity(gpu):
         flags = tf | (0x100 if ti else 0) | (0x200 if to else 0)
         lib.pack(d_x.data_ptr(), 0, shape[1], 1, d_p.data_ptr(), 0, o1 * o2 * o3,
                  o2 * o3, shape[0], shape[1], o0, o1, o2, o3, pad_bits, flags)
-        assert lib.last_kernel_name() in ("pack_stream", "pack_tiled", "pack_direct")
+        assert lib.last_kernel_name() in ("pack_stream", "pack_tiled", "pack_direct", "pack_transposing")
         got4 = d_p.cpu().numpy().view(dtype).reshape(want4.shape)
         assert np.array_equal(got4, want4)
         d_y = torch.full((x.size * x.itemsize,), 0x5A, dtype=torch.uint8, device="cuda")
