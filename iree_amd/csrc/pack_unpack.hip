@@ -161,6 +161,7 @@ struct TiledArgs {
   uint32_t lds_buf_bytes;           // one LDS buffer of the streaming kernels
   uint32_t mat_stride0_bytes32;     // == mat_stride0_bytes when it fits
   uint32_t sl0_bytes32, sl1_bytes32;
+  uint32_t streaming_stores;        // 16 KB-block streaming kernels: non-temporal stores
 };
 
 template <int N> struct Bytes;
@@ -467,6 +468,16 @@ __device__ __forceinline__ void gstore(char* gptr, typename GBytes<N>::type v) {
   else *reinterpret_cast<T4*>(gptr) = v;
 }
 
+// The non-temporal store chosen at run time, as assembly: beside a plain
+// store of the same value to the same address in the other branch, the
+// compiler merges the two into one plain store.
+template <int N>
+__device__ __forceinline__ void gstore_nt_asm(char* gptr, typename GBytes<N>::type v) {
+  if constexpr (N == 16) asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(gptr), "v"(v) : "memory");
+  else if constexpr (N == 8) asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(gptr), "v"(v) : "memory");
+  else asm volatile("global_store_dword %0, %1, off nt" : : "v"(gptr), "v"(v) : "memory");
+}
+
 constexpr uint32_t kStreamBlockBytes = 16384;     // matrix bytes per block, streaming kernels
 constexpr uint32_t kStreamBigBlockBytes = 65536;  // same, large transposing problems
 
@@ -620,6 +631,19 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
   using TileVec = typename GBytes<VEC>::type;
   static_assert(G >= 4, "streaming kernels move granules of at least 4 bytes");
 
+  // Non-temporal in the 64 KB-block kernels, and in the others when the host
+  // asks for it (outputs beyond the memory-side cache).
+  const bool nt_stores = kStreamingStores || a.streaming_stores;
+  auto store_tiled = [&](char* p, TileVec v) {
+    if constexpr (kStreamingStores) gstore<VEC, true>(p, v);
+    else if (nt_stores) gstore_nt_asm<VEC>(p, v);
+    else gstore<VEC, false>(p, v);
+  };
+  auto store_mat = [&](char* p, MatVec v) {
+    if constexpr (kStreamingStores) gstore<MV, true>(p, v);
+    else if (nt_stores) gstore_nt_asm<MV>(p, v);
+    else gstore<MV, false>(p, v);
+  };
   const uint32_t tid = threadIdx.x;
   const uint32_t total1 = a.block_rows * a.div_row_vecs.d;
   const uint32_t total2 = a.num_runs * a.run_vecs;
@@ -866,7 +890,7 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
 #pragma unroll
         for (int i = 0; i < N2; ++i) reg[i] = gather_granules<VEC, G>(lbuf, l2off[i], rot);
 #pragma unroll
-        for (int i = 0; i < N2; ++i) gstore<VEC, kStreamingStores>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
+        for (int i = 0; i < N2; ++i) store_tiled(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
         return;
       }
 #pragma unroll
@@ -882,7 +906,7 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
             tiled_item<VEC>(a, tid + i * NT, &run, &t, &in_tile, &tl0, &tl1);
             ok = blk0 * a.G0 + tl0 < a.outer0 && blk1 * a.G1 + tl1 < a.outer1;
           }
-          if (ok) gstore<VEC, kStreamingStores>(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
+          if (ok) store_tiled(const_cast<char*>(tiled_c) + g2off[i], reg[i]);
         }
       }
     } else {
@@ -895,7 +919,7 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
           for (int i = 0; i < N1; ++i) reg[i] = lds_load_static<MV, P>(lbuf + l1off[i]);
         });
 #pragma unroll
-        for (int i = 0; i < N1; ++i) gstore<MV, kStreamingStores>(const_cast<char*>(mat_c) + g1off[i], reg[i]);
+        for (int i = 0; i < N1; ++i) store_mat(const_cast<char*>(mat_c) + g1off[i], reg[i]);
       } else if (interior) {
         MatVec reg[N1];
 #pragma unroll
@@ -903,7 +927,7 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
           if (tid + i * NT < total1) reg[i] = lds_load_pieces<MV>(lbuf + l1off[i], piece);
 #pragma unroll
         for (int i = 0; i < N1; ++i)
-          if (tid + i * NT < total1) gstore<MV, kStreamingStores>(const_cast<char*>(mat_c) + g1off[i], reg[i]);
+          if (tid + i * NT < total1) store_mat(const_cast<char*>(mat_c) + g1off[i], reg[i]);
       } else {
         const uint32_t es = a.elem_bytes;
         for (uint32_t idx = tid; idx < total1; idx += NT) {
@@ -912,7 +936,7 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
           if (row_base + r >= a.mat_size0) continue;
           char* gp = const_cast<char*>(mat_c) + (r * a.mat_stride0_bytes32 + cb);
           if (col_base_bytes + cb + MV <= size1_bytes) {  // whole vector inside
-            gstore<MV, kStreamingStores>(gp, lds_load_pieces<MV>(lbuf + r * a.lds_pitch + cb, piece));
+            store_mat(gp, lds_load_pieces<MV>(lbuf + r * a.lds_pitch + cb, piece));
             continue;
           }
           __attribute__((aligned(16))) char reg[MV];
@@ -1118,6 +1142,11 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
                       ti, to, mat_is_dest, false);
   }
   plan.big = big;
+  // Outputs beyond the memory-side cache are not worth allocating there: the
+  // interior blocks of the 16 KB-block kernels store them non-temporally too
+  // (f32 8192x8192 unpack under TRANSPOSE_OUTER: 106 -> 77 us). Below that
+  // size the plain stores are as fast or faster.
+  a.streaming_stores = total_bytes >= (192ll << 20) && uk::pow2_divisor(mat_stride0 * es, 16) >= 16;
   if (plan.stream) {
     a.mat_vec = (uint32_t)plan.MV;
     a.div_row_vecs = FastDiv((uint32_t)(block_row_bytes / plan.MV));
