@@ -51,6 +51,7 @@ struct TrArgs {
   uint32_t lt0, lt1;        // log2 of the tile's extent along rows / columns, elements
   uint32_t nblk0, nblk1;    // blocks along rows / columns
   uint32_t strip;           // block columns per strip of the walk
+  uint32_t down;            // TRANSPOSE_OUTER: tiles that follow each other down the rows are neighbours
   uint32_t lds_pitch;       // bytes per LDS row
   uint32_t lds_buf_bytes;
   uint32_t pad32;           // the padding element replicated over 32 bits
@@ -68,9 +69,16 @@ __device__ __forceinline__ v2u read_tr(uint32_t lds_addr) {
 }
 
 // EB: bytes per transposed element. V: bytes a lane stores at once (16 where
-// the tile's extent along the rows is a multiple of 16 bytes, else 8).
-template <int EB, int V>
+// the tile's extent along the rows is a multiple of 16 bytes, else 8). IL: 0,
+// or the tile's extent along the rows where that is less than eight bytes (2
+// or 4 elements: the K0 = 2 tiles of the reference's x86 kernels from a
+// row-major [K][N] operand). A lane's 16 destination bytes are then 16 / IL
+// bytes of each of IL neighbouring rows, read as they lie and interleaved in
+// registers (v_perm_b32); neighbouring lanes take neighbouring columns, which
+// are neighbours in the tile.
+template <int EB, int V, int IL = 0>
 __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kernel(TrArgs a) {
+  static_assert(IL == 0 || (V == 16 && (IL * EB == 2 || IL * EB == 4)), "interleaved rows of 2 or 4 bytes");
   constexpr int kThreads = kBlockRows * kBlockRowBytes / 64;  // 64 bytes of the block per thread
   constexpr int kBlockBytes = kBlockRows * kBlockRowBytes;
   constexpr int VPR = kBlockRowBytes / 16;     // 16-byte vectors per block row
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kern
 
   const uint32_t tid = threadIdx.x;
   // Row groups of one tile (its extent along the rows over what an item takes).
-  const uint32_t lht = a.lt0 - (RPI == 16 ? 4 : RPI == 8 ? 3 : 2);  // log2
+  const uint32_t lht = IL ? 0 : a.lt0 - (RPI == 16 ? 4 : RPI == 8 ? 3 : 2);  // log2
 
   // ---- per-thread tables (the same for every block) ----
   uint32_t g1off[N1], l1off[N1];
@@ -102,13 +110,36 @@ __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kern
 #pragma unroll
   for (int i = 0; i < N2; ++i) {
     const uint32_t idx = tid + i * kThreads;
+    if constexpr (IL != 0) {
+      // Vector idx of the block: 16 / (IL * EB) columns of one tile row
+      // extent, columns first.
+      constexpr uint32_t CPV = 16 / (IL * EB), VPT = BC / CPV;
+      uint32_t rt = idx / VPT, c = (idx % VPT) * CPV;
+      if (a.down) {
+        // the vectors of a tile, then the tiles down the rows, then the next column of tiles
+        const uint32_t vpt = (1u << a.lt1) / CPV, v = idx % vpt, t = idx / vpt;
+        rt = t % (kBlockRows / IL);
+        c = (t / (kBlockRows / IL) * vpt + v) * CPV;
+      }
+      l2addr[i] = rt * IL * a.lds_pitch + c * EB;
+      tl0[i] = rt;
+      tl1[i] = c >> a.lt1;
+      g2off[i] = tl0[i] * (uint32_t)a.s0 + tl1[i] * (uint32_t)a.s1 + (c & ((1u << a.lt1) - 1)) * IL * EB;
+      continue;
+    }
     const uint32_t l = idx & 15, item = idx >> 4;
     // Items in the order (row group within the tile, column group, tile along
     // the rows): the four items of a wave's instruction then store bytes that
     // are neighbours in the destination wherever the tile shape allows.
     const uint32_t h = item & ((1u << lht) - 1);
-    const uint32_t cg = (item >> lht) & (NCG - 1);
-    const uint32_t rgt = (item >> lht) / NCG;
+    uint32_t cg = (item >> lht) & (NCG - 1);
+    uint32_t rgt = (item >> lht) / NCG;
+    if (a.down) {
+      // (row group within the tile, tile down the rows, column group)
+      const uint32_t tr = kBlockRows >> a.lt0;
+      rgt = (item >> lht) % tr;
+      cg = (item >> lht) / tr;
+    }
     const uint32_t r0 = ((rgt << lht) + h) * RPI;
     // What this lane addresses for the item's reads.
     l2addr[i] = (r0 + l / CH) * a.lds_pitch + (cg * 16 + (l % CH) * E) * EB;
@@ -206,6 +237,39 @@ __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kern
     if (blk + gridDim.x < nblocks) prefetch(block_at(blk + gridDim.x));
     __syncthreads();
 
+    if constexpr (IL != 0) {
+      // ---- LDS rows, interleaved -> tiles ----
+      v4u out[N2];
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        const char* lp = lbuf + l2addr[i];
+        if constexpr (IL == 2) {
+          const v2u r0 = *reinterpret_cast<const v2u*>(lp);
+          const v2u r1 = *reinterpret_cast<const v2u*>(lp + a.lds_pitch);
+          constexpr uint32_t kLo = EB == 2 ? 0x05040100u : 0x05010400u;  // elements 0 (and 1) of both rows
+          constexpr uint32_t kHi = EB == 2 ? 0x07060302u : 0x07030602u;
+          out[i] = v4u{__builtin_amdgcn_perm(r1[0], r0[0], kLo), __builtin_amdgcn_perm(r1[0], r0[0], kHi),
+                       __builtin_amdgcn_perm(r1[1], r0[1], kLo), __builtin_amdgcn_perm(r1[1], r0[1], kHi)};
+        } else {
+          uint32_t r[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) r[j] = *reinterpret_cast<const uint32_t*>(lp + j * a.lds_pitch);
+          // bytes (c, row): pairs of rows first, then pairs of pairs
+          const uint32_t a01 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);  // c0r0 c0r1 c1r0 c1r1
+          const uint32_t b01 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);  // c2r0 c2r1 c3r0 c3r1
+          const uint32_t a23 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+          const uint32_t b23 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+          out[i] = v4u{__builtin_amdgcn_perm(a23, a01, 0x05040100u), __builtin_amdgcn_perm(a23, a01, 0x07060302u),
+                       __builtin_amdgcn_perm(b23, b01, 0x05040100u), __builtin_amdgcn_perm(b23, b01, 0x07060302u)};
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        if (!b.interior && !(b.blk0 * tiles0 + tl0[i] < a.outer0 && b.blk1 * tiles1 + tl1[i] < a.outer1)) continue;
+        __builtin_nontemporal_store(out[i], reinterpret_cast<v4u*>(b.dst + g2off[i]));
+      }
+      continue;
+    }
     // ---- LDS, transposed -> tiles ----
     const uint32_t lb = lds_base + buf * a.lds_buf_bytes;
     v2u got[N2][R];
@@ -277,8 +341,12 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
   const int64_t outer0 = to ? p->out_size1 : p->out_size0;  // tiles along the matrix rows
   const int64_t outer1 = to ? p->out_size0 : p->out_size1;
   const int64_t bc = kBlockRowBytes / eb;
-  if (!is_pow2(t0) || !is_pow2(t1) || t0 > kBlockRows || t1 > bc || (t0 * eb) % 8 != 0) return false;
-  const int V = (t0 * eb) % 16 == 0 ? 16 : 8;
+  if (!is_pow2(t0) || !is_pow2(t1) || t0 > kBlockRows || t1 > bc) return false;
+  // Tiles less than eight bytes tall: rows interleaved in registers, a vector
+  // of 16 / (t0 * eb) columns inside one tile.
+  const int il = (t0 * eb == 2 || t0 * eb == 4) && t0 > 1 ? (int)t0 : 0;
+  if (il ? t1 * t0 * eb < 16 : (t0 * eb) % 8 != 0) return false;
+  const int V = il || (t0 * eb) % 16 == 0 ? 16 : 8;
   const int64_t s_outer = p->out_stride0 * es;
   const int64_t s0 = to ? tile_bytes : s_outer;
   const int64_t s1 = to ? s_outer : tile_bytes;
@@ -311,6 +379,7 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
   // Under TRANSPOSE_OUTER the tiles of one block column follow each other in
   // the destination: the walk goes down the block columns.
   a.strip = to ? 1u : (uint32_t)nblk1;
+  a.down = to ? 1u : 0u;
   // Rows that the lanes of one read touch lie 16 (one-byte elements: 16 rows
   // of 16 bytes per half wave) or 32 bytes apart modulo the 256 bytes of the banks.
   a.lds_pitch = kBlockRowBytes + 16 * eb;
@@ -321,6 +390,12 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
   const size_t lds = 2 * (size_t)a.lds_buf_bytes;
   const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
   const dim3 block(kBlockRows * kBlockRowBytes / 64);
+  if (il) {
+    if (eb == 2) uk::launch(0, pack_tr_kernel<2, 16, 2>, dim3(grid), block, lds, stream, a);
+    else if (il == 2) uk::launch(0, pack_tr_kernel<1, 16, 2>, dim3(grid), block, lds, stream, a);
+    else uk::launch(0, pack_tr_kernel<1, 16, 4>, dim3(grid), block, lds, stream, a);
+    return true;
+  }
   if (eb == 2 && V == 16) uk::launch(0, pack_tr_kernel<2, 16>, dim3(grid), block, lds, stream, a);
   else if (eb == 2) uk::launch(0, pack_tr_kernel<2, 8>, dim3(grid), block, lds, stream, a);
   else if (V == 16) uk::launch(0, pack_tr_kernel<1, 16>, dim3(grid), block, lds, stream, a);

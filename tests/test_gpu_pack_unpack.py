@@ -177,6 +177,10 @@ TRANSPOSING_TILES = [
     (uk.PACK_TYPE_I8I8, 16, 2, False), (uk.PACK_TYPE_I8I8, 8, 2, False), (uk.PACK_TYPE_I8I8, 64, 2, False),
     (uk.PACK_TYPE_I8I8, 16, 1, False), (uk.PACK_TYPE_I8I8, 8, 1, False),
     (uk.PACK_TYPE_F16F16, 16, 1, False), (uk.PACK_TYPE_BF16BF16, 4, 1, False),
+    # transposed tiles less than eight bytes tall (K0 = 2 and 4 from a row-major [K][N] operand)
+    (uk.PACK_TYPE_I8I8, 16, 2, True), (uk.PACK_TYPE_I8I8, 16, 4, True), (uk.PACK_TYPE_BF16BF16, 16, 2, True),
+    (uk.PACK_TYPE_I8I8, 8, 2, True), (uk.PACK_TYPE_F16F16, 8, 2, True), (uk.PACK_TYPE_I8I8, 4, 4, True),
+    (uk.PACK_TYPE_I8I8, 256, 2, True),
 ]
 
 
