@@ -37,7 +37,7 @@ EXTRA_WORKLOADS = [
     "c4_f8_prefill",
     "bf16_mmt4d_8192_k2", "bf16_mmt4d_8192_k8", "f8_mmt4d_8192_k32", "f32_mmt4d_4096_k1",
     "f32_mmt4d_4096_k4", "s16_mmt4d_4096_k2",
-    "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288",
+    "c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288", "pack_operand_forms",
     "conv_nchwc_f32_n16_56x56_c256_k256_3x3",
 ]
 
@@ -486,6 +486,18 @@ def main() -> int:
                 if "back" in keep:
                     entry["parity"] = {"round_trip_bit_exact": bool(
                         torch.equal(keep["back"].view(keep["rows"], keep["cols"]), keep["x"]))}
+            if name == "pack_operand_forms":
+                # every packed operand against the same regrouping written with
+                # torch's reshape and permute, bit for bit
+                ok = {}
+                for oname, x, out, X0, K0, kn in w.keep["forms"]:
+                    rows, cols = x.shape
+                    if kn:
+                        want = x.view(rows // K0, K0, cols // X0, X0).permute(2, 0, 3, 1)
+                    else:
+                        want = x.view(rows // X0, X0, cols // K0, K0).permute(0, 2, 1, 3)
+                    ok[oname] = bool(torch.equal(out.view(want.shape), want.contiguous()))
+                entry["parity"] = {"equals_reshape_permute": ok, "ok": all(ok.values())}
             extra[name] = entry
             del w
         result["extra"] = extra

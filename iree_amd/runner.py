@@ -456,6 +456,47 @@ class Runner:
                             "tiles k0=16 c0=16", [op], flops, nbytes, "f32",
                             dict(x=x, w=w, y=y, N=N, ICo=ICo, OCo=OCo, OH=OH, OW=OW, FH=FH, FW=FW,
                                  k0=k0, c0=c0))
+        if name == "pack_operand_forms":
+            # Matmul operands on their way into tiles, in the forms that need an
+            # element-wise transposition: the row-major [K][N] right-hand side
+            # (TRANSPOSE_INNER + TRANSPOSE_OUTER -> [N1][K1][N0][K0],
+            # tests/e2e/linalg/pack_i8.mlir:48-68) for the tile shapes of the
+            # other workloads, and the reference's 16x2 s8 tile from [M][K].
+            # Every form moves more than the 256 MB memory-side cache holds, so
+            # that repeated launches time HBM and not that cache.
+            forms = [  # (op name, torch dtype, pack type, element bytes, rows, cols, N0 or M0, K0, [K][N]?)
+                ("rhs_kn_f16_16x16", torch.float16, uk.PACK_TYPE_F16F16, 2, 8192, 16384, 16, 16, True),
+                ("rhs_kn_s8_16x8", torch.int8, uk.PACK_TYPE_I8I8, 1, 8192, 28672, 16, 8, True),
+                ("rhs_kn_f8_16x32", torch.int8, uk.PACK_TYPE_I8I8, 1, 8192, 28672, 16, 32, True),
+                ("rhs_kn_s8_16x16", torch.int8, uk.PACK_TYPE_I8I8, 1, 16384, 16384, 16, 16, True),
+                ("rhs_kn_s8_16x2", torch.int8, uk.PACK_TYPE_I8I8, 1, 16384, 16384, 16, 2, True),
+                ("rhs_kn_bf16_16x2", torch.bfloat16, uk.PACK_TYPE_BF16BF16, 2, 8192, 16384, 16, 2, True),
+                ("lhs_mk_s8_16x2", torch.int8, uk.PACK_TYPE_I8I8, 1, 16384, 16384, 16, 2, False),
+            ]
+            ops, keep = [], {"forms": []}
+            lib = self.lib
+            for i, (oname, dt, tf, es, rows, cols, X0, K0, kn) in enumerate(forms):
+                if dt == torch.int8:
+                    x = self.uniform_s8((rows, cols), 40 + i)
+                else:
+                    x = self.normal((rows, cols), dt, 40 + i)
+                out = self.empty(rows * cols, dt)
+                if kn:     # rows run along K, columns along N
+                    flags = tf | uk.PACK_TRANSPOSE_INNER | uk.PACK_TRANSPOSE_OUTER
+                    o0, o1 = cols // X0, rows // K0
+                else:      # rows along M, columns along K
+                    flags = tf
+                    o0, o1 = rows // X0, cols // K0
+
+                def launch(xp=x.data_ptr(), op_=out.data_ptr(), rows=rows, cols=cols, o0=o0, o1=o1,
+                           X0=X0, K0=K0, flags=flags):
+                    lib.pack(xp, 0, cols, 1, op_, 0, o1 * X0 * K0, X0 * K0, rows, cols, o0, o1, X0, K0,
+                             0, flags)
+                ops.append(Op(oname, launch, 0.0, float(2 * rows * cols * es), "hbm"))
+                keep["forms"].append((oname, x, out, X0, K0, kn))
+            return Workload(name, "pack of matmul operands that need an element-wise transposition: row-major "
+                            "[K][N] right-hand sides (TRANSPOSE_INNER + TRANSPOSE_OUTER) and the 16x2 s8 tile",
+                            ops, 0.0, sum(o.bytes for o in ops), "u8", keep)
         if name in ("c5_pack_f32_12288x12289", "c5_pack_f32_12289x12288"):
             rows, cols = (12288, 12289) if name.endswith("12289") else (12289, 12288)
             x = self.normal((rows, cols), torch.float32, 12)
