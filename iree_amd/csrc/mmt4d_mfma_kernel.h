@@ -95,6 +95,12 @@ struct Out32 {
   typedef Acc Acc4 __attribute__((aligned(4)));
   static __device__ __forceinline__ Acc load4(const char* p) { return *reinterpret_cast<const Acc4*>(p); }
   static __device__ __forceinline__ void store4(char* p, Acc v) { *reinterpret_cast<Acc4*>(p) = v; }
+  // The non-temporal form, chosen at run time (Args::nt_out). As assembly:
+  // beside the plain store of the same value in the other branch the compiler
+  // would merge the two into one plain store.
+  static __device__ __forceinline__ void store4_nt(char* p, Acc v) {
+    asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(p), "v"(v) : "memory");
+  }
   static __device__ __forceinline__ T load1(const char* p) { return *reinterpret_cast<const T*>(p); }
   static __device__ __forceinline__ void store1(char* p, T v) { *reinterpret_cast<T*>(p) = v; }
 };
@@ -110,6 +116,12 @@ struct Out16 {
   static __device__ __forceinline__ void store4(char* p, v4f v) {
     *reinterpret_cast<v4u16*>(p) = v4u16{uk::f32_to_small16<EB>(v[0]), uk::f32_to_small16<EB>(v[1]),
                                          uk::f32_to_small16<EB>(v[2]), uk::f32_to_small16<EB>(v[3])};
+  }
+  static __device__ __forceinline__ void store4_nt(char* p, v4f v) {
+    const v4u16 h = v4u16{uk::f32_to_small16<EB>(v[0]), uk::f32_to_small16<EB>(v[1]),
+                          uk::f32_to_small16<EB>(v[2]), uk::f32_to_small16<EB>(v[3])};
+    typedef uint32_t v2u32 __attribute__((ext_vector_type(2)));
+    asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(p), "v"(__builtin_bit_cast(v2u32, h)) : "memory");
   }
   static __device__ __forceinline__ float load1(const char* p) {
     return uk::small16_to_f32<EB>(*reinterpret_cast<const uint16_t*>(p));
@@ -253,6 +265,7 @@ struct Args {
   uint32_t tail;       // 1 when the last K step is partial
   uint32_t band;       // workgroup rows per rasterization band
   uint32_t vec_out;    // 1: 4 consecutive columns of a row are contiguous (and aligned enough)
+  uint32_t nt_out;     // 1: the final store of the accumulators is non-temporal (mmt4d_mfma_kernel.h only)
   // Where ACCUMULATE reads the initial accumulators: the same four-stride
   // addressing as the output. It is the output itself except in the first
   // launch of a dequantizing call, which reads a tiled accumulator buffer and
@@ -1491,8 +1504,15 @@ void mmt4d_mfma_kernel(Args a) {
       return;
     }
   }
+  // Outputs larger than the memory-side cache are stored non-temporally (s8
+  // 8192^3, 268 MB: 387-397 -> 377-385 us in the same process); smaller ones
+  // are not: whoever reads them next finds them in that cache (the f16 chain's
+  // step takes 3 us longer with non-temporal stores here, all of it in unpack).
   for_each_output(a.out, a.out_stride, a.out_sm0, a.out_spn,
-                  [&](int tm, int tn, char* p) { Out::store4(p, acc[tm][tn]); },
+                  [&](int tm, int tn, char* p) {
+                    if (a.nt_out) Out::store4_nt(p, acc[tm][tn]);
+                    else Out::store4(p, acc[tm][tn]);
+                  },
                   [&](int tm, int tn, int e, char* p) { Out::store1(p, acc[tm][tn][e]); });
 }
 

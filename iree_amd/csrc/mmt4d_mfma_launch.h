@@ -110,6 +110,10 @@ int launch_variant(const Problem& p, int kt_begin, int kt_count, bool accumulate
   };
   a.vec_out = vector_ok(p.out, p.out_stride, p.out_sm0, p.out_spn) &&
               (!accumulate || vector_ok(a.acc, a.acc_stride, a.acc_sm0, a.acc_spn));
+  // The launch that finishes K stores non-temporally when the output is
+  // larger than the memory-side cache can hand to its reader.
+  a.nt_out = kt_begin + kt_count == p.K1 &&
+             (int64_t)p.M1 * p.M0 * p.N1 * p.N0 * OB >= (192ll << 20);
   // 32-bit offsets inside a workgroup's share of each operand.
   const int64_t span_m = (int64_t)a.bpm * p.lhs_stride + (int64_t)p.K1 * kt_bytes_m;
   const int64_t span_n = (int64_t)a.bpn * p.rhs_stride + (int64_t)p.K1 * kt_bytes_n;
