@@ -454,10 +454,13 @@ template <> struct GBytes<16> { using type = v4u; };
 // Plain (cache-allocating) accesses on purpose: what pack writes is read by
 // mmt4d next, and what unpack reads was just written by mmt4d, so for operands
 // up to the size of the memory-side cache the hand-over never reaches HBM.
-template <int N>
+// STREAMING: a non-temporal load, for data that no later block and no later
+// kernel reads again (see TiledPlan::streaming_loads).
+template <int N, bool STREAMING = false>
 __device__ __forceinline__ typename GBytes<N>::type gload(const char* gptr) {
   typedef typename GBytes<N>::type T4 __attribute__((aligned(4)));
-  return *reinterpret_cast<const T4*>(gptr);
+  if constexpr (STREAMING) return __builtin_nontemporal_load(reinterpret_cast<const T4*>(gptr));
+  else return *reinterpret_cast<const T4*>(gptr);
 }
 // STREAMING: a non-temporal store, for the 64 KB-block kernels, whose output is
 // larger than the memory-side cache anyway (measured 3 % on a plain copy).
@@ -620,7 +623,7 @@ __device__ __forceinline__ bool with_static_piece(uint32_t piece, F f) {
   return false;
 }
 
-template <int G, int VEC, int MV, bool UNPACK, int BLK, int NT = kThreads, int DEPTH = 2>
+template <int G, int VEC, int MV, bool UNPACK, int BLK, int NT = kThreads, int DEPTH = 2, bool NTL = false>
 __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int N1 = BLK / MV / NT;   // 2-D side items per thread
@@ -760,10 +763,10 @@ __global__ __launch_bounds__(NT) void stream_tiled_kernel(TiledArgs a) {
     if (full) {
       if constexpr (!UNPACK) {
 #pragma unroll
-        for (int i = 0; i < N1; ++i) pre1[S][i] = gload<MV>(b.mat_c + g1off[i]);
+        for (int i = 0; i < N1; ++i) pre1[S][i] = gload<MV, NTL>(b.mat_c + g1off[i]);
       } else {
 #pragma unroll
-        for (int i = 0; i < N2; ++i) pre2[S][i] = gload<VEC>(b.tiled_c + g2off[i]);
+        for (int i = 0; i < N2; ++i) pre2[S][i] = gload<VEC, NTL>(b.tiled_c + g2off[i]);
       }
       return;
     }
@@ -977,6 +980,16 @@ struct TiledPlan {
   int G = 0, VEC = 0, MV = 0;
   bool stream = false;
   bool big = false;  // 64 KB blocks (see plan_tiled)
+  // 64 KB-block transposing kernels: interior blocks load non-temporally. The
+  // data is read once, and more of it than the caches hold: a line that is not
+  // kept leaves room for the lines that neighbouring blocks share. Right when
+  // no later block needs a line again, or only the next one in the walk: pack's
+  // row segments (their straddled lines are shared with the next block of the
+  // same block row), unpack's runs of tiles when they are whole 128-byte lines
+  // (f32 12289x12288: pack 248 -> 220 us; 12288x12289: unpack 255 -> 230 us;
+  // runs that start in the middle of a line share it with a block far away in
+  // the walk, and unpack lost 6 % there).
+  bool streaming_loads = false;
   uint32_t grid = 0;
   uint32_t lds_bytes = 0;
 };
@@ -1142,6 +1155,12 @@ TiledPlan plan_tiled(const TiledView& v, int es, const char* mat_ptr,
                       ti, to, mat_is_dest, false);
   }
   plan.big = big;
+  if (big && G == 4) {
+    // unpack: a run is (to ? G0 : G1) tiles, and runs lie (to ? sl1 : sl0) apart
+    const uint64_t run_bytes = (uint64_t)((to ? G0 : G1) * tile_bytes);
+    const uint64_t run_pitch = (uint64_t)((to ? v.sl1 : v.sl0) * es);
+    plan.streaming_loads = !mat_is_dest || ((uintptr_t)tiled_ptr | run_bytes | run_pitch) % 128 == 0;
+  }
   // Outputs beyond the memory-side cache are not worth allocating there: the
   // interior blocks of the 16 KB-block kernels store them non-temporally too
   // (f32 8192x8192 unpack under TRANSPOSE_OUTER: 106 -> 77 us). Below that
@@ -1207,6 +1226,12 @@ bool launch_stream(const TiledPlan& plan, hipStream_t stream) {
                  stream, plan.args);
       return true;
     };
+    if (plan.G == 4 && plan.streaming_loads) {
+      auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes, kBigThreads, 1, true>;
+      static hipError_t attr = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      return launch_big(kernel, attr);
+    }
     if (plan.G == 4) {
       auto kernel = stream_tiled_kernel<4, 16, 16, UNPACK, kStreamBigBlockBytes, kBigThreads, 1>;
       static hipError_t attr = hipFuncSetAttribute(
