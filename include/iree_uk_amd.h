@@ -435,8 +435,9 @@ IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_kernel_name(void);
  * pack / unpack that moves the same matrix between the same pitches.
  * *seconds_per_copy receives the average of the fastest of five ways of
  * writing the copy (1, 4 or 8 vectors in flight per lane, ordinary or
- * non-temporal stores, and one whose stores cover only whole 128-byte lines
- * of the destination whatever its pitch).
+ * non-temporal stores, non-temporal loads as well with 8 in flight, and one
+ * whose stores cover only whole 128-byte lines of the destination whatever
+ * its pitch).
  * iree_uk_amd_probe_copy2d_variants: the same, and seconds_per_variant[0..4]
  * (when not NULL) receive the average of every variant, the whole-line one
  * last. */

@@ -85,11 +85,11 @@ int run_mfma_peak(const v4i* operands, int n_operands, int iters, int workgroups
 // A workgroup copies 4 KiB pieces of rows (16 bytes per lane, 4-byte aligned
 // like the pack kernels' 2-D side), walking pieces grid-stride, DEPTH pieces
 // per turn: all loads of a turn are issued before its stores. NT: non-temporal
-// stores (the destination is not read again). LINES: the pieces of a row are
-// shifted so that every store of a wave covers whole 128-byte lines of the
+// stores (the destination is not read again). NTL: non-temporal loads too.
+// LINES: the pieces of a row are shifted so that every store of a wave covers whole 128-byte lines of the
 // destination whatever the pitch (one more, partial piece per row; the loads
 // are then the unaligned side).
-template <int DEPTH, bool NT, bool LINES = false>
+template <int DEPTH, bool NT, bool LINES = false, bool NTL = false>
 __global__ __launch_bounds__(256) void copy2d_kernel(const char* src, int64_t src_pitch, char* dst,
                                                      int64_t dst_pitch, int64_t row_bytes,
                                                      int64_t rows) {
@@ -115,7 +115,10 @@ __global__ __launch_bounds__(256) void copy2d_kernel(const char* src, int64_t sr
       so[d] = row * src_pitch + off;
       dof[d] = row * dst_pitch + off;
       whole[d] = p0 + d < total && off >= 0 && off + 16 <= row_bytes;
-      if (whole[d]) v[d] = *reinterpret_cast<const v4i_a4*>(src + so[d]);
+      if (whole[d]) {
+        if (NTL) v[d] = __builtin_nontemporal_load(reinterpret_cast<const v4i_a4*>(src + so[d]));
+        else v[d] = *reinterpret_cast<const v4i_a4*>(src + so[d]);
+      }
     }
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
@@ -283,7 +286,7 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_copy2d_variants(const void* src, int64_
       case 0: hipLaunchKernelGGL((copy2d_kernel<1, false>), dim3(cus * 8), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
       case 1: hipLaunchKernelGGL((copy2d_kernel<4, false>), dim3(cus * 4), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
       case 2: hipLaunchKernelGGL((copy2d_kernel<4, true>), dim3(cus * 4), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
-      case 3: hipLaunchKernelGGL((copy2d_kernel<8, true>), dim3(cus * 2), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
+      case 3: hipLaunchKernelGGL((copy2d_kernel<8, true, false, true>), dim3(cus * 2), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
       default: hipLaunchKernelGGL((copy2d_kernel<4, true, true>), dim3(cus * 4), dim3(256), 0, stream, s8, src_pitch, d8, dst_pitch, row_bytes, rows); break;
     }
   };
