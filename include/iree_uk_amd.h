@@ -404,6 +404,17 @@ IREE_UK_AMD_EXPORT int64_t iree_uk_amd_no_alloc_scratch_bytes(void);
 IREE_UK_AMD_EXPORT void iree_uk_amd_set_k_slices(int n);
 IREE_UK_AMD_EXPORT int iree_uk_amd_last_k_slices(void);
 
+/* A hint of the calling thread about where its weights are. 1: the wide
+ * operand of the decode-shaped (M-thin / N-thin) mmt4d calls that follow is
+ * read from HBM every time, as the layers of a model that evict each other
+ * from the caches are; such operands of 16 MB and more are then loaded
+ * non-temporally (58.7 MB of weights that no cache holds: 16.8 -> 15.4 us). 0,
+ * the default: ordinary loads, which are the faster ones when the same
+ * weights are used again while the 256 MB memory-side cache still holds
+ * them (12.3 against 14.3 us). Results are the same either way. No
+ * counterpart in the reference, whose callers have no such cache to manage. */
+IREE_UK_AMD_EXPORT void iree_uk_amd_set_streamed_weights(int on);
+
 /* Tuning / test knob of the calling thread: how many workgroups the
  * persistent mmt4d kernels launch (each walks its share of the output blocks
  * with one software pipeline running across block boundaries). 0, the

@@ -125,6 +125,7 @@ thread_local bool g_no_alloc = false;
 thread_local int g_k_slices = 0;
 thread_local int g_last_k_slices = 1;
 thread_local int g_persistent_workgroups = 0;
+thread_local bool g_streamed_weights = false;
 
 }  // namespace
 
@@ -132,6 +133,7 @@ namespace uk_mfma {
 
 int persistent_workgroups_override() { return g_persistent_workgroups; }
 int k_slices_override() { return g_k_slices; }
+int streamed_weights() { return g_streamed_weights ? 1 : 0; }
 void note_k_slices(int n) { g_last_k_slices = n; }
 
 int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStream_t stream,
@@ -216,6 +218,7 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
 extern "C" void iree_uk_amd_hip_set_no_alloc(int on) { g_no_alloc = on != 0; }
 
 extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_k_slices(int n) { g_k_slices = n > 0 ? n : 0; }
+extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_streamed_weights(int on) { g_streamed_weights = on != 0; }
 
 extern "C" IREE_UK_AMD_EXPORT int iree_uk_amd_last_k_slices(void) { return g_last_k_slices; }
 

@@ -154,6 +154,9 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
                              KSplitWorkspace* ws);
 // K slices set with iree_uk_amd_set_k_slices on this thread; 0 = choose.
 int k_slices_override();
+// 1: the calling thread has declared its weights streamed from HBM
+// (iree_uk_amd_set_streamed_weights).
+int streamed_weights();
 // Records the slice count of the launch for iree_uk_amd_last_k_slices.
 void note_k_slices(int n);
 
@@ -383,6 +386,13 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream, bool al
     } else {
       kslices = 1;
     }
+  }
+  // Weights that the caller has declared streamed, when they are too large for
+  // the L2s anyway: loaded non-temporally.
+  if (streamed_weights() && (int64_t)p.N1 * p.N0 * k_bytes / (S4 ? 2 : 1) >= (16ll << 20)) {
+    uk::launch(2, mmt4d_thin_kernel<E, RBC, TM, TN, KSPLIT, D, true>,
+               dim3((uint32_t)(grid_m * grid_n * kslices)), dim3(KSPLIT * 64), 0, stream, a);
+    return (int)hipGetLastError();
   }
   uk::launch(2, mmt4d_thin_kernel<E, RBC, TM, TN, KSPLIT, D>,
              dim3((uint32_t)(grid_m * grid_n * kslices)), dim3(KSPLIT * 64), 0, stream, a);

@@ -48,7 +48,11 @@ namespace uk_mfma {
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef v2i v2i_g __attribute__((aligned(1)));  // as v4i_g: read from global memory at any address
 
-template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
+// STREAMED: the wide operand (the kernel's RHS: weights) is loaded
+// non-temporally. For callers that say their weights come from HBM every time
+// (iree_uk_amd_set_streamed_weights): a layer's weights then pass through the
+// caches without displacing what is used again.
+template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D, bool STREAMED = false>
 __global__ __launch_bounds__(KSPLIT * 64)
 void mmt4d_thin_kernel(Args a) {
   using TT = ElemTraits<E>;
@@ -131,6 +135,17 @@ void mmt4d_thin_kernel(Args a) {
       return v4i{lo[0], lo[1], hi[0], hi[1]};
     }
   };
+  auto load_wide_operand = [&](const char* base, const uint32_t (&off)[PIECES], uint32_t adv) {
+    if constexpr (!STREAMED) {
+      return load_operand(base, off, adv);
+    } else if constexpr (RBC >= 16) {
+      return __builtin_nontemporal_load(reinterpret_cast<const v4i_g*>(base + (off[0] + adv)));
+    } else {
+      const v2i lo = __builtin_nontemporal_load(reinterpret_cast<const v2i_g*>(base + (off[0] + adv)));
+      const v2i hi = __builtin_nontemporal_load(reinterpret_cast<const v2i_g*>(base + (off[1] + adv)));
+      return v4i{lo[0], lo[1], hi[0], hi[1]};
+    }
+  };
   using BFrag = typename std::conditional<S4, v2i, v4i>::type;
   v4i fa[D][TM][HALVES];
   BFrag fb[D][TN][HALVES];
@@ -142,9 +157,11 @@ void mmt4d_thin_kernel(Args a) {
 #pragma unroll
       for (int h = 0; h < HALVES; ++h) {
         if constexpr (S4) {
-          fb[d][tn][h] = *reinterpret_cast<const v2i_g*>(base_b + (offb[tn][h][0] + s * sstep_b));
+          const v2i_g* pb = reinterpret_cast<const v2i_g*>(base_b + (offb[tn][h][0] + s * sstep_b));
+          if constexpr (STREAMED) fb[d][tn][h] = __builtin_nontemporal_load(pb);
+          else fb[d][tn][h] = *pb;
         } else {
-          fb[d][tn][h] = load_operand(base_b, offb[tn][h], s * sstep_b);
+          fb[d][tn][h] = load_wide_operand(base_b, offb[tn][h], s * sstep_b);
         }
       }
 #pragma unroll

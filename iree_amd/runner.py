@@ -400,20 +400,25 @@ class Runner:
 
                 def launch():
                     state["i"] = (state["i"] + 1) % COLD_COPIES
+                    lib.set_streamed_weights(True)   # what a serving loop says once per thread
                     lib.mmt4d_dequant_unpack(lp, 0, K1 * M0 * K0, rps[state["i"]], 0, K1 * N0 * K0,
                                              accp, 0, N1 * M0 * N0, yp, 0, N, Mlog, N,
                                              smp, snp, M1, N1, K1, M0, N0, K0, flags)
+                    lib.set_streamed_weights(False)
             else:
                 def launch():
                     state["i"] = (state["i"] + 1) % COLD_COPIES
+                    lib.set_streamed_weights(True)
                     lib.mmt4d(lp, 0, K1 * M0 * K0, rps[state["i"]], 0, K1 * N0 * K0, accp, 0,
                               N1 * M0 * N0, M1, N1, K1, M0, N0, K0, flags)
+                    lib.set_streamed_weights(False)
             src = base.ops[0]
             op = Op("mmt4d", launch, src.flops, src.bytes, "hbm", "s8")
             tensors = dict(t)
             tensors["weight_copies"] = copies
             return Workload(name, base.description + f"; weights rotate over {COLD_COPIES} copies "
-                            f"({COLD_COPIES * copies[0].numel() / 1e6:.0f} MB): every launch streams them from HBM",
+                            f"({COLD_COPIES * copies[0].numel() / 1e6:.0f} MB): every launch streams them from HBM, "
+                            "and says so (iree_uk_amd_set_streamed_weights)",
                             [op], base.flops, src.bytes, "s8", tensors)
         if name == "c4_f8_prefill":
             M, K, N = 2048, 8192, 28672

@@ -180,6 +180,8 @@ class UKernelLibrary:
         L.iree_uk_amd_no_alloc_scratch_bytes.restype = _i64
         L.iree_uk_amd_set_k_slices.argtypes = [ctypes.c_int]
         L.iree_uk_amd_set_k_slices.restype = None
+        L.iree_uk_amd_set_streamed_weights.argtypes = [ctypes.c_int]
+        L.iree_uk_amd_set_streamed_weights.restype = None
         L.iree_uk_amd_last_k_slices.restype = ctypes.c_int
         L.iree_uk_amd_mfma_decline_count.restype = ctypes.c_uint64
         L.iree_uk_amd_version.restype = ctypes.c_char_p
@@ -238,6 +240,11 @@ class UKernelLibrary:
         """K slices across workgroups of the thin mmt4d kernels on this thread
         (0 = choose, 1 = never split)."""
         self.lib.iree_uk_amd_set_k_slices(n)
+
+    def set_streamed_weights(self, on: bool):
+        """Hint of this thread: the weights of the decode-shaped mmt4d calls
+        that follow come from HBM every time (non-temporal loads)."""
+        self.lib.iree_uk_amd_set_streamed_weights(1 if on else 0)
 
     def last_k_slices(self) -> int:
         return int(self.lib.iree_uk_amd_last_k_slices())

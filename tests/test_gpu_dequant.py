@@ -190,21 +190,18 @@ def test_decode_layer_fused_equals_the_integer_product_scaled(gpu):
 def test_dequant_unpack_contract(lib):
     """Needs no device: a 16-bit out type, a matrix larger than the tiles and a
     missing accumulator buffer are contract violations; empty shapes return."""
-    lib.raise_on_violation(True)
-    try:
-        def call(flags, rows=16, cols=16, acc=None, M=1):
-            lib.mmt4d_dequant_unpack(None, 0, 0, None, 0, 0, acc, 0, 0, None, 0, cols, rows, cols,
-                                     None, None, M, 1, 1, 16, 16, 16, flags)
-        with pytest.raises(uk.ContractViolation):
-            call(uk.MMT4D_TYPE_F16F16F16 | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS)
-        with pytest.raises(uk.ContractViolation):
-            call(uk.MMT4D_TYPE_S8S8S32, rows=17)
-        with pytest.raises(uk.ContractViolation):
-            call(uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE)
-        call(uk.MMT4D_TYPE_S8S8S32, rows=0)
-        call(uk.MMT4D_TYPE_S8S8S32, rows=0, M=0)
-    finally:
-        lib.raise_on_violation(False)
+    lib.raise_on_violation(True)   # (the session's setting; left on)
+    def call(flags, rows=16, cols=16, acc=None, M=1):
+        lib.mmt4d_dequant_unpack(None, 0, 0, None, 0, 0, acc, 0, 0, None, 0, cols, rows, cols,
+                                 None, None, M, 1, 1, 16, 16, 16, flags)
+    with pytest.raises(uk.ContractViolation):
+        call(uk.MMT4D_TYPE_F16F16F16 | uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS)
+    with pytest.raises(uk.ContractViolation):
+        call(uk.MMT4D_TYPE_S8S8S32, rows=17)
+    with pytest.raises(uk.ContractViolation):
+        call(uk.MMT4D_TYPE_S8S8S32 | uk.MMT4D_ACCUMULATE)
+    call(uk.MMT4D_TYPE_S8S8S32, rows=0)
+    call(uk.MMT4D_TYPE_S8S8S32, rows=0, M=0)
 
 
 @pytest.mark.gpu

@@ -130,3 +130,51 @@ def test_k_slices_on_the_32_column_blocks(gpu, oracle):
         got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
         assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
         assert lib.last_kernel_name() == "mmt4d_mfma_thin" and lib.last_k_slices() == 2
+
+
+@pytest.mark.parametrize("n_thin", [False, True])
+@pytest.mark.parametrize("tf,M0,N0,K0", [(uk.MMT4D_TYPE_S8S8S32, 32, 16, 8), (uk.MMT4D_TYPE_S8S8S32, 16, 16, 16),
+                                         (uk.MMT4D_TYPE_F16F16F32, 16, 16, 16), (uk.MMT4D_TYPE_S8S4S32, 16, 16, 32)])
+def test_streamed_weights_hint_changes_no_result(gpu, tf, M0, N0, K0, n_thin):
+    """iree_uk_amd_set_streamed_weights: the decode-shaped kernels then load
+    weights of 16 MB and more non-temporally. Same bytes out as without the
+    hint, thin in M and thin in N (the transposed problem), with and without a
+    K split; and the hint is the calling thread's own, reset here."""
+    lib, torch = gpu
+    wide, K = 4608, 4096                      # 18.9 MB of 1-byte weights
+    if tf == uk.MMT4D_TYPE_S8S4S32:
+        wide *= 2                             # two elements per byte
+    if n_thin and tf == uk.MMT4D_TYPE_S8S4S32:
+        pytest.skip("the 4-bit operand is the right-hand side only")
+    lhs_es = {uk.MMT4D_TYPE_F16F16F32: 2}.get(tf, 1)
+    M1, N1 = (wide // M0, 1) if n_thin else (1, wide // N0)
+    K1 = K // K0
+    g = torch.Generator(device="cuda"); g.manual_seed(5)
+
+    def operand(rows_tiles, X0, packed_nibbles=False):
+        n = rows_tiles * K1 * X0 * K0
+        if lhs_es == 2:
+            return (torch.randint(-8, 8, (n,), generator=g, device="cuda", dtype=torch.int32)).to(torch.float16)
+        if packed_nibbles:
+            return torch.randint(-128, 128, (n // 2,), generator=g, device="cuda", dtype=torch.int8)
+        return torch.randint(-128, 128, (n,), generator=g, device="cuda", dtype=torch.int8)
+
+    lhs = operand(M1, M0)
+    rhs = operand(N1, N0, packed_nibbles=tf == uk.MMT4D_TYPE_S8S4S32)
+    out_dt = torch.float32 if lhs_es == 2 else torch.int32
+    outs = []
+    try:
+        for hint, slices in ((False, 0), (True, 0), (True, 1)):
+            lib.set_streamed_weights(hint)
+            lib.set_k_slices(slices)
+            out = torch.zeros(M1 * N1 * M0 * N0, device="cuda", dtype=out_dt)
+            lib.mmt4d(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, out.data_ptr(), 0,
+                      N1 * M0 * N0, M1, N1, K1, M0, N0, K0, tf | 0x200)
+            lib.synchronize()
+            assert lib.last_kernel_name().startswith("mmt4d_mfma_thin"), lib.last_kernel_name()
+            outs.append(out)
+    finally:
+        lib.set_streamed_weights(False)
+        lib.set_k_slices(0)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert bool(outs[0].any())
