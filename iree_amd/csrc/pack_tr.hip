@@ -362,7 +362,7 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
   const int64_t nblk0 = uk::ceil_div(outer0, tiles0), nblk1 = uk::ceil_div(outer1, tiles1);
   if (nblk0 * nblk1 >= (1ll << 31) || nblk0 * nblk1 == 0) return false;
 
-  TrArgs a;
+  TrArgs a{};
   a.src = src;
   a.dst = dst;
   a.src_pitch = pitch;
