@@ -351,6 +351,60 @@ TARGET_PACK = {
 }
 
 
+def vendor_gemm_context(torch) -> dict:
+    """Context, not a baseline: the GEMM that this image's PyTorch dispatches to
+    the vendor library (torch.matmul / torch._int_mm / torch._scaled_mm on
+    row-major operands, B given as [N][K]) at the sizes of the mmt4d targets, on
+    the same device in the same run, as microseconds and as a fraction of the
+    same published peaks. It shows where a tuned library sits under this part's
+    power limit; its operands are not tiled, so it is not the same interface."""
+    out = {}
+
+    def timed(f, n=10):
+        for _ in range(3):
+            f()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.2:   # clocks settle under load
+            f()
+            torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            f()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / n
+
+    def entry(name, S, peak, f):
+        try:
+            us = timed(f)
+            out[name] = {"us": round(us, 1), "frac": round(2.0 * S ** 3 / us / 1e6 / peak, 4)}
+        except Exception as e:   # an op this build of torch does not have
+            out[name] = {"error": repr(e)[:120]}
+
+    for dt, nm in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+        for S in (4096, 8192):
+            x = torch.randn(S, S, device="cuda", dtype=dt)
+            y = torch.randn(S, S, device="cuda", dtype=dt)
+            entry(f"{nm}_{S}", S, 2500.0, lambda: torch.matmul(x, y.t()))
+            del x, y
+    S = 8192
+    x = torch.randint(-128, 128, (S, S), device="cuda", dtype=torch.int8)
+    y = torch.randint(-128, 128, (S, S), device="cuda", dtype=torch.int8)
+    entry("s8_8192", S, 5000.0, lambda: torch._int_mm(x, y.t()))
+    del x, y
+    try:
+        x = torch.randn(S, S, device="cuda").to(torch.float8_e4m3fn)
+        y = torch.randn(S, S, device="cuda").to(torch.float8_e4m3fn)
+        one = torch.tensor(1.0, device="cuda")
+        entry("f8_8192", S, 5000.0,
+              lambda: torch._scaled_mm(x, y.t(), scale_a=one, scale_b=one, out_dtype=torch.float32))
+    except Exception as e:
+        out["f8_8192"] = {"error": repr(e)[:120]}
+    torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -427,6 +481,13 @@ def main() -> int:
     # and clock), the published peak being that product at 2.4 GHz.
     result["measured_mfma_only_clock_GHz"] = {
         dt: round(2.4 * v / rn.PEAK_TFLOPS["s8" if dt.startswith("s8") else dt], 3) for dt, v in peaks.items()}
+    # What one wave per SIMD can feed the matrix pipe against what two can (s8
+    # loop, one workgroup per CU; zeros: free of the power limit).
+    wz, wr = R.measured_mfma_waves(zeros=True), R.measured_mfma_waves(zeros=False)
+    result["measured_mfma_only_waves_per_simd_TOPS"] = {
+        "zero_operands": {"two": round(wz[2], 1), "one": round(wz[1], 1), "one_over_two": round(wz[1] / wz[2], 3)},
+        "random_operands": {"two": round(wr[2], 1), "one": round(wr[1], 1), "one_over_two": round(wr[1] / wr[2], 3)}}
+    result["vendor_gemm_same_device"] = vendor_gemm_context(torch)
     if roof["bound"] == "mfma" and wl.dtype in peaks and peaks[wl.dtype] > 0:
         # the same kernel against the ceiling measured in this run
         roof["of_measured_mfma_only"] = round(roof["achieved"] / peaks[wl.dtype], 4)

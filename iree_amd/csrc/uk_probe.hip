@@ -26,9 +26,9 @@ using uk_mfma::v4i;
 
 constexpr int kTM = 8, kTN = 4, kWaves = 8;
 
-template <Elem E>
-__global__ __launch_bounds__(kWaves * 64) void mfma_peak_kernel(const v4i* operands, int n_operands,
-                                                               int iters, int* sink, int sink_enable) {
+template <Elem E, int WAVES = kWaves>
+__global__ __launch_bounds__(WAVES * 64) void mfma_peak_kernel(const v4i* operands, int n_operands,
+                                                              int iters, int* sink, int sink_enable) {
   using TT = ElemTraits<E>;
   using Acc = typename TT::Acc;
   constexpr int H = TT::kHalves;
@@ -79,6 +79,22 @@ int run_mfma_peak(const v4i* operands, int n_operands, int iters, int workgroups
   hipLaunchKernelGGL(mfma_peak_kernel<E>, dim3(workgroups), dim3(kWaves * 64), 0, stream, operands,
                      n_operands, iters, sink, /*sink_enable=*/0);
   *ops = 2.0 * 16 * 16 * k_per_mfma<E>() * kTM * kTN * (double)iters * kWaves * workgroups;
+  return (int)hipGetLastError();
+}
+
+// The same loop with exactly `WAVES / 4` waves on every SIMD: one workgroup per
+// CU (its LDS allocation leaves no room for a second one).
+template <Elem E, int WAVES>
+int run_mfma_peak_waves(const v4i* operands, int n_operands, int iters, int cus, int* sink,
+                        hipStream_t stream, double* ops) {
+  constexpr size_t kLds = 84 * 1024;
+  auto kernel = mfma_peak_kernel<E, WAVES>;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+  if (attr != hipSuccess) return (int)attr;
+  hipLaunchKernelGGL(kernel, dim3(cus), dim3(WAVES * 64), kLds, stream, operands, n_operands, iters, sink,
+                     /*sink_enable=*/0);
+  *ops = 2.0 * 16 * 16 * k_per_mfma<E>() * kTM * kTN * (double)iters * WAVES * cus;
   return (int)hipGetLastError();
 }
 
@@ -227,6 +243,52 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(uint32_t type_flags, const vo
     }
   };
   st = run(iters / 8 + 1);  // warm-up
+  if (st == 0) st = (int)hipEventRecord(start, stream);
+  if (st == 0) st = run(iters);
+  if (st == 0) st = (int)hipEventRecord(stop, stream);
+  if (st == 0) st = (int)hipEventSynchronize(stop);
+  float ms = 0.f;
+  if (st == 0) st = (int)hipEventElapsedTime(&ms, start, stop);
+  (void)hipEventDestroy(start);
+  (void)hipEventDestroy(stop);
+  if (st != 0) return st;
+  *ops_per_second = ops / ((double)ms * 1e-3);
+  return 0;
+}
+
+// The MFMA-only loop of the s8 instruction with `waves_per_simd` (1 or 2)
+// waves on every SIMD of every CU. A wave on its own cannot keep the matrix
+// pipe full with back-to-back v_mfma_i32_16x16x64_i8 (0.84 of what two waves
+// reach, on operands that draw no power): the reason the mmt4d kernels run two
+// waves per SIMD rather than one with twice the tile.
+IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak_waves(const void* operands, int64_t operand_bytes,
+                                                         int iters, int waves_per_simd, void* sink,
+                                                         void* stream_v, double* ops_per_second) {
+  hipStream_t stream = (hipStream_t)stream_v;
+  if (!operands || operand_bytes < 16 || iters < 1 || !sink || !ops_per_second ||
+      (waves_per_simd != 1 && waves_per_simd != 2)) {
+    return (int)hipErrorInvalidValue;
+  }
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    return (int)hipErrorUnknown;
+  }
+  const v4i* ops_ptr = (const v4i*)operands;
+  const int n = (int)(operand_bytes / 16);
+  hipEvent_t start, stop;
+  if (hipEventCreate(&start) != hipSuccess) return (int)hipErrorUnknown;
+  if (hipEventCreate(&stop) != hipSuccess) {
+    (void)hipEventDestroy(start);
+    return (int)hipErrorUnknown;
+  }
+  double ops = 0;
+  auto run = [&](int it) {
+    return waves_per_simd == 1
+               ? run_mfma_peak_waves<Elem::kS8, 4>(ops_ptr, n, it, cus, (int*)sink, stream, &ops)
+               : run_mfma_peak_waves<Elem::kS8, 8>(ops_ptr, n, it, cus, (int*)sink, stream, &ops);
+  };
+  int st = run(iters / 8 + 1);  // warm-up
   if (st == 0) st = (int)hipEventRecord(start, stream);
   if (st == 0) st = run(iters);
   if (st == 0) st = (int)hipEventRecord(stop, stream);

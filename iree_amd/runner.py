@@ -739,6 +739,31 @@ class Runner:
                                f"published peak of {peak / 1e12:.1f}: not a valid ceiling")
         return best / 1e12
 
+    def measured_mfma_waves(self, zeros: bool, seconds: float = 0.02) -> dict:
+        """TOP/s of the s8 MFMA-only loop with one and with two waves on every
+        SIMD (one workgroup per CU): a lone wave does not keep the matrix pipe
+        full, which is why the mmt4d kernels run two waves per SIMD and not one
+        with twice the tile. On all-zero operands the comparison is free of the
+        power limit."""
+        torch = self.torch
+        n = 1 << 16
+        operands = (torch.zeros(n, dtype=torch.uint8, device="cuda") if zeros
+                    else self.uniform_s8((n,), 901).view(torch.uint8))
+        sink = torch.zeros(4 * 512 * 1024, dtype=torch.int32, device="cuda")
+        st = self.stream.cuda_stream
+        self.stream.synchronize()
+        out = {}
+        for waves in (2, 1):
+            rate = self.lib.probe_mfma_peak_waves(operands.data_ptr(), n, 2000, waves, sink.data_ptr(), st)
+            per_iter = 2.0 * 16 * 16 * 64 * 32 * (4 * waves) * 256
+            iters = max(1000, int(rate * seconds / per_iter))
+            best = 0.0
+            for _ in range(4):
+                best = max(best, self.lib.probe_mfma_peak_waves(operands.data_ptr(), n, iters, waves,
+                                                                sink.data_ptr(), st))
+            out[waves] = best / 1e12
+        return out
+
     def copy2d_ceiling_gbps(self, rows: int, row_bytes: int, src_pitch: int, dst_pitch: int,
                             iters: int = 10) -> float:
         """GB/s (read + write) of a plain copy of rows x row_bytes between the

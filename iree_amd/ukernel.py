@@ -195,6 +195,9 @@ class UKernelLibrary:
         L.iree_uk_amd_probe_mfma_peak.argtypes = [_u32, _vp, _i64, ctypes.c_int, ctypes.c_int, _vp,
                                                   _vp, ctypes.POINTER(ctypes.c_double)]
         L.iree_uk_amd_probe_mfma_peak.restype = ctypes.c_int
+        L.iree_uk_amd_probe_mfma_peak_waves.argtypes = [_vp, _i64, ctypes.c_int, ctypes.c_int, _vp, _vp,
+                                                        ctypes.POINTER(ctypes.c_double)]
+        L.iree_uk_amd_probe_mfma_peak_waves.restype = ctypes.c_int
         L.iree_uk_amd_probe_copy2d.argtypes = [_vp, _i64, _vp, _i64, _i64, _i64, ctypes.c_int, _vp,
                                                ctypes.POINTER(ctypes.c_double)]
         L.iree_uk_amd_probe_copy2d.restype = ctypes.c_int
@@ -324,6 +327,16 @@ class UKernelLibrary:
         if st != 0:
             raise RuntimeError(f"iree_uk_amd_probe_copy2d: status {st}")
         return sec.value
+
+    def probe_mfma_peak_waves(self, operands, operand_bytes, iters, waves_per_simd, sink, stream) -> float:
+        """Operations per second of the s8 MFMA-only loop with 1 or 2 waves on
+        every SIMD."""
+        rate = ctypes.c_double(0.0)
+        st = self.lib.iree_uk_amd_probe_mfma_peak_waves(operands, operand_bytes, iters, waves_per_simd,
+                                                        sink, stream, ctypes.byref(rate))
+        if st != 0:
+            raise RuntimeError(f"iree_uk_amd_probe_mfma_peak_waves: status {st}")
+        return rate.value
 
     def probe_copy2d_variants(self, src, src_pitch, dst, dst_pitch, row_bytes, rows, iters, stream):
         """(seconds of the fastest copy variant, [seconds of each of the five
