@@ -482,7 +482,8 @@ def main() -> int:
     result["measured_mfma_only_clock_GHz"] = {
         dt: round(2.4 * v / rn.PEAK_TFLOPS["s8" if dt.startswith("s8") else dt], 3) for dt, v in peaks.items()}
     # What one wave per SIMD can feed the matrix pipe against what two can (s8
-    # loop, one workgroup per CU; zeros: free of the power limit).
+    # loop with its MFMAs as assembly, one workgroup per CU; zeros: free of the
+    # power limit).
     wz, wr = R.measured_mfma_waves(zeros=True), R.measured_mfma_waves(zeros=False)
     result["measured_mfma_only_waves_per_simd_TOPS"] = {
         "zero_operands": {"two": round(wz[2], 1), "one": round(wz[1], 1), "one_over_two": round(wz[1] / wz[2], 3)},

@@ -455,9 +455,10 @@ IREE_UK_AMD_EXPORT const char* iree_uk_amd_last_kernel_name(void);
 IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(
     uint32_t type_flags, const void* operands, int64_t operand_bytes, int iters,
     int workgroups, void* sink, void* stream, double* ops_per_second);
-/* The s8 MFMA-only loop with exactly `waves_per_simd` (1 or 2) waves on every
- * SIMD (one workgroup per CU): what a lone wave can feed the matrix pipe
- * against what two can. Arguments as for iree_uk_amd_probe_mfma_peak. */
+/* The s8 MFMA-only loop, its MFMAs written as assembly, with exactly
+ * `waves_per_simd` (1 or 2) waves on every SIMD (one workgroup per CU): what a
+ * lone wave can feed the matrix pipe against what two can. Arguments as for
+ * iree_uk_amd_probe_mfma_peak. */
 IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak_waves(
     const void* operands, int64_t operand_bytes, int iters, int waves_per_simd,
     void* sink, void* stream, double* ops_per_second);

@@ -82,13 +82,52 @@ int run_mfma_peak(const v4i* operands, int n_operands, int iters, int workgroups
   return (int)hipGetLastError();
 }
 
-// The same loop with exactly `WAVES / 4` waves on every SIMD: one workgroup per
+// The s8 loop with its MFMAs written as assembly, in the order and on the
+// registers given: what a wave can issue, not what the compiler makes of the
+// loop. (With 256 threads the compiler moves the accumulators to the
+// accumulator file and shuffles them around every MFMA; that loop reads 0.84
+// of the rate below and says nothing about the hardware.)
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void mfma_asm_kernel(const v4i* operands, int n_operands,
+                                                             int iters, int* sink, int sink_enable) {
+  v4i fa[kTM], fb[kTN];
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < kTM; ++i) fa[i] = operands[(t * 31u + (uint32_t)i * 977u) % (uint32_t)n_operands];
+#pragma unroll
+  for (int i = 0; i < kTN; ++i) fb[i] = operands[(t * 17u + 7919u + (uint32_t)i * 613u) % (uint32_t)n_operands];
+  v4i acc[kTM][kTN];
+#pragma unroll
+  for (int i = 0; i < kTM; ++i)
+#pragma unroll
+    for (int j = 0; j < kTN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < kTM; ++i)
+#pragma unroll
+      for (int j = 0; j < kTN; ++j)
+        asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fb[j]), "v"(fa[i]));
+  }
+  // The last results leave the matrix pipe before anything reads them (the
+  // compiler does not know that the assembly is MFMAs).
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  v4i s = acc[0][0];
+#pragma unroll
+  for (int i = 0; i < kTM; ++i)
+#pragma unroll
+    for (int j = 0; j < kTN; ++j)
+      if (i || j) s = s + acc[i][j];
+  if (sink_enable) sink[t] = s[0] ^ s[1] ^ s[2] ^ s[3];
+}
+
+// That loop with exactly `WAVES / 4` waves on every SIMD: one workgroup per
 // CU (its LDS allocation leaves no room for a second one).
 template <Elem E, int WAVES>
 int run_mfma_peak_waves(const v4i* operands, int n_operands, int iters, int cus, int* sink,
                         hipStream_t stream, double* ops) {
+  static_assert(E == Elem::kS8, "the assembly loop is the s8 instruction");
   constexpr size_t kLds = 84 * 1024;
-  auto kernel = mfma_peak_kernel<E, WAVES>;
+  auto kernel = mfma_asm_kernel<WAVES>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
   if (attr != hipSuccess) return (int)attr;
@@ -256,11 +295,10 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak(uint32_t type_flags, const vo
   return 0;
 }
 
-// The MFMA-only loop of the s8 instruction with `waves_per_simd` (1 or 2)
-// waves on every SIMD of every CU. A wave on its own cannot keep the matrix
-// pipe full with back-to-back v_mfma_i32_16x16x64_i8 (0.84 of what two waves
-// reach, on operands that draw no power): the reason the mmt4d kernels run two
-// waves per SIMD rather than one with twice the tile.
+// The MFMA-only loop of the s8 instruction, written as assembly, with
+// `waves_per_simd` (1 or 2) waves on every SIMD of every CU: a wave on its own
+// keeps the matrix pipe as full as two do (0.98 on operands that draw no
+// power), so the instruction itself does not ask for a second wave.
 IREE_UK_AMD_EXPORT int iree_uk_amd_probe_mfma_peak_waves(const void* operands, int64_t operand_bytes,
                                                          int iters, int waves_per_simd, void* sink,
                                                          void* stream_v, double* ops_per_second) {

@@ -740,11 +740,10 @@ class Runner:
         return best / 1e12
 
     def measured_mfma_waves(self, zeros: bool, seconds: float = 0.02) -> dict:
-        """TOP/s of the s8 MFMA-only loop with one and with two waves on every
-        SIMD (one workgroup per CU): a lone wave does not keep the matrix pipe
-        full, which is why the mmt4d kernels run two waves per SIMD and not one
-        with twice the tile. On all-zero operands the comparison is free of the
-        power limit."""
+        """TOP/s of the s8 MFMA-only loop (MFMAs as assembly) with one and with
+        two waves on every SIMD (one workgroup per CU): a lone wave keeps the
+        matrix pipe as full as two do. On all-zero operands the comparison is
+        free of the power limit."""
         torch = self.torch
         n = 1 << 16
         operands = (torch.zeros(n, dtype=torch.uint8, device="cuda") if zeros
