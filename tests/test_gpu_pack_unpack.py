@@ -263,7 +263,10 @@ def test_pack_unpack_round_trip_and_numpy_identity(gpu):
             (np.int32, uk.PACK_TYPE_I32I32, 16, 16, True, True, (1000, 999)),
             # above 192 MB: the 64 KB-block kernels for large element-granular
             # transposes, with rows that are only 4-byte aligned and ragged edges
-            (np.float32, uk.PACK_TYPE_F32F32, 16, 1, False, True, (7169, 7171))):
+            (np.float32, uk.PACK_TYPE_F32F32, 16, 1, False, True, (7169, 7171)),
+            # above 192 MB with whole tile rows as granules under TRANSPOSE_OUTER:
+            # the 16 KB-block kernels with their non-temporal stores
+            (np.float32, uk.PACK_TYPE_F32F32, 16, 16, False, True, (8192, 8192 - 16))):
         x = rng.integers(-30000, 30000, shape).astype(dtype)
         pad_val = dtype(-1)
         pad_bits = int(np.array([pad_val]).view({2: np.uint16, 4: np.uint32}[x.itemsize])[0])
