@@ -1361,10 +1361,22 @@ int elem_bytes_of(uint32_t flags) {
 bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const char* src, char* dst,
                                 hipStream_t stream);
 
-extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
+extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p_in,
                                            void* stream_v, int kernel_mode,
                                            const char** kernel_name) {
   hipStream_t stream = (hipStream_t)stream_v;
+  // A tile that is a single row or a single column is the same bytes with and
+  // without TRANSPOSE_INNER: take it as the untransposed tile of the swapped
+  // shape, whose granules are whole tile rows instead of single elements (the
+  // reference's f32 16x16x1 right-hand side from [K][N]: [N1][K1][16][1] under
+  // both transposes is [N1][K1][1][16] under TRANSPOSE_OUTER alone).
+  iree_uk_pack_params_t canonical = *p_in;
+  if ((canonical.flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER) &&
+      (canonical.out_size2 == 1 || canonical.out_size3 == 1)) {
+    std::swap(canonical.out_size2, canonical.out_size3);
+    canonical.flags &= ~(uint32_t)IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
+  }
+  const iree_uk_pack_params_t* p = &canonical;
   const int es = elem_bytes_of(p->flags);
   if (!es) return (int)hipErrorInvalidValue;
   const bool ti = p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
@@ -1428,10 +1440,18 @@ extern "C" int iree_uk_amd_hip_launch_pack(const iree_uk_pack_params_t* p,
   return (int)hipGetLastError();
 }
 
-extern "C" int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* p,
+extern "C" int iree_uk_amd_hip_launch_unpack(const iree_uk_unpack_params_t* p_in,
                                              void* stream_v, int kernel_mode,
                                              const char** kernel_name) {
   hipStream_t stream = (hipStream_t)stream_v;
+  // (single-row and single-column tiles: see iree_uk_amd_hip_launch_pack)
+  iree_uk_unpack_params_t canonical = *p_in;
+  if ((canonical.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER) &&
+      (canonical.in_size2 == 1 || canonical.in_size3 == 1)) {
+    std::swap(canonical.in_size2, canonical.in_size3);
+    canonical.flags &= ~(uint32_t)IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER;
+  }
+  const iree_uk_unpack_params_t* p = &canonical;
   const int es = elem_bytes_of(p->flags);
   if (!es) return (int)hipErrorInvalidValue;
   const bool ti = p->flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER;

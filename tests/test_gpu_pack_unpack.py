@@ -252,6 +252,52 @@ def test_pack_transposing_kernel_declines_what_it_does_not_serve(gpu, oracle):
         assert np.array_equal(got, want), c.label()
 
 
+SINGLE_LINE_TILES = [
+    (uk.PACK_TYPE_F32F32, 16, 1), (uk.PACK_TYPE_F32F32, 1, 16), (uk.PACK_TYPE_I32I32, 8, 1),
+    (uk.PACK_TYPE_F16F16, 1, 16), (uk.PACK_TYPE_BF16BF16, 16, 1), (uk.PACK_TYPE_I8I8, 1, 16),
+    (uk.PACK_TYPE_I8I8, 16, 1), (uk.PACK_TYPE_F32F32, 1, 1), (uk.PACK_TYPE_F32F32, 1, 7),
+]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("tile", SINGLE_LINE_TILES, ids=lambda t: f"type{t[0]}_{t[1]}x{t[2]}")
+def test_single_row_and_single_column_tiles_under_transpose_inner(gpu, oracle, tile, mode):
+    """A tile that is one row or one column holds the same bytes with and without
+    TRANSPOSE_INNER, and the library takes it as the untransposed tile of the
+    swapped shape (the reference's f32 16x16x1 right-hand side packed from
+    [K][N], arch/x86_64/mmt4d_x86_64_tiles.inl). Pack and unpack, both outer
+    orders, ragged edges, loose pitches: whole buffers against the oracle."""
+    lib, torch = gpu
+    lib.set_kernel_mode(mode)
+    tf, s2, s3 = tile
+    es = uk.PACK_TYPE_BYTES[tf]
+    a0, a1 = s3, s2                       # TRANSPOSE_INNER: extents along matrix rows / columns
+    g = T.Lcg(77 + 3 * s2 + s3)
+    ci = 0
+    for (in0, in1) in ((1, 1), (33, 70), (130, 257), (64, 512)):
+        for to in (0, 1):
+            for variant in range(2):
+                o0, o1 = -(-in0 // a0) + variant, -(-in1 // a1)
+                os0, os1 = (o1, o0) if to else (o0, o1)
+                flags = tf | 0x100 | (0x200 if to else 0)
+                c = T.PackCase(flags, in0, in1, os0, os1, s2, s3, in1 + (0, 5)[variant], 1,
+                               os1 * s2 * s3 + (0, 3)[variant], (0, 2)[variant], (0, 9)[variant], g.u64())
+                inp, out0 = T.make_pack_buffers(c, np.random.default_rng(4100 + ci))
+                want = out0.copy()
+                G.run_pack_case(oracle, c, inp, want)
+                got = T.gpu_pack(lib, torch, c, inp, out0)
+                assert np.array_equal(got, want), (c.label(), lib.last_kernel_name())
+                if es > 1:                # unpack has no 1-byte type (exported_bits.h:76)
+                    u = T.UnpackCase(flags, os0, os1, s2, s3, in0, in1, c.out_stride0, c.in_stride0, 1,
+                                     c.out_offset, c.in_offset)
+                    uin, uout0 = T.make_unpack_buffers(u, np.random.default_rng(4200 + ci))
+                    uwant = uout0.copy()
+                    G.run_unpack_case(oracle, u, uin, uwant)
+                    ugot = T.gpu_unpack(lib, torch, u, uin, uout0)
+                    assert np.array_equal(ugot, uwant), (u.label(), lib.last_kernel_name())
+                ci += 1
+
+
 def test_pack_unpack_round_trip_and_numpy_identity(gpu):
     """Size-independent properties at a size the oracle would be slow on:
     pack == pad+reshape+transpose, unpack(pack(x)) == x."""
