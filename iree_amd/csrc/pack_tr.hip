@@ -1,5 +1,6 @@
-// pack with an element-granular transposition inside the tile, for 1- and
-// 2-byte elements, on the LDS transposing reads of gfx950.
+// pack with an element-granular transposition inside the tile: 1- and 2-byte
+// elements on the LDS transposing reads of gfx950, 4-byte elements on plain
+// 32-bit LDS reads.
 //
 // TRANSPOSE_INNER stores a tile as [b1][b0] (b0 the position along the rows of
 // the source matrix, b1 along its columns; index algebra of
@@ -11,7 +12,7 @@
 // reference's x86 tiles for s8, 16x2 (arch/x86_64/mmt4d_x86_64_tiles.inl),
 // are 16 two-byte elements that run down the source column.
 //
-// A workgroup stages a block of 64 rows x 256 bytes of the matrix in LDS, row
+// A workgroup stages a block of 32 rows x 512 bytes of the matrix in LDS, row
 // major, and reads it back with ds_read_b64_tr_b16 / ds_read_b64_tr_b8. Within
 // a block of 16 lanes these hand lane i, as element j of its eight bytes,
 // element i % E of what lane (16 / E) j + i / E addressed (E = 4 two-byte or 8
@@ -32,10 +33,13 @@
 
 namespace {
 
-// A block is 64 rows x 256 bytes of the matrix: 16 KB, 256 threads, four
-// workgroups per CU. (64 KB blocks of 1024 threads, 256 x 256 or 64 x 1024,
-// were measured on operands of 64 to 470 MB and were no faster.)
-constexpr int kBlockRows = 64, kBlockRowBytes = 256;
+// A block is 32 rows x 512 bytes of the matrix: 16 KB, 256 threads, four
+// workgroups per CU. Measured on operands of 128 to 600 MB that no earlier
+// launch had left in the memory-side cache: 64 x 256 is 3 to 8 % slower
+// (row segments of 256 bytes), 64 x 512 with 512 threads in between, 64 x 1024
+// with 1024 threads and 128 x 256 slower again. When the source is still in
+// that cache all of them run alike.
+constexpr int kBlockRows = 32, kBlockRowBytes = 512;
 
 typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
@@ -68,8 +72,10 @@ __device__ __forceinline__ v2u read_tr(uint32_t lds_addr) {
   return v;
 }
 
-// EB: bytes per transposed element. V: bytes a lane stores at once (16 where
-// the tile's extent along the rows is a multiple of 16 bytes, else 8). IL: 0,
+// EB: bytes per transposed element (4: no transposing read exists; a lane
+// reads its column's word from four consecutive rows). V: bytes a lane stores
+// at once (16 where the tile's extent along the rows is a multiple of 16 bytes,
+// else 8). IL: 0,
 // or the tile's extent along the rows where that is less than eight bytes (2
 // or 4 elements: the K0 = 2 tiles of the reference's x86 kernels from a
 // row-major [K][N] operand). A lane's 16 destination bytes are then 16 / IL
@@ -79,12 +85,13 @@ __device__ __forceinline__ v2u read_tr(uint32_t lds_addr) {
 template <int EB, int V, int IL = 0>
 __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kernel(TrArgs a) {
   static_assert(IL == 0 || (V == 16 && (IL * EB == 2 || IL * EB == 4)), "interleaved rows of 2 or 4 bytes");
+  static_assert(EB != 4 || (V == 16 && IL == 0), "4-byte elements: four rows per 16-byte vector");
   constexpr int kThreads = kBlockRows * kBlockRowBytes / 64;  // 64 bytes of the block per thread
   constexpr int kBlockBytes = kBlockRows * kBlockRowBytes;
   constexpr int VPR = kBlockRowBytes / 16;     // 16-byte vectors per block row
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  constexpr int E = 8 / EB;                    // elements per lane and read
-  constexpr int CH = 16 / E;                   // 8-byte column chunks per 16 columns
+  constexpr int E = EB == 4 ? 4 : 8 / EB;      // elements per lane and read (4-byte elements: per vector)
+  constexpr int CH = EB == 4 ? 16 : 16 / E;    // 8-byte column chunks per 16 columns (4-byte elements: lanes)
   constexpr int BC = kBlockRowBytes / EB;      // block columns, elements
   constexpr int NCG = BC / 16;                 // groups of 16 columns
   constexpr int RPI = V / EB;                  // rows per item
@@ -142,7 +149,8 @@ __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kern
     }
     const uint32_t r0 = ((rgt << lht) + h) * RPI;
     // What this lane addresses for the item's reads.
-    l2addr[i] = (r0 + l / CH) * a.lds_pitch + (cg * 16 + (l % CH) * E) * EB;
+    if constexpr (EB == 4) l2addr[i] = r0 * a.lds_pitch + (cg * 16 + l) * EB;  // its own column, four rows down
+    else l2addr[i] = (r0 + l / CH) * a.lds_pitch + (cg * 16 + (l % CH) * E) * EB;
     // What it receives: column cg * 16 + l of rows r0 .. r0 + RPI - 1.
     const uint32_t c = cg * 16 + l;
     tl0[i] = r0 >> a.lt0;
@@ -225,7 +233,8 @@ __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kern
             const char* gp = b.src + g1off[i];
             const uint32_t left = a.row_bytes - (b.col_base_bytes + cb);
             for (uint32_t bb = 0; bb + EB <= left && bb < 16; bb += EB) {
-              if constexpr (EB == 2) *reinterpret_cast<uint16_t*>(reg + bb) = *reinterpret_cast<const uint16_t*>(gp + bb);
+              if constexpr (EB == 4) *reinterpret_cast<uint32_t*>(reg + bb) = *reinterpret_cast<const uint32_t*>(gp + bb);
+              else if constexpr (EB == 2) *reinterpret_cast<uint16_t*>(reg + bb) = *reinterpret_cast<const uint16_t*>(gp + bb);
               else reg[bb] = gp[bb];
             }
             val = *reinterpret_cast<const v4u*>(reg);
@@ -270,13 +279,29 @@ __global__ __launch_bounds__(kBlockRows * kBlockRowBytes / 64) void pack_tr_kern
       }
       continue;
     }
+    if constexpr (EB == 4) {
+      // ---- LDS columns, word by word -> tiles ----
+      v4u out[N2];
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        const char* lp = lbuf + l2addr[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) out[i][j] = *reinterpret_cast<const uint32_t*>(lp + j * a.lds_pitch);
+      }
+#pragma unroll
+      for (int i = 0; i < N2; ++i) {
+        if (!b.interior && !(b.blk0 * tiles0 + tl0[i] < a.outer0 && b.blk1 * tiles1 + tl1[i] < a.outer1)) continue;
+        __builtin_nontemporal_store(out[i], reinterpret_cast<v4u*>(b.dst + g2off[i]));
+      }
+      continue;
+    }
     // ---- LDS, transposed -> tiles ----
     const uint32_t lb = lds_base + buf * a.lds_buf_bytes;
     v2u got[N2][R];
 #pragma unroll
     for (int i = 0; i < N2; ++i)
 #pragma unroll
-      for (int h = 0; h < R; ++h) got[i][h] = read_tr<EB>(lb + l2addr[i] + (uint32_t)h * E * a.lds_pitch);
+      for (int h = 0; h < R; ++h) got[i][h] = read_tr<EB == 4 ? 2 : EB>(lb + l2addr[i] + (uint32_t)h * E * a.lds_pitch);
     // The compiler does not count these reads: wait for them here, and tie the
     // registers to the wait so that nothing uses them before it.
 #define UK_GOT(k) "+v"(got[(k) % N2][(k) / N2 % R])
@@ -328,24 +353,32 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
   int eb;
   int64_t t0, t1, size1;
   if (ti) {
-    if (es > 2) return false;
+    if (es > 4) return false;
     eb = es; t0 = p->out_size3; t1 = p->out_size2; size1 = p->in_size1;
   } else {
-    // Tile rows of one or two bytes: the row is the element.
+    // Tile rows of one, two or four bytes: the row is the element.
+    if (p->out_size3 * es > 4) return false;
     eb = (int)(p->out_size3 * es);
-    if (eb != 1 && eb != 2) return false;
+    if (eb != 1 && eb != 2 && eb != 4) return false;
     if (p->in_size1 % p->out_size3 != 0) return false;  // (a last row of half padding)
     t0 = p->out_size2; t1 = 1; size1 = p->in_size1 / p->out_size3;
   }
   const int64_t tile_bytes = t0 * t1 * eb;
   const int64_t outer0 = to ? p->out_size1 : p->out_size0;  // tiles along the matrix rows
   const int64_t outer1 = to ? p->out_size0 : p->out_size1;
+  // Four-byte elements are also what the streaming kernel's 4-byte granules
+  // serve. Up to some hundreds of megabytes this kernel is the faster one
+  // (f32 16x1 tiles of 2048 x 2048: 5.2 against 11.2 us; 4096 x 4096: 21
+  // against 25; 6144 x 6144: 49 against 67), beyond that the other one, with
+  // its 64 KB blocks (12288 x 12288: 241 against 194 us, 288 against 225 under
+  // TRANSPOSE_OUTER).
+  if (eb == 4 && p->in_size0 * size1 * eb + outer0 * outer1 * tile_bytes > (448ll << 20)) return false;
   const int64_t bc = kBlockRowBytes / eb;
   if (!is_pow2(t0) || !is_pow2(t1) || t0 > kBlockRows || t1 > bc) return false;
   // Tiles less than eight bytes tall: rows interleaved in registers, a vector
   // of 16 / (t0 * eb) columns inside one tile.
   const int il = (t0 * eb == 2 || t0 * eb == 4) && t0 > 1 ? (int)t0 : 0;
-  if (il ? t1 * t0 * eb < 16 : (t0 * eb) % 8 != 0) return false;
+  if (il ? t1 * t0 * eb < 16 : (t0 * eb) % (eb == 4 ? 16 : 8) != 0) return false;
   const int V = il || (t0 * eb) % 16 == 0 ? 16 : 8;
   const int64_t s_outer = p->out_stride0 * es;
   const int64_t s0 = to ? tile_bytes : s_outer;
@@ -382,10 +415,12 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
   a.down = to ? 1u : 0u;
   // Rows that the lanes of one read touch lie 16 (one-byte elements: 16 rows
   // of 16 bytes per half wave) or 32 bytes apart modulo the 256 bytes of the banks.
-  a.lds_pitch = kBlockRowBytes + 16 * eb;
+  // Four-byte elements: the four items of one read are row groups four rows
+  // apart over the same 64 bytes of columns; 4 x 272 = 64 modulo 256.
+  a.lds_pitch = kBlockRowBytes + (eb == 4 ? 16 : 16 * eb);
   a.lds_buf_bytes = kBlockRows * a.lds_pitch;
-  uint64_t pad = p->padding_value & (es == 1 ? 0xFFull : 0xFFFFull);
-  a.pad32 = es == 1 ? (uint32_t)(pad * 0x01010101ull) : (uint32_t)(pad * 0x00010001ull);
+  uint64_t pad = p->padding_value & (es == 1 ? 0xFFull : es == 2 ? 0xFFFFull : 0xFFFFFFFFull);
+  a.pad32 = es == 1 ? (uint32_t)(pad * 0x01010101ull) : es == 2 ? (uint32_t)(pad * 0x00010001ull) : (uint32_t)pad;
   const uint32_t nblocks = (uint32_t)(nblk0 * nblk1);
   const size_t lds = 2 * (size_t)a.lds_buf_bytes;
   const uint32_t grid = nblocks < 1024 ? nblocks : 1024;
@@ -396,7 +431,8 @@ bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const ch
     else uk::launch(0, pack_tr_kernel<1, 16, 4>, dim3(grid), block, lds, stream, a);
     return true;
   }
-  if (eb == 2 && V == 16) uk::launch(0, pack_tr_kernel<2, 16>, dim3(grid), block, lds, stream, a);
+  if (eb == 4) uk::launch(0, pack_tr_kernel<4, 16>, dim3(grid), block, lds, stream, a);
+  else if (eb == 2 && V == 16) uk::launch(0, pack_tr_kernel<2, 16>, dim3(grid), block, lds, stream, a);
   else if (eb == 2) uk::launch(0, pack_tr_kernel<2, 8>, dim3(grid), block, lds, stream, a);
   else if (V == 16) uk::launch(0, pack_tr_kernel<1, 16>, dim3(grid), block, lds, stream, a);
   else uk::launch(0, pack_tr_kernel<1, 8>, dim3(grid), block, lds, stream, a);

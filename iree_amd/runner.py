@@ -521,11 +521,25 @@ class Runner:
     # ------------------------------------------------------------------ timing
     KIND = {"pack": 0, "unpack": 1, "mmt4d": 2, "conv": 3}
 
-    def time_op(self, op: Op, iters: int, warmup: int = 5):
+    def evict_cache(self):
+        """Reads 1 GiB that nothing else uses (a torch reduction on the launch
+        stream): afterwards the 256 MB memory-side cache holds none of the
+        operands of earlier launches, and no modified lines either. Launches
+        that rotate over three sets of buffers time the same (measured on pack:
+        98.8 / 98.9, 91.6 / 91.2, 251 / 254 us)."""
+        torch = self.torch
+        if getattr(self, "_evict", None) is None:
+            self._evict = torch.zeros(1 << 28, dtype=torch.int32, device="cuda")
+        with torch.cuda.stream(self.stream):
+            self._evict.max()
+
+    def time_op(self, op: Op, iters: int, warmup: int = 5, cold: bool = False):
         """(average, minimum, median) device duration in microseconds of
         `iters` launches. Each launch carries its own HIP start/stop event pair
         on the launch stream (iree_uk_amd_timing_begin/end), which timestamps
-        the kernel itself."""
+        the kernel itself. `cold`: the memory-side cache is emptied of the
+        operands before every timed launch (launches on the same buffers one
+        after the other find up to 256 MB of them still there)."""
         torch = self.torch
         import time
         if op.external:
@@ -554,6 +568,8 @@ class Runner:
             self.stream.synchronize()
             self.lib.timing_begin()
             for _ in range(iters):
+                if cold:
+                    self.evict_cache()
                 op.launch()
             recs = self.lib.timing_end()
         # A call may launch two kernels (whole K steps + remainder): sum per call.
@@ -764,11 +780,15 @@ class Runner:
         return out
 
     def copy2d_ceiling_gbps(self, rows: int, row_bytes: int, src_pitch: int, dst_pitch: int,
-                            iters: int = 10) -> float:
+                            iters: int = 10, cold: bool = False) -> float:
         """GB/s (read + write) of a plain copy of rows x row_bytes between the
         two pitches: what a pack / unpack of that matrix could reach if the
-        transposition were free."""
+        transposition were free. `cold`: as many times the rows as make each
+        side 3 GB or more, so that what one launch leaves in the 256 MB
+        memory-side cache is a small part of what the next one moves."""
         torch = self.torch
+        if cold:
+            rows *= max(1, -(-(3 << 30) // (rows * row_bytes)))
         src = torch.empty(rows * src_pitch, dtype=torch.uint8, device="cuda")
         dst = torch.empty(rows * dst_pitch, dtype=torch.uint8, device="cuda")
         self.stream.synchronize()

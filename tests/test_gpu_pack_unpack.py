@@ -171,21 +171,27 @@ def test_pack_direct_kernel_exact_untransposed_tilings(gpu, oracle, tf, t0, t1):
 # arch/x86_64/mmt4d_x86_64_tiles.inl).
 TRANSPOSING_TILES = [
     (uk.PACK_TYPE_F16F16, 16, 16, True), (uk.PACK_TYPE_BF16BF16, 16, 8, True), (uk.PACK_TYPE_F16F16, 16, 4, True),
-    (uk.PACK_TYPE_F16F16, 32, 64, True), (uk.PACK_TYPE_F16F16, 1, 16, True), (uk.PACK_TYPE_BF16BF16, 128, 16, True),
+    (uk.PACK_TYPE_F16F16, 64, 32, True), (uk.PACK_TYPE_F16F16, 1, 16, True), (uk.PACK_TYPE_BF16BF16, 128, 16, True),
     (uk.PACK_TYPE_I8I8, 16, 8, True), (uk.PACK_TYPE_I8I8, 16, 16, True), (uk.PACK_TYPE_I8I8, 16, 32, True),
-    (uk.PACK_TYPE_I8I8, 8, 64, True), (uk.PACK_TYPE_I8I8, 256, 8, True), (uk.PACK_TYPE_I8I8, 2, 16, True),
-    (uk.PACK_TYPE_I8I8, 16, 2, False), (uk.PACK_TYPE_I8I8, 8, 2, False), (uk.PACK_TYPE_I8I8, 64, 2, False),
+    (uk.PACK_TYPE_I8I8, 8, 32, True), (uk.PACK_TYPE_I8I8, 256, 8, True), (uk.PACK_TYPE_I8I8, 2, 16, True),
+    (uk.PACK_TYPE_I8I8, 16, 2, False), (uk.PACK_TYPE_I8I8, 8, 2, False), (uk.PACK_TYPE_I8I8, 32, 2, False),
     (uk.PACK_TYPE_I8I8, 16, 1, False), (uk.PACK_TYPE_I8I8, 8, 1, False),
     (uk.PACK_TYPE_F16F16, 16, 1, False), (uk.PACK_TYPE_BF16BF16, 4, 1, False),
     # transposed tiles less than eight bytes tall (K0 = 2 and 4 from a row-major [K][N] operand)
     (uk.PACK_TYPE_I8I8, 16, 2, True), (uk.PACK_TYPE_I8I8, 16, 4, True), (uk.PACK_TYPE_BF16BF16, 16, 2, True),
     (uk.PACK_TYPE_I8I8, 8, 2, True), (uk.PACK_TYPE_F16F16, 8, 2, True), (uk.PACK_TYPE_I8I8, 4, 4, True),
     (uk.PACK_TYPE_I8I8, 256, 2, True),
+    # four-byte elements: f32 / s32 tiles one element wide, 16-bit pairs and s8 quadruples as tile rows
+    # (the reference's 16x16x1 f32 and 16x16x2 bf16 tiles on x86, 8x8x4 s8 on arm64), and f32 transposed
+    (uk.PACK_TYPE_F32F32, 16, 1, False), (uk.PACK_TYPE_I32I32, 8, 1, False), (uk.PACK_TYPE_F32F32, 4, 1, False),
+    (uk.PACK_TYPE_F32F32, 32, 1, False), (uk.PACK_TYPE_BF16BF16, 16, 2, False), (uk.PACK_TYPE_F16F16, 8, 2, False),
+    (uk.PACK_TYPE_I8I8, 16, 4, False), (uk.PACK_TYPE_I8I8, 8, 4, False),
+    (uk.PACK_TYPE_F32F32, 16, 4, True), (uk.PACK_TYPE_F32F32, 8, 8, True), (uk.PACK_TYPE_I32I32, 64, 16, True), (uk.PACK_TYPE_F16F16, 8, 32, True),
 ]
 
 
 def _transposing_cases(tf, s2, s3, ti):
-    """Matrix shapes around the kernel's 64-row x 256-byte blocks: one block and
+    """Matrix shapes around the kernel's 32-row x 512-byte blocks: one block and
     less, several with ragged edges in both directions, tile grids larger than
     the matrix (tiles of nothing but padding), both outer orders, loose pitches
     and offsets that keep the alignment the kernel asks for (4 bytes on the
@@ -193,9 +199,9 @@ def _transposing_cases(tf, s2, s3, ti):
     es = uk.PACK_TYPE_BYTES[tf]
     a0, a1 = (s3, s2) if ti else (s2, s3)    # tile extent along matrix rows / columns
     g = T.Lcg(1234 + s2 * 7 + s3)
-    even = 2 if (not ti and s3 == 2) else 1  # (whole two-byte tile rows)
-    for (in0, in1, extra) in ((5, 6, 0), (64, 256 // es, 0), (67, 2 * (256 // es) + 10, 0), (200, 130, 1),
-                              (129, 700, 0), (3 * 64, 3 * (256 // es), 2)):
+    even = 1 if ti else s3                   # (whole tile rows)
+    for (in0, in1, extra) in ((5, 6, 0), (32, 512 // es, 0), (67, 2 * (512 // es) + 10, 0), (200, 130, 1),
+                              (129, 700, 0), (3 * 32, 3 * (512 // es), 2)):
         in1 = -(-in1 // even) * even
         for to in (0, 1):
             for variant in range(2):
@@ -236,13 +242,14 @@ def test_pack_transposing_kernel(gpu, oracle, tile):
 
 def test_pack_transposing_kernel_declines_what_it_does_not_serve(gpu, oracle):
     """Rows that are only 2-byte aligned, tile extents that are not powers of
-    two, an odd number of columns under two-byte tile rows: other kernels, same
-    bytes."""
+    two, an odd number of columns under two-byte tile rows, four-byte elements
+    in tiles less than 16 bytes tall: other kernels, same bytes."""
     lib, torch = gpu
     cases = [T.PackCase(uk.PACK_TYPE_F16F16 | 0x100, 70, 131, 5, 9, 16, 16, 131, 1, 9 * 256, 0, 0, 7),
              T.PackCase(uk.PACK_TYPE_I8I8 | 0x100, 70, 130, 6, 6, 24, 12, 132, 1, 6 * 288, 0, 0, 7),
              T.PackCase(uk.PACK_TYPE_I8I8, 70, 131, 5, 66, 16, 2, 132, 1, 66 * 32, 0, 0, 7),
-             T.PackCase(uk.PACK_TYPE_F32F32 | 0x100, 70, 130, 9, 9, 16, 8, 132, 1, 9 * 128, 0, 0, 7)]
+             T.PackCase(uk.PACK_TYPE_F32F32 | 0x100, 70, 130, 35, 9, 16, 2, 132, 1, 9 * 32, 0, 0, 7),
+             T.PackCase(uk.PACK_TYPE_F32F32, 70, 130, 35, 130, 2, 1, 132, 1, 130 * 2, 0, 0, 7)]
     for ci, c in enumerate(cases):
         inp, out0 = T.make_pack_buffers(c, np.random.default_rng(ci))
         want = out0.copy()

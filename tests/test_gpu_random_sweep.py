@@ -76,29 +76,30 @@ def test_pack_random_sweep(gpu, oracle):
 
 
 def test_pack_random_sweep_element_transpositions(gpu, oracle):
-    """1- and 2-byte types with TRANSPOSE_INNER, and untransposed tiles with rows
-    of one or two bytes, at sizes of several 64-row x 256-byte blocks: the
-    domain of the kernel on the LDS transposing reads (most cases) and its
-    borders (tile sides that are not powers of two, rows that are only 2-byte
-    aligned, tiles too small for a 16-byte vector), which other kernels serve."""
+    """Every element size with TRANSPOSE_INNER, and untransposed tiles with rows
+    of one, two or four bytes, at sizes of several 32-row x 512-byte blocks: the
+    domain of the element-transposing kernel (most cases) and its borders (tile
+    sides that are not powers of two, rows that are only 2-byte aligned, tiles
+    too small for a 16-byte vector), which other kernels serve."""
     lib, torch = gpu
     rng = np.random.default_rng(77)
     served = 0
-    for ci in range(120):
-        tf = [uk.PACK_TYPE_I8I8, uk.PACK_TYPE_F16F16, uk.PACK_TYPE_BF16BF16][ci % 3]
+    for ci in range(200):
+        tf = [uk.PACK_TYPE_I8I8, uk.PACK_TYPE_F16F16, uk.PACK_TYPE_BF16BF16, uk.PACK_TYPE_F32F32,
+              uk.PACK_TYPE_I32I32][ci % 5]
         es = uk.PACK_TYPE_BYTES[tf]
         ti = int(rng.integers(0, 4)) != 0
         if ti:
             s2 = int(rng.choice([1, 2, 4, 8, 16, 32, 64, 12]))       # columns of the matrix per tile
             s3 = int(rng.choice([2, 4, 8, 16, 32, 64, 6]))           # rows of the matrix per tile
         else:
-            s2, s3 = int(rng.choice([4, 8, 16, 32, 64, 24])), (int(rng.choice([1, 2])) if es == 1 else 1)
+            s2, s3 = int(rng.choice([4, 8, 16, 32, 64, 24])), int(rng.choice([1, 2, 4][:3 - es // 2]))
         if s2 * s3 * es > 4096:
             continue
         a0, a1 = (s3, s2) if ti else (s2, s3)
         in0, in1 = int(rng.integers(1, 330)), int(rng.integers(1, 700))
-        if not ti and s3 == 2 and rng.integers(0, 4):
-            in1 += in1 % 2
+        if not ti and s3 > 1 and rng.integers(0, 4):
+            in1 = -(-in1 // s3) * s3
         to = int(rng.integers(0, 2))
         o0 = -(-in0 // a0) + int(rng.integers(0, 2))
         o1 = -(-in1 // a1) + int(rng.integers(0, 3))
@@ -115,7 +116,7 @@ def test_pack_random_sweep_element_transpositions(gpu, oracle):
         got = T.gpu_pack(lib, torch, c, inp, out)
         assert np.array_equal(got, want), (ci, c, lib.last_kernel_name())
         served += lib.last_kernel_name() == "pack_transposing"
-    assert served >= 50, served
+    assert served >= 80, served
 
 
 def test_unpack_random_sweep(gpu, oracle):
