@@ -455,6 +455,13 @@ def main() -> int:
         per_kernel[op.name] = {"kernel": op.kernel, "avg_us": round(avg, 2), "min_us": round(mn, 2),
                                "median_us": round(med, 2),
                                "achieved": r["achieved"], "unit": r["unit"], "frac": r["frac"]}
+        if r["bound"] == "hbm" and op.bytes >= COLD_FROM_BYTES and not op.external \
+                and not args.workload.endswith("_cold"):
+            # (the same launches with the memory-side cache emptied before each)
+            cavg, cmn, cmed = R.time_op(op, max(5, min(args.steps, 30) // 2), cold=True)
+            rc = R.roofline(op, cavg)
+            per_kernel[op.name].update({"cold_avg_us": round(cavg, 2), "cold_min_us": round(cmn, 2),
+                                        "cold_achieved": rc["achieved"], "cold_frac": rc["frac"]})
 
     if wl.flops:
         metric = ("conv_nchwc TFLOP/s" if dominant == "conv"
