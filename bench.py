@@ -422,6 +422,9 @@ def main() -> int:
     ap.add_argument("--sweep", metavar="WORKLOAD", default=None,
                     help="print T(K) of a square mmt4d workload (e.g. s8_mmt4d_8192_k16) under the "
                          "big kernel variants, with a straight-line fit, instead of the JSON line")
+    ap.add_argument("--shapes", action="store_true",
+                    help="print mmt4d timings over transformer-like M x N x K shapes beside the vendor "
+                         "library's GEMM on the same device, instead of the JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards by tile rows with no "
@@ -437,6 +440,11 @@ def main() -> int:
     if args.sweep:
         print("command: python bench.py --sweep " + args.sweep)
         print(R.k_sweep(args.sweep))
+        R.close()
+        return 0
+    if args.shapes:
+        print("command: python bench.py --shapes")
+        print(R.shape_survey())
         R.close()
         return 0
     wl = R.workload(args.workload)

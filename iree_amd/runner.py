@@ -646,6 +646,89 @@ class Runner:
         dom_us = dom_total / (steps * max(1, n_kind if n_dom == 0 else n_kind)) if recs else math.nan
         return (t1 - t0) / steps, (t3 - t2) / steps, dom_us
 
+    def shape_survey(self, reps: int = 15) -> str:
+        """mmt4d on M x N x K problems shaped like a transformer's projections
+        (M tokens from 256 to 4096 against five weight shapes), 16x16 tiles with
+        16-byte tile rows, s8 / f16 / bf16: microseconds, fraction of the
+        published peak and the kernel that ran, and beside each the GEMM that
+        this image's PyTorch dispatches to the vendor library for the same
+        problem on row-major operands (torch._int_mm / torch.matmul, B given as
+        [N][K]) in the same process. The operands of the two differ in layout
+        only; the comparison is context, not a baseline."""
+        import time
+        torch, lib = self.torch, self.lib
+
+        def settle(f):
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < 0.25:
+                for _ in range(4):
+                    f()
+                torch.cuda.synchronize()
+
+        def time_ours(f):
+            with torch.cuda.stream(self.stream):
+                settle(f)
+                for _ in range(3):
+                    f()
+                name = lib.last_kernel_name()
+                lib.timing_begin()
+                for _ in range(reps):
+                    f()
+                recs = lib.timing_end()
+            per = len(recs) // reps
+            ts = sorted(sum(t for _, t in recs[i * per:(i + 1) * per]) for i in range(reps))
+            return ts[len(ts) // 2], name
+
+        def time_torch(f):
+            settle(f)
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                   for _ in range(reps)]
+            for a, b in evs:
+                a.record()
+                f()
+                b.record()
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+            return ts[len(ts) // 2]
+
+        lines = ["type     M x N x K              ours us  frac  kernel                  vendor us  frac  ours/vendor"]
+        ratios = {}
+        for (tname, tflag, tdt, K0, peak) in (("s8", uk.MMT4D_TYPE_S8S8S32, torch.int8, 16, PEAK_TFLOPS["s8"]),
+                                              ("f16", uk.MMT4D_TYPE_F16F16F32, torch.float16, 8, PEAK_TFLOPS["f16"]),
+                                              ("bf16", uk.MMT4D_TYPE_BF16BF16F32, torch.bfloat16, 8, PEAK_TFLOPS["bf16"])):
+            for (N, K) in ((4096, 4096), (14336, 4096), (4096, 14336), (28672, 8192), (8192, 8192)):
+                for M in (256, 512, 1024, 2048, 4096):
+                    M1, N1, K1 = M // 16, N // 16, K // K0
+                    if tdt == torch.int8:
+                        a = torch.randint(-128, 128, (M, K), device="cuda", dtype=tdt)
+                        b = torch.randint(-128, 128, (N, K), device="cuda", dtype=tdt)
+                    else:
+                        a = torch.randn(M, K, device="cuda", dtype=tdt)
+                        b = torch.randn(N, K, device="cuda", dtype=tdt)
+                    out = torch.empty(M * N, device="cuda",
+                                      dtype=torch.int32 if tdt == torch.int8 else torch.float32)
+                    lp, rp, op_ = a.data_ptr(), b.data_ptr(), out.data_ptr()
+                    # (the same bytes read as tiled operands: timing does not depend on the values' order)
+                    us, kn = time_ours(lambda: lib.mmt4d(lp, 0, K1 * 16 * K0, rp, 0, K1 * 16 * K0, op_, 0,
+                                                         N1 * 256, M1, N1, K1, 16, 16, K0, tflag))
+                    bt = b.t()
+                    try:
+                        v = time_torch((lambda: torch._int_mm(a, bt)) if tdt == torch.int8
+                                       else (lambda: torch.matmul(a, bt)))
+                    except Exception:   # an op this build of torch does not have
+                        v = float("nan")
+                    fl = 2.0 * M * N * K
+                    ratios.setdefault(tname, []).append(us / v)
+                    lines.append(f"{tname:5s} {M:5d} x {N:5d} x {K:5d}  {us:9.1f}  {fl / us / 1e6 / peak:.3f}  "
+                                 f"{kn.replace('mmt4d_mfma_', ''):22s} {v:9.1f}  {fl / v / 1e6 / peak:.3f}  {us / v:.2f}")
+                    del a, b, bt, out
+        for tname, r in ratios.items():
+            r = sorted(x for x in r if x == x)
+            if r:
+                lines.append(f"{tname}: ours/vendor between {r[0]:.2f} and {r[-1]:.2f}, median {r[len(r) // 2]:.2f} "
+                             f"over {len(r)} shapes")
+        return "\n".join(lines)
+
     def k_sweep(self, name: str, variants=(0, 16, 8, 1), reps: int = 15) -> str:
         """T(K) of the mmt4d op of a square workload (`<type>_mmt4d_<size>_k<K0>`)
         under forced kernel variants, K from 1/16 of the workload's K up to all
