@@ -8,7 +8,7 @@
 // contiguous in the destination runs down a column of the source. That is the
 // form a row-major [K][N] right-hand side takes on its way to [N1][K1][N0][K0]
 // (tests/e2e/linalg/pack_i8.mlir:48-68). An untransposed tile whose rows hold
-// one or two bytes is the same problem with the tile row as the element: the
+// one, two or four bytes is the same problem with the tile row as the element: the
 // reference's x86 tiles for s8, 16x2 (arch/x86_64/mmt4d_x86_64_tiles.inl),
 // are 16 two-byte elements that run down the source column.
 //

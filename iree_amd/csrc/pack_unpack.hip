@@ -1357,7 +1357,7 @@ int elem_bytes_of(uint32_t flags) {
 
 }  // namespace
 
-// pack_tr.hip: tiles transposed element by element, 1- and 2-byte elements.
+// pack_tr.hip: tiles transposed element by element (1-, 2- and 4-byte elements).
 bool iree_uk_amd_launch_pack_tr(const iree_uk_pack_params_t* p, int es, const char* src, char* dst,
                                 hipStream_t stream);
 

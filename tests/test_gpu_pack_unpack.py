@@ -166,8 +166,8 @@ def test_pack_direct_kernel_exact_untransposed_tilings(gpu, oracle, tf, t0, t1):
 
 
 # (type, stored tile shape out_size2 x out_size3, TRANSPOSE_INNER): element-wise
-# transpositions of 1- and 2-byte elements, and untransposed tiles whose rows
-# are one or two bytes (the reference's 16x2 s8 tile,
+# transpositions, and untransposed tiles whose rows are one, two or four bytes
+# (the reference's 16x2 s8 tile,
 # arch/x86_64/mmt4d_x86_64_tiles.inl).
 TRANSPOSING_TILES = [
     (uk.PACK_TYPE_F16F16, 16, 16, True), (uk.PACK_TYPE_BF16BF16, 16, 8, True), (uk.PACK_TYPE_F16F16, 16, 4, True),
