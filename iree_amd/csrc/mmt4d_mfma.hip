@@ -121,6 +121,7 @@ struct OwnedWorkspaces : std::vector<OwnedWorkspace> {
 // hold a megabyte and more per stream handle it ever saw).
 constexpr size_t kMaxOwnedWorkspaces = 8;
 thread_local OwnedWorkspaces g_workspaces;
+thread_local OwnedWorkspaces g_expand_workspaces;   // s4 weights expanded to s8 (n_counters unused)
 thread_local bool g_no_alloc = false;
 thread_local int g_k_slices = 0;
 thread_local int g_last_k_slices = 1;
@@ -210,6 +211,50 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
   g_workspaces.push_back(OwnedWorkspace{dev, stream, base, want_partials, want_counters, now});
   ws->partials = base;
   ws->counters = (uint32_t*)(base + want_partials);
+  return 0;
+}
+
+int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base_out) {
+  if (g_no_alloc || bytes == 0 || bytes > ((size_t)2 << 30)) return 1;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) { (void)hipGetLastError(); return 1; }
+  if (capture != hipStreamCaptureStatusNone) return 1;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 1;
+  OwnedWorkspaces& pool = g_expand_workspaces;
+  const uint64_t now = ++pool.uses;
+  for (OwnedWorkspace& w : pool) {
+    if (w.device == dev && w.stream == stream && w.partial_bytes >= bytes) {
+      w.last_use = now;
+      *base_out = w.base;
+      return 0;
+    }
+  }
+  // Nothing fits: the stream's smaller buffer goes, and beyond two buffers per
+  // thread the one used longest ago (hipFree waits for the device first).
+  for (size_t i = 0; i < pool.size();) {
+    if (pool[i].device == dev && pool[i].stream == stream) {
+      (void)hipFree(pool[i].base);
+      pool.erase(pool.begin() + (ptrdiff_t)i);
+    } else {
+      ++i;
+    }
+  }
+  while (pool.size() >= 2) {
+    size_t oldest = 0;
+    for (size_t i = 1; i < pool.size(); ++i) {
+      if (pool[i].last_use < pool[oldest].last_use) oldest = i;
+    }
+    (void)hipFree(pool[oldest].base);
+    pool.erase(pool.begin() + (ptrdiff_t)oldest);
+  }
+  size_t want = (size_t)16 << 20;
+  while (want < bytes) want <<= 1;
+  char* base = nullptr;
+  if (hipMalloc((void**)&base, want) != hipSuccess) { (void)hipGetLastError(); return 1; }
+  iree_uk_amd_hip_note_device_alloc();
+  pool.push_back(OwnedWorkspace{dev, stream, base, want, 0, now});
+  *base_out = base;
   return 0;
 }
 

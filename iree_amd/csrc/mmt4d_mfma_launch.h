@@ -152,6 +152,13 @@ struct KSplitWorkspace {
 };
 int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStream_t stream,
                              KSplitWorkspace* ws);
+// A buffer of `bytes` for s4 weights expanded to s8 (mmt4d_mfma_s8s4.hip), kept
+// per host thread and stream like the K split's workspace and apart from it
+// (the s8 launch that reads the expanded weights may itself split K). Returns
+// 0 and the pointer, or 1 when there is none to be had: under
+// iree_uk_amd_mmt4d_no_alloc, while the stream is being captured into a graph,
+// or when the allocation fails.
+int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base);
 // K slices set with iree_uk_amd_set_k_slices on this thread; 0 = choose.
 int k_slices_override();
 // 1: the calling thread has declared its weights streamed from HBM

@@ -80,3 +80,69 @@ def test_s8s4_decode_shape_equals_integer_product(gpu):
     b = vals.permute(0, 2, 1, 3).reshape(N1 * N0, K1 * K0)
     want = (a @ b.T).reshape(M1, M0, N1, N0).permute(0, 2, 1, 3) + init.cpu().to(torch.int64)
     assert torch.equal(out.cpu().to(torch.int64), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M0,N0,K0", [(16, 16, 16), (16, 16, 32), (32, 8, 64), (24, 20, 32), (1, 16, 16)])
+def test_s8s4_many_rows_run_on_expanded_weights(gpu, oracle, M0, N0, K0):
+    """From 512 rows on the 4-bit weights are expanded to s8 once and the s8
+    kernels run on the copy: full-range inputs, ACCUMULATE off and on, loose
+    strides and offsets (the reference's case grid), bit for bit against the
+    oracle; 511 rows still run on the thin kernel."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    step = 64 // K0
+    rows = -(-512 // M0)
+    shapes = [(rows, 3, 2 * step), (rows + 3, 9, 5 * step), (2 * rows + 1, 1, step)]
+    for si, (M1, N1, K1) in enumerate(shapes):
+        for ci, c in enumerate(T.mmt4d_cases(TF, M0, N0, K0, seed=900 + si, slack=16,
+                                             shapes=((M1, N1, K1),))):
+            rng = np.random.default_rng(100 * si + ci)
+            lhs, rhs, out0 = _full_range(c, rng)
+            want = out0.copy()
+            G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+            got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+            assert lib.last_kernel_name() == "mmt4d_mfma_s8s4_expanded", (c.label(), lib.last_kernel_name())
+            assert np.array_equal(got, want), c.label()
+    if (511 // M0) * M0 >= 64:
+        c = next(iter(T.mmt4d_cases(TF, M0, N0, K0, seed=7, slack=16, shapes=((511 // M0, 3, 2 * step),))))
+        lhs, rhs, out0 = _full_range(c, np.random.default_rng(3))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert lib.last_kernel_name() == "mmt4d_mfma_thin_s8s4", lib.last_kernel_name()
+        assert np.array_equal(got, want), c.label()
+
+
+@pytest.mark.gpu
+def test_s8s4_prefill_shape_equals_integer_product(gpu):
+    """A prefill-sized call (2048 rows against 4096 x 2048 4-bit weights, tiles
+    16x16x32, ACCUMULATE) against the exact integer product of the unpacked
+    operands, twice in a row with different weights (the second call reuses the
+    library's buffer for the expanded weights), and once through the entry
+    point that may not allocate, which keeps the thin kernel."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    M0, N0, K0 = 16, 16, 32
+    M1, N1, K1 = 128, 256, 64
+    g = torch.Generator(device="cuda"); g.manual_seed(11)
+    for rep in range(3):
+        lhs = torch.randint(-128, 128, (M1, K1, M0, K0), generator=g, device="cuda", dtype=torch.int8)
+        rhs = torch.randint(0, 256, (N1, K1, N0, K0 // 2), generator=g, device="cuda", dtype=torch.uint8)
+        out = torch.randint(-10 ** 6, 10 ** 6, (M1, N1, M0, N0), generator=g, device="cuda", dtype=torch.int32)
+        init = out.clone()
+        call = lib.mmt4d_no_alloc if rep == 2 else lib.mmt4d
+        call(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, out.data_ptr(), 0,
+             N1 * M0 * N0, M1, N1, K1, M0, N0, K0, TF | uk.MMT4D_ACCUMULATE | 0x200)
+        lib.synchronize()
+        assert lib.last_kernel_name() == ("mmt4d_mfma_thin_s8s4" if rep == 2 else "mmt4d_mfma_s8s4_expanded")
+        r = rhs.to(torch.int64)
+        lo, hi = r & 0xF, r >> 4
+        lo = torch.where(lo >= 8, lo - 16, lo)
+        hi = torch.where(hi >= 8, hi - 16, hi)
+        vals = torch.stack([lo, hi], dim=-1).reshape(N1, K1, N0, K0)        # element 2h = low nibble
+        a = lhs.permute(0, 2, 1, 3).reshape(M1 * M0, K1 * K0).double()
+        b = vals.permute(0, 2, 1, 3).reshape(N1 * N0, K1 * K0).double()
+        # (every partial sum is an integer below 2^53: the f64 product is exact)
+        want = (a @ b.T).to(torch.int64).reshape(M1, M0, N1, N0).permute(0, 2, 1, 3) + init.to(torch.int64)
+        assert torch.equal(out.to(torch.int64), want), rep
