@@ -45,7 +45,9 @@ def test_s16_types_on_the_dot_product_kernel(gpu, oracle, tile, slack):
         if c.M and c.N and c.K:
             # (s16 x s16 with K in whole 64-element steps and more than 32 rows
             # and columns runs on the matrix cores: tests/test_gpu_s16_mfma.py)
-            served = {"mmt4d_dot2"} | ({"mmt4d_mfma_128x128_s16"} if tf == uk.MMT4D_TYPE_S16S16S32 else set())
+            # (the other two from 128 rows and columns on, on a widened right-hand side)
+            served = {"mmt4d_dot2"} | ({"mmt4d_mfma_128x128_s16"} if tf == uk.MMT4D_TYPE_S16S16S32
+                                       else {"mmt4d_mfma_128x128_s16_widened"})
             assert lib.last_kernel_name() in served, lib.last_kernel_name()
 
 

@@ -126,3 +126,49 @@ def test_s16_matrix_core_kernel_agrees_with_the_dot_product_kernel_at_size(gpu):
         outs.append((lib.last_kernel_name(), out))
     assert outs[0][0] == MFMA_NAME and outs[1][0] == "mmt4d_dot2", [n for n, _ in outs]
     assert torch.equal(outs[0][1], outs[1][1])
+
+
+# (type, M0, N0, K0): the reference's x86 tiles for these types (16x16x2 for
+# s16 x s8, 1x32x8 for s16 x u4: arch/x86_64/mmt4d_x86_64_tiles.inl) and others.
+WIDENED_TILES = [(uk.MMT4D_TYPE_S16S8S32, 16, 16, 2), (uk.MMT4D_TYPE_S16S8S32, 8, 8, 16),
+                 (uk.MMT4D_TYPE_S16S8S32, 24, 12, 4), (uk.MMT4D_TYPE_S16U4S32, 1, 32, 8),
+                 (uk.MMT4D_TYPE_S16U4S32, 16, 16, 32), (uk.MMT4D_TYPE_S16U4S32, 4, 8, 2)]
+WIDENED_NAME = "mmt4d_mfma_128x128_s16_widened"
+
+
+@pytest.mark.parametrize("slack", [0, 16])
+@pytest.mark.parametrize("tile", WIDENED_TILES, ids=lambda t: f"type{t[0]:#x}_{t[1]}x{t[2]}x{t[3]}")
+def test_s16_by_s8_and_u4_run_on_a_widened_right_hand_side(gpu, oracle, tile, slack):
+    """s16 x s8 and s16 x u4 with 128 rows and columns or more and K in whole
+    steps of 64 elements: the right-hand side is widened to s16 and the s16
+    matrix-core kernel runs; full-range inputs (every byte value on the RHS:
+    all s8 values, both nibbles from 0 to 15), ACCUMULATE off and on, loose
+    strides and offsets, bit for bit against the oracle. One row or column
+    fewer, or a K remainder, stays on the dot-product kernel."""
+    lib, torch = gpu
+    tf, M0, N0, K0 = tile
+    ks = 64 // K0
+    mb, nb = -(-128 // M0), -(-128 // N0)
+    shapes = ((mb, nb, ks), (mb + 1, 2 * nb + 1, 3 * ks), (2 * mb + 1, nb, 5 * ks))
+    rhs_bits = 8 if tf == uk.MMT4D_TYPE_S16S8S32 else 4
+    for ci, c in enumerate(T.mmt4d_cases(tf, M0, N0, K0, seed=300 + M0 + K0, slack=slack, shapes=shapes)):
+        rng = np.random.default_rng(7000 + 100 * slack + ci)
+        lhs = _full_range(rng, max(1, (c.M * c.lhs_stride0 + c.lhs_offset) * 2 + 64))
+        rhs = rng.integers(0, 256, (c.N * c.rhs_stride0 + c.rhs_offset) * rhs_bits // 8 + 64, dtype=np.uint8)
+        out0 = rng.integers(-2**31, 2**31, c.M * c.out_stride0 + c.out_offset + 16,
+                            dtype=np.int64).astype(np.int32).view(np.uint8).copy()
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+        assert lib.last_kernel_name() == WIDENED_NAME, (c.label(), lib.last_kernel_name())
+        assert np.array_equal(got, want), c.label()
+    if M0 > 1:
+        for shape in ((mb - 1, nb, ks), (mb, nb, ks + 1)):
+            c = next(iter(T.mmt4d_cases(tf, M0, N0, K0, seed=5, slack=0, shapes=(shape,))))
+            rng = np.random.default_rng(31)
+            lhs, rhs, out0 = T.make_mmt4d_buffers(c, rng)
+            want = out0.copy()
+            G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+            got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
+            assert lib.last_kernel_name() == "mmt4d_dot2", (shape, lib.last_kernel_name())
+            assert np.array_equal(got, want), c.label()
