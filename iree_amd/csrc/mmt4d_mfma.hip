@@ -334,7 +334,8 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
   Elem e;
   int eb, ob;
   // s8 x s4 -> s32 has a kernel for some shapes only (K0 a power of two in
-  // [16, 64], K in whole 64-element steps): it does not count as "supported"
+  // [16, 64], K in whole 64-element steps; from 512 rows on, what the s8
+  // kernels take): it does not count as "supported"
   // for iree_uk_mmt4d_info, but is tried before the generic kernel.
   const bool s8s4 = (p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32;
   // s16 x s16 -> s32 likewise: four 8-bit products per element pair in the
@@ -345,7 +346,9 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     e = Elem::kS8S4;
     eb = 1;
     ob = 4;
-    if (p->K0 != 16 && p->K0 != 32 && p->K0 != 64) return -1;
+    // (K0 below 16 - the reference's arm64 tiles Mx16x2 and Mx8x8 - only on
+    // expanded weights, i.e. from 512 rows on: launch_s8s4)
+    if (p->K0 != 2 && p->K0 != 4 && p->K0 != 8 && p->K0 != 16 && p->K0 != 32 && p->K0 != 64) return -1;
     if (p->M0 < 1 || p->N0 < 1 || p->M0 > 64 || p->N0 > 64) return -1;
     if (forced_variant != 0 && forced_variant != 4) return -1;
   } else if (s16) {

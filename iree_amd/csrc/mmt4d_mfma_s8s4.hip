@@ -4,10 +4,16 @@
 // (a prefill against 4-bit weights): the weights are expanded to s8 once, into
 // a buffer the library keeps, and the s8 kernels run on that.
 #include "mmt4d_mfma_launch.h"
+#include "uk_hip_abi.h"
 
 namespace uk_mfma {
 
 int launch_s8(const Problem& p, int forced, hipStream_t stream, const char** name);
+}  // namespace uk_mfma
+
+extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0, int32_t K0, uint32_t flags);
+
+namespace uk_mfma {
 
 namespace {
 
@@ -55,7 +61,8 @@ int launch_s8s4(const Problem& p, hipStream_t stream, const char** name) {
   const int64_t rows_m = std::min<int64_t>((int64_t)p.M1 * p.M0, p.out_rows);  // rows that are stored
   const int64_t panel_in_bytes = ((int64_t)p.K1 * p.N0 * p.rb) / 2;
   if (rows_m >= kExpandFromRows && p.N1 > 0 && p.N1 < 65536 && panel_in_bytes % 8 == 0 &&
-      panel_in_bytes < (1ll << 31)) {
+      panel_in_bytes < (1ll << 31) &&
+      iree_uk_amd_hip_mmt4d_mfma_supported(p.M0, p.N0, p.rb, IREE_UK_FLAG_MMT4D_TYPE_S8S8S32)) {
     char* expanded = nullptr;
     if (acquire_expand_workspace((size_t)(2 * panel_in_bytes * p.N1), stream, &expanded) == 0) {
       const uint32_t per_panel = (uint32_t)std::min<int64_t>(uk::ceil_div(panel_in_bytes, (int64_t)(256 * 8)), 64);
@@ -73,6 +80,7 @@ int launch_s8s4(const Problem& p, hipStream_t stream, const char** name) {
       // (not served as s8: the thin kernel below reads the packed weights)
     }
   }
+  if (p.rb < 16) return -1;  // the thin kernel unpacks 16 nibbles per lane: tile rows of 16 and more
   int st;
   if (rows_m <= 16) {
     st = launch_thin<Elem::kS8S4, 16, 1, 2, 4, 4>(p, false, stream, true);

@@ -83,15 +83,18 @@ def test_s8s4_decode_shape_equals_integer_product(gpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M0,N0,K0", [(16, 16, 16), (16, 16, 32), (32, 8, 64), (24, 20, 32), (1, 16, 16)])
+@pytest.mark.parametrize("M0,N0,K0", [(16, 16, 16), (16, 16, 32), (32, 8, 64), (24, 20, 32), (1, 16, 16),
+                                      (8, 8, 8), (16, 16, 2), (4, 8, 4)])
 def test_s8s4_many_rows_run_on_expanded_weights(gpu, oracle, M0, N0, K0):
     """From 512 rows on the 4-bit weights are expanded to s8 once and the s8
     kernels run on the copy: full-range inputs, ACCUMULATE off and on, loose
     strides and offsets (the reference's case grid), bit for bit against the
-    oracle; 511 rows still run on the thin kernel."""
+    oracle; 511 rows still run on the thin kernel, or, for tile rows under 16
+    elements (arm64's 8x8x8 among them: arch/arm_64/mmt4d_arm_64_dotprod.c:85),
+    on the scalar one."""
     lib, torch = gpu
     lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
-    step = 64 // K0
+    step = max(1, 64 // K0)
     rows = -(-512 // M0)
     shapes = [(rows, 3, 2 * step), (rows + 3, 9, 5 * step), (2 * rows + 1, 1, step)]
     for si, (M1, N1, K1) in enumerate(shapes):
@@ -110,7 +113,8 @@ def test_s8s4_many_rows_run_on_expanded_weights(gpu, oracle, M0, N0, K0):
         want = out0.copy()
         G.run_mmt4d_case(oracle, c, lhs, rhs, want)
         got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0)
-        assert lib.last_kernel_name() == "mmt4d_mfma_thin_s8s4", lib.last_kernel_name()
+        assert lib.last_kernel_name() == ("mmt4d_mfma_thin_s8s4" if K0 >= 16 else "mmt4d_generic"), \
+            lib.last_kernel_name()
         assert np.array_equal(got, want), c.label()
 
 
