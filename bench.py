@@ -425,6 +425,9 @@ def main() -> int:
     ap.add_argument("--shapes", action="store_true",
                     help="print mmt4d timings over transformer-like M x N x K shapes beside the vendor "
                          "library's GEMM on the same device, instead of the JSON line")
+    ap.add_argument("--tiles", action="store_true",
+                    help="print, for every mmt4d type on the tile shapes of the reference's CPU kernels, "
+                         "the kernel that serves it and its rate at 2048^3, instead of the JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards by tile rows with no "
@@ -440,6 +443,11 @@ def main() -> int:
     if args.sweep:
         print("command: python bench.py --sweep " + args.sweep)
         print(R.k_sweep(args.sweep))
+        R.close()
+        return 0
+    if args.tiles:
+        print("command: python bench.py --tiles")
+        print(R.tile_survey())
         R.close()
         return 0
     if args.shapes:

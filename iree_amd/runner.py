@@ -729,6 +729,61 @@ class Runner:
                              f"over {len(r)} shapes")
         return "\n".join(lines)
 
+    def tile_survey(self, size: int = 2048, reps: int = 5) -> str:
+        """Every mmt4d type on the tile shapes the reference's own CPU kernels
+        use (arch/x86_64/mmt4d_x86_64_tiles.inl, arch/arm_64/mmt4d_arm_64_tiles.inl
+        and the s8 x s4 kernels of arch/arm_64/mmt4d_arm_64_*.c) at size^3:
+        which kernel serves it, microseconds, operations per second. The 16-bit
+        outputs run once as the reference defines them without
+        SKIP_INTERMEDIATE_ROUNDINGS (a rounding per K tile, which only the
+        scalar kernel reproduces) and once with the flag."""
+        torch, lib = self.torch, self.lib
+        skip = uk.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+        cases = [
+            ("f32", uk.MMT4D_TYPE_F32F32F32, (32, 32, 32), [(16, 16, 1), (8, 8, 1), (8, 4, 1)]),
+            ("f16 -> f32", uk.MMT4D_TYPE_F16F16F32, (16, 16, 32), [(16, 16, 1), (8, 8, 1)]),
+            ("f16 -> f16", uk.MMT4D_TYPE_F16F16F16, (16, 16, 16), [(16, 16, 1), (8, 8, 1)]),
+            ("f16 -> f16, skip", uk.MMT4D_TYPE_F16F16F16 | skip, (16, 16, 16), [(16, 16, 1), (8, 8, 1)]),
+            ("bf16 -> f32", uk.MMT4D_TYPE_BF16BF16F32, (16, 16, 32), [(16, 16, 2), (8, 8, 4)]),
+            ("bf16 -> bf16", uk.MMT4D_TYPE_BF16BF16BF16, (16, 16, 16), [(16, 16, 2), (8, 8, 4)]),
+            ("bf16 -> bf16, skip", uk.MMT4D_TYPE_BF16BF16BF16 | skip, (16, 16, 16), [(16, 16, 2), (8, 8, 4)]),
+            ("s8", uk.MMT4D_TYPE_S8S8S32, (8, 8, 32), [(16, 16, 2), (8, 8, 1), (8, 8, 4), (8, 8, 8)]),
+            ("s16 x s16", uk.MMT4D_TYPE_S16S16S32, (16, 16, 32), [(16, 16, 2), (8, 8, 1)]),
+            ("s16 x s8", uk.MMT4D_TYPE_S16S8S32, (16, 8, 32), [(16, 16, 2)]),
+            ("s16 x u4", uk.MMT4D_TYPE_S16U4S32, (16, 4, 32), [(1, 32, 8)]),
+            ("s8 x s4", uk.MMT4D_TYPE_S8S4S32, (8, 4, 32), [(4, 16, 2), (8, 8, 8), (4, 8, 16), (1, 8, 16)]),
+        ]
+        S = size
+        lines = [f"mmt4d {S}^3 on the reference's CPU tile shapes",
+                 "type                 M0xN0xK0          us      TOP/s  kernel"]
+        for nm, tf, bits, tiles in cases:
+            for (M0, N0, K0) in tiles:
+                M1, N1, K1 = S // M0, S // N0, S // K0
+                # small byte values: finite in every float type, and timing does not depend on them
+                a = torch.randint(0, 40, (S * S * bits[0] // 8,), device="cuda", dtype=torch.uint8)
+                b = torch.randint(0, 40, (S * S * bits[1] // 8,), device="cuda", dtype=torch.uint8)
+                out = torch.empty(S * S * bits[2] // 8, device="cuda", dtype=torch.uint8)
+                ap, bp, op_ = a.data_ptr(), b.data_ptr(), out.data_ptr()
+                flags = tf | uk.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
+
+                def f():
+                    lib.mmt4d(ap, 0, K1 * M0 * K0, bp, 0, K1 * N0 * K0, op_, 0, N1 * M0 * N0,
+                              M1, N1, K1, M0, N0, K0, flags)
+                with torch.cuda.stream(self.stream):
+                    for _ in range(2):
+                        f()
+                    name = lib.last_kernel_name()
+                    lib.timing_begin()
+                    for _ in range(reps):
+                        f()
+                    recs = lib.timing_end()
+                per = len(recs) // reps
+                ts = sorted(sum(t for _, t in recs[i * per:(i + 1) * per]) for i in range(reps))
+                us = ts[len(ts) // 2]
+                lines.append(f"{nm:20s} {M0:2d}x{N0:2d}x{K0:2d}  {us:10.1f}  {2.0 * S ** 3 / us / 1e6:9.1f}  {name}")
+                del a, b, out
+        return "\n".join(lines)
+
     def k_sweep(self, name: str, variants=(0, 16, 8, 1), reps: int = 15) -> str:
         """T(K) of the mmt4d op of a square workload (`<type>_mmt4d_<size>_k<K0>`)
         under forced kernel variants, K from 1/16 of the workload's K up to all
