@@ -15,6 +15,9 @@ extern "C" int iree_uk_amd_hip_mmt4d_mfma_supported(int32_t M0, int32_t N0,
 extern "C" int iree_uk_amd_hip_launch_mmt4d_s16_widened(
     const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
     void* stream, const char** kernel_name);
+extern "C" int iree_uk_amd_hip_launch_mmt4d_retiled(
+    const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
+    void* stream, const char** kernel_name);
 extern "C" int iree_uk_amd_hip_launch_mmt4d_dot2(
     const iree_uk_mmt4d_params_t* p, const iree_uk_amd_rowmajor_out_t* rowmajor,
     void* stream);
@@ -60,6 +63,12 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d(const iree_uk_mmt4d_params_t* p,
     // one the info query advertises, count the call so that the cliff shows.
     if (st >= 0) return st;
     if (!maybe && kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO && p->K != 0) ++g_declined;
+  }
+  if (kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO) {
+    // Tile rows under 16 bytes in shapes the matrix-core kernels decline:
+    // regrouped along K first (mmt4d_mfma.hip).
+    const int st = iree_uk_amd_hip_launch_mmt4d_retiled(p, rowmajor, stream, kernel_name);
+    if (st >= 0) return st;
   }
   if (kernel_mode == IREE_UK_AMD_KERNEL_MODE_AUTO) {
     // s16 x s8 and s16 x u4 with enough rows and columns: the matrix-core s16

@@ -214,6 +214,57 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
   return 0;
 }
 
+namespace {
+typedef uint32_t v4u_rt __attribute__((ext_vector_type(4)));
+
+template <int SRC_BITS>
+__global__ __launch_bounds__(256) void retile_rows_kernel(const char* src, int64_t src_stride, char* dst,
+                                                           int64_t dst_stride, uint32_t R0, uint32_t rb,
+                                                           uint32_t K1, uint32_t K1p) {
+  const char* s = src + (int64_t)blockIdx.y * src_stride;
+  char* d = dst + (int64_t)blockIdx.y * dst_stride;
+  const uint32_t g = 16 / rb;            // source tiles per destination tile
+  const uint32_t pieces = K1p * R0;      // one 16-byte tile row each
+  for (uint32_t idx = blockIdx.x * 256 + threadIdx.x; idx < pieces; idx += gridDim.x * 256) {
+    const uint32_t ktp = idx / R0, r = idx - ktp * R0;
+    __attribute__((aligned(16))) unsigned char out[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) out[i] = 0;
+    for (uint32_t j = 0; j < g; ++j) {
+      const uint32_t kt = ktp * g + j;
+      if (kt >= K1) break;
+      if constexpr (SRC_BITS == 8) {
+        const char* sp = s + ((int64_t)kt * R0 + r) * rb;
+        for (uint32_t b = 0; b < rb; ++b) out[j * rb + b] = (unsigned char)sp[b];
+      } else {
+        const char* sp = s + ((int64_t)kt * R0 + r) * (rb / 2);
+        for (uint32_t b = 0; b < rb / 2; ++b) {
+          const int v = (signed char)sp[b];
+          out[j * rb + 2 * b] = (unsigned char)(((v << 28) >> 28) & 0xFF);   // low nibble first, sign-extended
+          out[j * rb + 2 * b + 1] = (unsigned char)((v >> 4) & 0xFF);
+        }
+      }
+    }
+    *reinterpret_cast<v4u_rt*>(d + (int64_t)idx * 16) = *reinterpret_cast<const v4u_rt*>(out);
+  }
+}
+}  // namespace
+
+void retile_rows(const char* src, int64_t src_stride, int panels, int R0, int rb, int K1, int src_bits,
+                 char* dst, hipStream_t stream) {
+  const int g = 16 / rb;
+  const uint32_t K1p = (uint32_t)((K1 + g - 1) / g);
+  const int64_t dst_stride = (int64_t)K1p * R0 * 16;
+  const uint32_t per_panel = (uint32_t)std::min<int64_t>(((int64_t)K1p * R0 + 255) / 256, 64);
+  if (src_bits == 4) {
+    uk::launch(2, retile_rows_kernel<4>, dim3(per_panel, (uint32_t)panels), dim3(256), 0, stream, src, src_stride,
+               dst, dst_stride, (uint32_t)R0, (uint32_t)rb, (uint32_t)K1, K1p);
+  } else {
+    uk::launch(2, retile_rows_kernel<8>, dim3(per_panel, (uint32_t)panels), dim3(256), 0, stream, src, src_stride,
+               dst, dst_stride, (uint32_t)R0, (uint32_t)rb, (uint32_t)K1, K1p);
+  }
+}
+
 int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base_out) {
   if (g_no_alloc || bytes == 0 || bytes > ((size_t)2 << 30)) return 1;
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -438,4 +489,67 @@ extern "C" int iree_uk_amd_hip_launch_mmt4d_mfma(const iree_uk_mmt4d_params_t* p
     case Elem::kBF16BF16: return uk_mfma::launch_bf16bf16(pr, forced_variant, stream, kernel_name);
   }
   return -1;
+}
+
+// Tile rows under 16 bytes that the matrix-core kernels do not take as they
+// are (one-byte rows; rows of 2, 4 or 8 bytes in tiles whose height is not a
+// multiple of the 16 / rb rows a 16-byte piece spans; f8 rows under 16 bytes):
+// both operands are regrouped along K into tiles of the same height with
+// 16-byte rows, in the buffer the library keeps for expanded weights, and the
+// call goes on with K0 = 16 bytes. The K order of the products is unchanged and
+// the zero bytes that fill up the last tile pair zero with zero, so integers
+// come out the same and floats as the matrix-core kernels give them for the
+// wider tile. Returns a HIP status, or a negative value when the call is not
+// served this way (nothing launched then).
+extern "C" int iree_uk_amd_hip_launch_mmt4d_retiled(const iree_uk_mmt4d_params_t* p,
+                                                    const iree_uk_amd_rowmajor_out_t* rowmajor,
+                                                    void* stream_v, const char** kernel_name) {
+  const uint32_t type = p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK;
+  Elem e = Elem::kS16;
+  int eb, ob;
+  if (type == IREE_UK_FLAG_MMT4D_TYPE_S16S16S32) {
+    eb = 2;
+  } else if (!elem_of(p->flags, &e, &eb, &ob)) {
+    return -1;
+  }
+  const int64_t rb = (int64_t)p->K0 * eb;
+  if (rb != 1 && rb != 2 && rb != 4 && rb != 8) return -1;
+  if (p->M0 < 1 || p->N0 < 1 || p->M0 > 64 || p->N0 > 64) return -1;
+  // A shape the kernels take as it is has been declined for another reason
+  // (strides, spans), which the regrouping does not change.
+  const bool whole_rows = rb >= 2 && p->M0 % (16 / rb) == 0 && p->N0 % (16 / rb) == 0;
+  if (whole_rows && (type == IREE_UK_FLAG_MMT4D_TYPE_S16S16S32 || e != Elem::kF8)) return -1;
+  if (type == IREE_UK_FLAG_MMT4D_TYPE_S16S16S32) {
+    // (what the s16 kernel asks for: K in whole steps of 64 elements, more than 32 rows and columns)
+    const int64_t k_tiles = ((int64_t)p->K + 16 / rb - 1) / (16 / rb);
+    if ((k_tiles * 8) % 64 != 0 || (int64_t)p->M * p->M0 <= 32 || (int64_t)p->N * p->N0 <= 32) return -1;
+  }
+  if (p->M <= 0 || p->N <= 0 || p->K <= 0 || p->M >= 65536 || p->N >= 65536) return -1;
+  // The two passes over the operands cost a few microseconds: from about 256^3
+  // multiply-adds on that is less than the scalar kernel loses.
+  if ((double)p->M * p->M0 * (double)p->N * p->N0 * (double)p->K * p->K0 < 16777216.0) return -1;
+  const int g = (int)(16 / rb);
+  const int64_t K1p = ((int64_t)p->K + g - 1) / g;
+  const int64_t lhs_bytes = (int64_t)p->M * K1p * p->M0 * 16, rhs_bytes = (int64_t)p->N * K1p * p->N0 * 16;
+  if (K1p * p->M0 * 16 >= (1ll << 31) || K1p * p->N0 * 16 >= (1ll << 31) || K1p >= (1ll << 31)) return -1;
+  hipStream_t stream = (hipStream_t)stream_v;
+  char* ws = nullptr;
+  if (uk_mfma::acquire_expand_workspace((size_t)(lhs_bytes + rhs_bytes), stream, &ws) != 0) return -1;
+  uk_mfma::retile_rows((const char*)p->lhs_buffer + p->lhs_offset * eb, p->lhs_stride0 * eb, (int)p->M, p->M0,
+                       (int)rb, (int)p->K, 8, ws, stream);
+  uk_mfma::retile_rows((const char*)p->rhs_buffer + p->rhs_offset * eb, p->rhs_stride0 * eb, (int)p->N, p->N0,
+                       (int)rb, (int)p->K, 8, ws + lhs_bytes, stream);
+  iree_uk_mmt4d_params_t q = *p;
+  q.K0 = 16 / eb;
+  q.K = (iree_uk_index_t)K1p;
+  q.lhs_buffer = ws;
+  q.lhs_offset = 0;
+  q.lhs_stride0 = K1p * p->M0 * q.K0;
+  q.rhs_buffer = ws + lhs_bytes;
+  q.rhs_offset = 0;
+  q.rhs_stride0 = K1p * p->N0 * q.K0;
+  const char* inner = nullptr;
+  const int st = iree_uk_amd_hip_launch_mmt4d_mfma(&q, rowmajor, stream_v, 0, &inner);
+  if (st >= 0) *kernel_name = "mmt4d_mfma_retiled";
+  return st;
 }

@@ -159,6 +159,14 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
 // iree_uk_amd_mmt4d_no_alloc, while the stream is being captured into a graph,
 // or when the allocation fails.
 int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base);
+// Regroups the K tiles of an operand so that every tile row holds 16 bytes:
+// `panels` panels of K1 tiles of R0 rows of `rb` bytes (rb = 1, 2, 4 or 8; panel
+// n at src + n * src_stride) become ceil(K1 * rb / 16) tiles of R0 rows of 16
+// bytes at dst + n * (that count * R0 * 16), the last one filled up with zero
+// bytes. src_bits = 4: the source holds signed nibbles, low nibble first, half
+// as many bytes, and `rb` counts the bytes they widen to. dst 16-byte aligned.
+void retile_rows(const char* src, int64_t src_stride, int panels, int R0, int rb, int K1, int src_bits,
+                 char* dst, hipStream_t stream);
 // K slices set with iree_uk_amd_set_k_slices on this thread; 0 = choose.
 int k_slices_override();
 // 1: the calling thread has declared its weights streamed from HBM

@@ -80,6 +80,36 @@ int launch_s8s4(const Problem& p, hipStream_t stream, const char** name) {
       // (not served as s8: the thin kernel below reads the packed weights)
     }
   }
+  // Tile rows under 16 elements in a tile the s8 kernels do not take (arm64's
+  // Mx16x2 with M = 1, 2, 4: arch/arm_64/mmt4d_arm_64_base.c:296): both operands
+  // are regrouped along K into 16-byte rows, the weights widened on the way.
+  if (rows_m >= kExpandFromRows && p.rb < 16 && p.rb >= 2 && p.M1 > 0 && p.M1 < 65536 && p.N1 > 0 &&
+      p.N1 < 65536 && !iree_uk_amd_hip_mmt4d_mfma_supported(p.M0, p.N0, p.rb, IREE_UK_FLAG_MMT4D_TYPE_S8S8S32) &&
+      iree_uk_amd_hip_mmt4d_mfma_supported(p.M0, p.N0, 16, IREE_UK_FLAG_MMT4D_TYPE_S8S8S32)) {
+    const int g = 16 / p.rb;
+    const int64_t K1p = ((int64_t)p.K1 + g - 1) / g;
+    const int64_t lhs_bytes = (int64_t)p.M1 * K1p * p.M0 * 16, rhs_bytes = (int64_t)p.N1 * K1p * p.N0 * 16;
+    char* ws = nullptr;
+    if (K1p * 64 * 16 < (1ll << 31) &&
+        acquire_expand_workspace((size_t)(lhs_bytes + rhs_bytes), stream, &ws) == 0) {
+      retile_rows(p.lhs, p.lhs_stride, p.M1, p.M0, p.rb, p.K1, 8, ws, stream);
+      retile_rows(p.rhs, p.rhs_stride, p.N1, p.N0, p.rb, p.K1, 4, ws + lhs_bytes, stream);
+      Problem q = p;
+      q.lhs = ws;
+      q.lhs_stride = K1p * p.M0 * 16;
+      q.rhs = ws + lhs_bytes;
+      q.rhs_stride = K1p * p.N0 * 16;
+      q.K1 = (int32_t)K1p;
+      q.rb = 16;
+      q.lrb = 4;
+      const char* s8_name = nullptr;
+      const int st = launch_s8(q, 0, stream, &s8_name);
+      if (st >= 0) {
+        *name = "mmt4d_mfma_s8s4_expanded";
+        return st;
+      }
+    }
+  }
   if (p.rb < 16) return -1;  // the thin kernel unpacks 16 nibbles per lane: tile rows of 16 and more
   int st;
   if (rows_m <= 16) {
