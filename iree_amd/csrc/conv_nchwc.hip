@@ -233,12 +233,18 @@ int launch_mfma(const ConvArgs& a, int64_t N, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+// Workgroups a launch with TW panels and TO output-channel blocks per wave has.
+int64_t mfma_blocks(const ConvArgs& a, int64_t N, int tw, int to) {
+  const int64_t px_chunks = uk::ceil_div(a.OH * a.OW, (int64_t)16 * tw);
+  return N * uk::ceil_div(a.OC, (int64_t)to) * uk::ceil_div(px_chunks, (int64_t)(kThreads / 64));
+}
+
 template <int TO>
-int launch_mfma_for_pixels(const ConvArgs& a, int64_t N, hipStream_t stream) {
+int launch_mfma_for_pixels(const ConvArgs& a, int64_t N, hipStream_t stream, bool one_panel) {
   const int64_t pixels = a.OH * a.OW;
   // Two panels per wave: four measured no faster (608 against 583 us on a 3x3
   // 256 -> 256 channel layer at 56x56) and leave fewer, longer work items.
-  if (pixels > 16) return launch_mfma<2, TO>(a, N, stream);
+  if (pixels > 16 && !one_panel) return launch_mfma<2, TO>(a, N, stream);
   return launch_mfma<1, TO>(a, N, stream);
 }
 
@@ -280,9 +286,24 @@ extern "C" int iree_uk_amd_hip_launch_conv_nchwc(const iree_uk_conv_nchwc_params
     // than two would (each input piece then meets four filter tiles: 583 -> 554
     // us on a 3x3 256 -> 256 channel layer at 56x56), else two, else one.
     const bool four = a.OC > 2 && uk::ceil_div(a.OC, (int64_t)4) * 4 == uk::ceil_div(a.OC, (int64_t)2) * 2;
-    int st = four       ? launch_mfma_for_pixels<4>(a, p->N, stream)
-             : a.OC > 1 ? launch_mfma_for_pixels<2>(a, p->N, stream)
-                        : launch_mfma_for_pixels<1>(a, p->N, stream);
+    // A layer with few output pixels (the last stages of an image network at
+    // batch 1: 512 -> 512 channels, 7x7 outputs) leaves most compute units
+    // without a workgroup at those sizes: the wave's share shrinks, first in
+    // output channels, then in pixels, until the workgroups outnumber the units
+    // (8 -> 32 workgroups on that layer: 189 -> 72 us; 256 -> 256 channels at 56x56, batch 1: 97 -> 70 us).
+    int to = four ? 4 : a.OC > 1 ? 2 : 1;
+    int tw = a.OH * a.OW > 16 ? 2 : 1;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+      (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    }
+    while (mfma_blocks(a, p->N, tw, to) < cus && (to > 1 || tw > 1)) {
+      if (to > 1) to /= 2;
+      else tw = 1;
+    }
+    int st = to == 4   ? launch_mfma_for_pixels<4>(a, p->N, stream, tw == 1)
+             : to == 2 ? launch_mfma_for_pixels<2>(a, p->N, stream, tw == 1)
+                       : launch_mfma_for_pixels<1>(a, p->N, stream, tw == 1);
     if (st >= 0) {
       *kernel_name = "conv_nchwc_mfma";
       return st;

@@ -467,8 +467,10 @@ class Runner:
             # (TRANSPOSE_INNER + TRANSPOSE_OUTER -> [N1][K1][N0][K0],
             # tests/e2e/linalg/pack_i8.mlir:48-68) for the tile shapes of the
             # other workloads, and the reference's 16x2 s8 tile from [M][K].
-            # Every form moves more than the 256 MB memory-side cache holds, so
-            # that repeated launches time HBM and not that cache.
+            # Every form moves more than the 256 MB memory-side cache holds, but
+            # its source alone fits, and launches on the same buffers one after
+            # the other read it from there: bench.py times each form a second
+            # time with that cache emptied before every launch.
             forms = [  # (op name, torch dtype, pack type, element bytes, rows, cols, N0 or M0, K0, [K][N]?)
                 ("rhs_kn_f16_16x16", torch.float16, uk.PACK_TYPE_F16F16, 2, 8192, 16384, 16, 16, True),
                 ("rhs_kn_s8_16x8", torch.int8, uk.PACK_TYPE_I8I8, 1, 8192, 28672, 16, 8, True),
