@@ -230,3 +230,45 @@ def test_decode_without_pack_row_major_activations_are_m0_1_tiles(gpu):
     prod = (act.cpu().to(torch.int64) @ w.cpu().to(torch.int64).T).to(torch.int32)
     want = (prod.float() * rs.cpu()[:, None]) * cs.cpu()[None, :]
     assert torch.equal(y.cpu(), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tf,M0,N0,K0,M1,N1,K1,name", [
+    (uk.MMT4D_TYPE_S8S4S32, 16, 16, 16, 33, 9, 12, "mmt4d_mfma_s8s4_expanded"),
+    (uk.MMT4D_TYPE_S16S8S32, 16, 16, 2, 9, 10, 64, "mmt4d_mfma_128x128_s16_widened"),
+    (uk.MMT4D_TYPE_S16U4S32, 1, 32, 8, 130, 5, 16, "mmt4d_mfma_128x128_s16_widened"),
+    (uk.MMT4D_TYPE_S8S8S32, 8, 8, 1, 33, 33, 272, "mmt4d_mfma_retiled")])
+def test_dequant_unpack_on_operands_the_library_prepares_first(gpu, oracle, tf, M0, N0, K0, M1, N1, K1, name):
+    """The calls whose operands the library widens or regroups before the
+    matrix-core kernels run (4-bit weights from 512 rows on, s16 x s8 / u4 from
+    128 rows and columns on, one-byte tile rows) through the fused entry point:
+    ragged row-major result, ACCUMULATE from the tiled buffer, both scales."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    lk, rk, ok = T.MMT4D_KINDS[tf]
+    for acc in (0, 1):
+        rows, cols = M1 * M0 - min(3, M0 - 1), N1 * N0 - min(5, N0 - 1)
+        pitch, off = cols + 3, 5 * acc
+        acc_stride, acc_off = N1 * M0 * N0 + 8, 4
+        c = T.Mmt4dCase(tf | 0x200 | (uk.MMT4D_ACCUMULATE if acc else 0), M1, N1, K1, M0, N0,
+                        K0, K1 * M0 * K0, K1 * N0 * K0, N1 * M0 * N0, 0, 0, 0)
+        rng = np.random.default_rng(77 + acc)
+        lhs, rhs, _ = T.make_mmt4d_buffers(c, rng)
+        acc_buf = rng.integers(-9, 9, acc_off + M1 * acc_stride).astype(np.int32)
+        acc_dense = np.concatenate([acc_buf[acc_off + i * acc_stride:][:N1 * M0 * N0] for i in range(M1)])
+        rs = rng.random(rows, dtype=np.float32) * 0.02 + 0.001
+        cs = rng.random(cols, dtype=np.float32) * 0.02 + 0.001
+        want_mat = _want(oracle, c, lhs, rhs, acc_dense if acc else None, rows, cols, rs, cs, ok)
+        out0 = rng.random(off + rows * pitch, dtype=np.float32)
+        want = out0.copy()
+        for i in range(rows):
+            want[off + i * pitch:off + i * pitch + cols] = want_mat[i]
+        d = [T.DeviceBytes(torch, x) for x in (lhs, rhs, acc_buf, out0, rs, cs)]
+        lib.mmt4d_dequant_unpack(
+            d[0].ptr, 0, c.lhs_stride0, d[1].ptr, 0, c.rhs_stride0,
+            d[2].ptr if acc else None, acc_off, acc_stride, d[3].ptr, off, pitch, rows, cols,
+            d[4].ptr, d[5].ptr, M1, N1, K1, M0, N0, K0, c.flags)
+        lib.synchronize()
+        assert lib.last_kernel_name() == name, lib.last_kernel_name()
+        got = d[3].numpy().view(np.float32)
+        assert np.array_equal(got.view(np.int32), want.view(np.int32)), (tf, acc)
