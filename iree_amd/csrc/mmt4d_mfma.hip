@@ -217,35 +217,90 @@ int acquire_ksplit_workspace(size_t partial_bytes, uint32_t n_counters, hipStrea
 namespace {
 typedef uint32_t v4u_rt __attribute__((ext_vector_type(4)));
 
-template <int SRC_BITS>
+// An unsigned integer of BYTES bytes, and the same read from any address.
+template <int BYTES> struct PieceOf;
+template <> struct PieceOf<1> { typedef uint8_t type; typedef uint8_t loaded; };
+template <> struct PieceOf<2> { typedef uint16_t type; typedef uint16_t loaded __attribute__((aligned(1))); };
+template <> struct PieceOf<4> { typedef uint32_t type; typedef uint32_t loaded __attribute__((aligned(1))); };
+template <> struct PieceOf<8> { typedef uint64_t type; typedef uint64_t loaded __attribute__((aligned(1))); };
+
+// Signed nibbles of the low BYTES bytes of v, low nibble first, as 2 * BYTES bytes.
+template <int BYTES>
+__device__ __forceinline__ uint64_t widen_nibbles(uint32_t v) {
+  uint64_t out = 0;
+#pragma unroll
+  for (int i = 0; i < 2 * BYTES; ++i) {
+    out |= (uint64_t)((uint32_t)__builtin_amdgcn_sbfe((int)v, 4 * i, 4) & 0xFFu) << (8 * i);
+  }
+  return out;
+}
+
+// One thread per 16-byte destination row: 16 / RB source tile rows of RB bytes
+// (SRC_BITS = 4: of RB / 2 bytes holding RB nibbles), one load each.
+template <int SRC_BITS, int RB>
 __global__ __launch_bounds__(256) void retile_rows_kernel(const char* src, int64_t src_stride, char* dst,
-                                                           int64_t dst_stride, uint32_t R0, uint32_t rb,
-                                                           uint32_t K1, uint32_t K1p) {
+                                                           int64_t dst_stride, uint32_t R0, uint32_t K1,
+                                                           uint32_t K1p) {
+  constexpr uint32_t G = 16 / RB;         // source tiles per destination tile
+  constexpr int SB = RB * SRC_BITS / 8;   // bytes of a source tile row
+  typedef typename PieceOf<RB>::type out_piece_t;
+  typedef typename PieceOf<SB>::loaded src_piece_t;
   const char* s = src + (int64_t)blockIdx.y * src_stride;
   char* d = dst + (int64_t)blockIdx.y * dst_stride;
-  const uint32_t g = 16 / rb;            // source tiles per destination tile
-  const uint32_t pieces = K1p * R0;      // one 16-byte tile row each
+  const uint32_t pieces = K1p * R0;
   for (uint32_t idx = blockIdx.x * 256 + threadIdx.x; idx < pieces; idx += gridDim.x * 256) {
     const uint32_t ktp = idx / R0, r = idx - ktp * R0;
-    __attribute__((aligned(16))) unsigned char out[16];
+    union {
+      v4u_rt v;
+      out_piece_t p[G];
+    } out;
+    out.v = v4u_rt{0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int i = 0; i < 16; ++i) out[i] = 0;
-    for (uint32_t j = 0; j < g; ++j) {
-      const uint32_t kt = ktp * g + j;
+    for (uint32_t j = 0; j < G; ++j) {
+      const uint32_t kt = ktp * G + j;
       if (kt >= K1) break;
+      const char* sp = s + ((int64_t)kt * R0 + r) * SB;
       if constexpr (SRC_BITS == 8) {
-        const char* sp = s + ((int64_t)kt * R0 + r) * rb;
-        for (uint32_t b = 0; b < rb; ++b) out[j * rb + b] = (unsigned char)sp[b];
+        out.p[j] = *reinterpret_cast<const src_piece_t*>(sp);
       } else {
-        const char* sp = s + ((int64_t)kt * R0 + r) * (rb / 2);
-        for (uint32_t b = 0; b < rb / 2; ++b) {
-          const int v = (signed char)sp[b];
-          out[j * rb + 2 * b] = (unsigned char)(((v << 28) >> 28) & 0xFF);   // low nibble first, sign-extended
-          out[j * rb + 2 * b + 1] = (unsigned char)((v >> 4) & 0xFF);
-        }
+        const uint32_t packed = *reinterpret_cast<const src_piece_t*>(sp);
+        out.p[j] = (out_piece_t)widen_nibbles<SB>(packed);
       }
     }
-    *reinterpret_cast<v4u_rt*>(d + (int64_t)idx * 16) = *reinterpret_cast<const v4u_rt*>(out);
+    *reinterpret_cast<v4u_rt*>(d + (int64_t)idx * 16) = out.v;
+  }
+}
+
+// One-byte tile rows in tiles whose height is a multiple of four: a thread
+// takes four rows of one destination tile, loads them as sixteen words (four
+// rows of one K position each) and transposes bytes in registers.
+__global__ __launch_bounds__(256) void retile_bytes_by_four_rows_kernel(const char* src, int64_t src_stride,
+                                                                         char* dst, int64_t dst_stride,
+                                                                         uint32_t R0, uint32_t K1, uint32_t K1p) {
+  typedef uint32_t u32_g __attribute__((aligned(1)));
+  const char* s = src + (int64_t)blockIdx.y * src_stride;
+  char* d = dst + (int64_t)blockIdx.y * dst_stride;
+  const uint32_t r4s = R0 / 4, items = K1p * r4s;
+  for (uint32_t idx = blockIdx.x * 256 + threadIdx.x; idx < items; idx += gridDim.x * 256) {
+    const uint32_t ktp = idx / r4s, r = (idx - ktp * r4s) * 4;
+    uint32_t w[16];
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j) {
+      const uint32_t kt = ktp * 16 + j;
+      w[j] = kt < K1 ? *reinterpret_cast<const u32_g*>(s + (int64_t)kt * R0 + r) : 0u;
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      const uint32_t pick = i | ((4 + i) << 8);   // byte i of the first word, byte i of the second
+      v4u_rt row;
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) {
+        const uint32_t lo = __builtin_amdgcn_perm(w[4 * q + 1], w[4 * q], pick);
+        const uint32_t hi = __builtin_amdgcn_perm(w[4 * q + 3], w[4 * q + 2], pick);
+        row[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+      }
+      *reinterpret_cast<v4u_rt*>(d + ((int64_t)ktp * R0 + r + i) * 16) = row;
+    }
   }
 }
 }  // namespace
@@ -255,14 +310,28 @@ void retile_rows(const char* src, int64_t src_stride, int panels, int R0, int rb
   const int g = 16 / rb;
   const uint32_t K1p = (uint32_t)((K1 + g - 1) / g);
   const int64_t dst_stride = (int64_t)K1p * R0 * 16;
-  const uint32_t per_panel = (uint32_t)std::min<int64_t>(((int64_t)K1p * R0 + 255) / 256, 64);
-  if (src_bits == 4) {
-    uk::launch(2, retile_rows_kernel<4>, dim3(per_panel, (uint32_t)panels), dim3(256), 0, stream, src, src_stride,
-               dst, dst_stride, (uint32_t)R0, (uint32_t)rb, (uint32_t)K1, K1p);
-  } else {
-    uk::launch(2, retile_rows_kernel<8>, dim3(per_panel, (uint32_t)panels), dim3(256), 0, stream, src, src_stride,
-               dst, dst_stride, (uint32_t)R0, (uint32_t)rb, (uint32_t)K1, K1p);
+  if (src_bits == 8 && rb == 1 && R0 % 4 == 0) {
+    const uint32_t per_panel = (uint32_t)std::min<int64_t>(((int64_t)K1p * (R0 / 4) + 255) / 256, 64);
+    uk::launch(2, retile_bytes_by_four_rows_kernel, dim3(per_panel, (uint32_t)panels), dim3(256), 0, stream, src,
+               src_stride, dst, dst_stride, (uint32_t)R0, (uint32_t)K1, K1p);
+    return;
   }
+  const uint32_t per_panel = (uint32_t)std::min<int64_t>(((int64_t)K1p * R0 + 255) / 256, 64);
+  const dim3 grid(per_panel, (uint32_t)panels), block(256);
+#define UK_RETILE(BITS, RB)                                                                              \
+  uk::launch(2, retile_rows_kernel<BITS, RB>, grid, block, 0, stream, src, src_stride, dst, dst_stride, \
+             (uint32_t)R0, (uint32_t)K1, K1p)
+  if (src_bits == 4) {
+    if (rb == 2) UK_RETILE(4, 2);
+    else if (rb == 4) UK_RETILE(4, 4);
+    else UK_RETILE(4, 8);
+  } else {
+    if (rb == 1) UK_RETILE(8, 1);
+    else if (rb == 2) UK_RETILE(8, 2);
+    else if (rb == 4) UK_RETILE(8, 4);
+    else UK_RETILE(8, 8);
+  }
+#undef UK_RETILE
 }
 
 int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base_out) {
