@@ -380,6 +380,29 @@ int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base_out) 
 
 }  // namespace uk_mfma
 
+extern "C" IREE_UK_AMD_EXPORT int64_t iree_uk_amd_workspace_bytes(void) {
+  int64_t total = 0;
+  for (const OwnedWorkspace& w : g_workspaces) total += (int64_t)w.partial_bytes + (int64_t)w.n_counters * 4;
+  for (const OwnedWorkspace& w : g_expand_workspaces) total += (int64_t)w.partial_bytes;
+  return total;
+}
+
+extern "C" IREE_UK_AMD_EXPORT int iree_uk_amd_release_workspaces(void) {
+  int status = 0, current = 0;
+  (void)hipGetDevice(&current);
+  for (OwnedWorkspaces* pool : {&g_workspaces, &g_expand_workspaces}) {
+    for (OwnedWorkspace& w : *pool) {
+      if (!w.base) continue;
+      (void)hipSetDevice(w.device);
+      const hipError_t err = hipFree(w.base);   // waits for the device: nothing in flight still uses it
+      if (err != hipSuccess && !status) status = (int)err;
+    }
+    pool->clear();
+  }
+  (void)hipSetDevice(current);
+  return status;
+}
+
 extern "C" void iree_uk_amd_hip_set_no_alloc(int on) { g_no_alloc = on != 0; }
 
 extern "C" IREE_UK_AMD_EXPORT void iree_uk_amd_set_k_slices(int n) { g_k_slices = n > 0 ? n : 0; }

@@ -190,6 +190,8 @@ class UKernelLibrary:
         L.iree_uk_amd_staging_bytes.restype = _i64
         L.iree_uk_amd_device_alloc_count.restype = _i64
         L.iree_uk_amd_release_staging.restype = ctypes.c_int
+        L.iree_uk_amd_workspace_bytes.restype = _i64
+        L.iree_uk_amd_release_workspaces.restype = ctypes.c_int
         L.iree_uk_amd_timing_end.argtypes = [_vp, _vp, ctypes.c_int]
         L.iree_uk_amd_timing_end.restype = ctypes.c_int
         L.iree_uk_amd_probe_mfma_peak.argtypes = [_u32, _vp, _i64, ctypes.c_int, ctypes.c_int, _vp,
@@ -429,6 +431,14 @@ class UKernelLibrary:
     def device_alloc_count(self) -> int:
         """hipMalloc calls the library has made in this process so far."""
         return int(self.lib.iree_uk_amd_device_alloc_count())
+
+    def workspace_bytes(self) -> int:
+        """Bytes of K-split workspaces and prepared-operand buffers the calling thread holds."""
+        return int(self.lib.iree_uk_amd_workspace_bytes())
+
+    def release_workspaces(self) -> int:
+        """Frees them; 0 or a hipError_t value."""
+        return int(self.lib.iree_uk_amd_release_workspaces())
 
     def release_staging(self) -> int:
         """Frees the calling thread's staging arena; 0 or a hipError_t value."""

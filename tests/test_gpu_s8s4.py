@@ -150,3 +150,36 @@ def test_s8s4_prefill_shape_equals_integer_product(gpu):
         # (every partial sum is an integer below 2^53: the f64 product is exact)
         want = (a @ b.T).to(torch.int64).reshape(M1, M0, N1, N0).permute(0, 2, 1, 3) + init.to(torch.int64)
         assert torch.equal(out.to(torch.int64), want), rep
+
+
+@pytest.mark.gpu
+def test_prepared_operand_buffer_is_reported_and_can_be_released(gpu):
+    """The buffer for the expanded weights is kept for the next call on the same
+    stream, shows in iree_uk_amd_workspace_bytes, is freed by
+    iree_uk_amd_release_workspaces, and a later call allocates it again."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    M0, N0, K0, M1, N1, K1 = 16, 16, 16, 32, 16, 8
+    lhs = torch.randint(-128, 128, (M1 * K1 * M0 * K0,), device="cuda", dtype=torch.int8)
+    rhs = torch.randint(0, 256, (N1 * K1 * N0 * K0 // 2,), device="cuda", dtype=torch.uint8)
+    out = torch.zeros(M1 * N1 * M0 * N0, device="cuda", dtype=torch.int32)
+
+    def call():
+        lib.mmt4d(lhs.data_ptr(), 0, K1 * M0 * K0, rhs.data_ptr(), 0, K1 * N0 * K0, out.data_ptr(), 0,
+                  N1 * M0 * N0, M1, N1, K1, M0, N0, K0, TF | 0x200)
+        lib.synchronize()
+        assert lib.last_kernel_name() == "mmt4d_mfma_s8s4_expanded"
+        return out.clone()
+
+    lib.release_workspaces()
+    assert lib.workspace_bytes() == 0
+    first = call()
+    held = lib.workspace_bytes()
+    assert held >= N1 * K1 * N0 * K0
+    allocs = lib.device_alloc_count()
+    second = call()
+    assert lib.device_alloc_count() == allocs and lib.workspace_bytes() == held   # reused, not grown
+    assert lib.release_workspaces() == 0 and lib.workspace_bytes() == 0
+    third = call()
+    assert lib.workspace_bytes() == held
+    assert torch.equal(first, second) and torch.equal(first, third)
