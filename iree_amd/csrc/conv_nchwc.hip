@@ -19,11 +19,18 @@
 //     generic path bit for bit.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <type_traits>
 
 #include "uk_device_common.h"
 #include "uk_hip_abi.h"
 #include "uk_launch.h"
+
+namespace uk_mfma {
+// mmt4d_mfma.hip: a buffer the library keeps per host thread and stream (0 and
+// the pointer, or 1 when there is none to be had).
+int acquire_expand_workspace(size_t bytes, hipStream_t stream, char** base);
+}  // namespace uk_mfma
 
 namespace {
 
@@ -40,6 +47,16 @@ struct ConvArgs {
   int32_t k0, c0, stride_h, stride_w;
   uint32_t accumulate;
   int64_t total;
+  // conv_nchwc_mfma only: IC_outer split over `ic_slices` workgroups per output
+  // block (1 = none). Slice s takes ic_per consecutive values of ic_outer and
+  // stores its sums, as if it were the whole call without ACCUMULATE, at
+  // `partial` + s * partial_stride with the output's own strides;
+  // conv_reduce_slices_kernel adds the slices up in order.
+  int64_t N;
+  int32_t ic_slices;
+  int64_t ic_per;
+  float* partial;
+  int64_t partial_stride;
 };
 
 __global__ __launch_bounds__(kThreads) void conv_nchwc_generic_kernel(ConvArgs a) {
@@ -107,8 +124,13 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
   const uint32_t nb = gridDim.x, xcd = blockIdx.x & 7u;
   int64_t t = (int64_t)(xcd * (nb / 8u) + min(xcd, nb % 8u) + (blockIdx.x >> 3));
   const int64_t pxg = t % px_groups; t /= px_groups;
-  const int64_t occ = t % oc_chunks;
-  const int64_t n = t / oc_chunks;
+  const int64_t occ = t % oc_chunks; t /= oc_chunks;
+  const int64_t n = t % a.N;
+  const int64_t slice = t / a.N;
+  const int64_t ic0 = slice * a.ic_per;
+  const int64_t ic_count = a.ic_slices > 1 ? min(a.ic_per, a.IC - ic0) : a.IC;
+  float* const out_base = a.ic_slices > 1 ? a.partial + slice * a.partial_stride : a.out;
+  const bool accumulate = a.ic_slices > 1 ? false : a.accumulate != 0;
   const int64_t pxc_raw = pxg * 4 + wave;
   const bool wave_ok = pxc_raw < px_chunks;
   const int64_t pxc = wave_ok ? pxc_raw : px_chunks - 1;
@@ -123,20 +145,20 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
     const int64_t px = pxc * (16 * TW) + tw * 16 + r;
     const int64_t px_in = px < pixels ? px : pixels - 1;
     const int64_t oh = px_in / a.OW, ow = px_in - oh * a.OW;
-    pa[tw] = a.in + n * a.in_sn + (oh * a.stride_h) * a.in_sh + (ow * a.stride_w) * a.c0 + 4 * q;
+    pa[tw] = a.in + n * a.in_sn + ic0 * a.in_sic + (oh * a.stride_h) * a.in_sh + (ow * a.stride_w) * a.c0 + 4 * q;
 #pragma unroll
     for (int to = 0; to < TO; ++to) {
       const int64_t oc = occ * TO + to;
       const int64_t oc_in = oc < a.OC ? oc : a.OC - 1;
       ok[tw][to] = wave_ok && px < pixels && oc < a.OC;
-      po[tw][to] = a.out + n * a.out_sn + oc_in * a.out_soc + oh * a.out_soh + ow * 16 + 4 * q;
+      po[tw][to] = out_base + n * a.out_sn + oc_in * a.out_soc + oh * a.out_soh + ow * 16 + 4 * q;
     }
   }
   // Loader lanes (waves 0..TO-1): wave `wave` copies channel block occ*TO+wave,
   // lane l the 16 bytes [ci = l / 4][ko = 4 * (l % 4) ..].
   const bool loader = wave < TO;
   const int64_t oc_ld = min(occ * TO + (loader ? wave : 0), a.OC - 1);
-  const float* pf = a.flt + oc_ld * a.f_soc + lane * 4;
+  const float* pf = a.flt + oc_ld * a.f_soc + ic0 * a.f_sic + lane * 4;
   const int f_dst = (loader ? wave : 0) * kFilterTile + (lane >> 2) * kFilterRow + (lane & 3) * 4;
   const int f_src = (4 * q) * kFilterRow + r;   // + to * kFilterTile + w * kFilterRow
 
@@ -146,13 +168,13 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
 #pragma unroll
     for (int to = 0; to < TO; ++to) {
       acc[tw][to] = v4f{0.f, 0.f, 0.f, 0.f};
-      if (a.accumulate && ok[tw][to]) acc[tw][to] = *reinterpret_cast<const v4f_a4*>(po[tw][to]);
+      if (accumulate && ok[tw][to]) acc[tw][to] = *reinterpret_cast<const v4f_a4*>(po[tw][to]);
     }
 
   // Within one (ic_outer, fh) consecutive steps follow each other at 16 input
   // floats and 256 filter floats.
   const int64_t taps = a.FW * (a.c0 / 16);
-  const int64_t steps = a.IC * a.FH * taps;
+  const int64_t steps = ic_count * a.FH * taps;
   if (steps > 0) {
     int64_t ic = 0, fh = 0, tap = 0;  // the step the next prefetch loads
     v4f av[2][TW];
@@ -168,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) av[B][tw] = *reinterpret_cast<const v4f_a4*>(pa[tw] + ao);
       // Advance, staying on the last step once it is reached.
-      if (!(ic == a.IC - 1 && fh == a.FH - 1 && tap == taps - 1)) {
+      if (!(ic == ic_count - 1 && fh == a.FH - 1 && tap == taps - 1)) {
         if (++tap == taps) {
           tap = 0;
           if (++fh == a.FH) {
@@ -221,15 +243,40 @@ __global__ __launch_bounds__(kThreads) void conv_nchwc_mfma_kernel(ConvArgs a, i
       if (ok[tw][to]) *reinterpret_cast<v4f_a4*>(po[tw][to]) = acc[tw][to];
 }
 
+// out = (ACCUMULATE ? out : 0) + slice 0 + slice 1 + ..., four channels per thread.
+__global__ __launch_bounds__(kThreads) void conv_reduce_slices_kernel(ConvArgs a) {
+  const int64_t quads = a.total / 4;   // k0 = 16: four quads per pixel
+  for (int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x; idx < quads;
+       idx += (int64_t)gridDim.x * kThreads) {
+    int64_t t = idx;
+    const int64_t q = t % 4; t /= 4;
+    const int64_t ow = t % a.OW; t /= a.OW;
+    const int64_t oh = t % a.OH; t /= a.OH;
+    const int64_t oc = t % a.OC;
+    const int64_t n = t / a.OC;
+    const int64_t off = n * a.out_sn + oc * a.out_soc + oh * a.out_soh + ow * 16 + 4 * q;
+    v4f sum = a.accumulate ? *reinterpret_cast<const v4f_a4*>(a.out + off) : v4f{0.f, 0.f, 0.f, 0.f};
+    for (int32_t s = 0; s < a.ic_slices; ++s) {
+      sum += *reinterpret_cast<const v4f_a4*>(a.partial + s * a.partial_stride + off);
+    }
+    *reinterpret_cast<v4f_a4*>(a.out + off) = sum;
+  }
+}
+
 template <int TW, int TO>
 int launch_mfma(const ConvArgs& a, int64_t N, hipStream_t stream) {
   const int64_t px_chunks = uk::ceil_div(a.OH * a.OW, (int64_t)16 * TW);
   const int64_t px_groups = uk::ceil_div(px_chunks, (int64_t)(kThreads / 64));
   const int64_t oc_chunks = uk::ceil_div(a.OC, (int64_t)TO);
-  const int64_t blocks = N * oc_chunks * px_groups;
+  const int64_t blocks = N * oc_chunks * px_groups * a.ic_slices;
   if (blocks >= (1ll << 31)) return -1;
   uk::launch(3, conv_nchwc_mfma_kernel<TW, TO>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
              a, px_chunks, px_groups, oc_chunks);
+  if (a.ic_slices > 1) {
+    const int64_t rblocks = uk::ceil_div(a.total / 4, (int64_t)kThreads);
+    uk::launch(3, conv_reduce_slices_kernel, dim3((uint32_t)std::min<int64_t>(rblocks, 4096)), dim3(kThreads), 0,
+               stream, a);
+  }
   return (int)hipGetLastError();
 }
 
@@ -276,6 +323,11 @@ extern "C" int iree_uk_amd_hip_launch_conv_nchwc(const iree_uk_conv_nchwc_params
   a.k0 = p->k0; a.c0 = p->c0; a.stride_h = p->stride_h; a.stride_w = p->stride_w;
   a.accumulate = (p->flags & IREE_UK_FLAG_CONV_NCHWC_ACCUMULATE) != 0;
   a.total = p->N * p->OC_outer * p->OH * p->OW * (int64_t)p->k0;
+  a.N = p->N;
+  a.ic_slices = 1;
+  a.ic_per = p->IC_outer;
+  a.partial = nullptr;
+  a.partial_stride = 0;
   if (a.total == 0) {
     *kernel_name = "";
     return 0;
@@ -300,6 +352,29 @@ extern "C" int iree_uk_amd_hip_launch_conv_nchwc(const iree_uk_conv_nchwc_params
     while (mfma_blocks(a, p->N, tw, to) < cus && (to > 1 || tw > 1)) {
       if (to > 1) to /= 2;
       else tw = 1;
+    }
+    // Still fewer workgroups than half the units: IC_outer is split over
+    // several workgroups per output block, whose sums meet in a buffer the
+    // library keeps and are added up in slice order by a second kernel (the
+    // same result on every run; 512 -> 512 channels at 7x7, batch 1: 72 -> 17
+    // us). While the stream is being captured into a graph there is no buffer
+    // to be had, and the call runs unsplit.
+    const int64_t blocks0 = mfma_blocks(a, p->N, tw, to);
+    const int64_t steps_per_ic = a.FH * a.FW * (a.c0 / 16);
+    if (blocks0 * 2 <= cus && a.IC >= 2 && a.out_sn >= 0 && a.out_soc >= 0 && a.out_soh >= 0) {
+      int64_t slices = std::min<int64_t>(std::min<int64_t>(a.IC, cus / blocks0), 16);
+      while (slices > 1 && uk::ceil_div(a.IC, slices) * steps_per_ic < 8) --slices;
+      const int64_t ic_per = uk::ceil_div(a.IC, std::max<int64_t>(slices, 1));
+      slices = uk::ceil_div(a.IC, ic_per);
+      const int64_t span = (p->N - 1) * a.out_sn + (a.OC - 1) * a.out_soc + (a.OH - 1) * a.out_soh + a.OW * 16;
+      char* ws = nullptr;
+      if (slices > 1 && span * slices * 4 <= (64ll << 20) &&
+          uk_mfma::acquire_expand_workspace((size_t)(span * slices * 4), stream, &ws) == 0) {
+        a.ic_slices = (int32_t)slices;
+        a.ic_per = ic_per;
+        a.partial = (float*)ws;
+        a.partial_stride = span;
+      }
     }
     int st = to == 4   ? launch_mfma_for_pixels<4>(a, p->N, stream, tw == 1)
              : to == 2 ? launch_mfma_for_pixels<2>(a, p->N, stream, tw == 1)
