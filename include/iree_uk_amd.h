@@ -502,12 +502,14 @@ IREE_UK_AMD_EXPORT int iree_uk_amd_timing_end(double* elapsed_us, int* kinds,
 IREE_UK_AMD_EXPORT int64_t iree_uk_amd_staging_bytes(void);
 IREE_UK_AMD_EXPORT int iree_uk_amd_release_staging(void);
 
-/* Device buffers that iree_uk_mmt4d keeps per calling thread and stream beyond
- * a call: the workspace of the thin kernels' K split over workgroups (a few
- * megabytes) and the buffer for operands the library prepares before the
- * matrix-core kernels run (4-bit weights expanded to s8 from 512 rows on, the
- * right-hand side of s16 x s8 / s16 x u4 widened to s16, narrow tile rows
- * regrouped along K: as large as the prepared operands, at most 2 GiB).
+/* Device buffers that iree_uk_mmt4d and iree_uk_conv_nchwc keep per calling
+ * thread and stream beyond a call: the workspace of the thin kernels' K split
+ * over workgroups (a few megabytes) and the buffer for operands the library
+ * prepares before the matrix-core kernels run (4-bit weights expanded to s8
+ * from 512 rows on, the right-hand side of s16 x s8 / s16 x u4 widened to s16,
+ * narrow tile rows regrouped along K: as large as the prepared operands, at
+ * most 2 GiB), which also holds the partial sums of a convolution whose input
+ * channels are split over workgroups (at most 64 MB).
  * workspace_bytes reports what the calling thread holds; release_workspaces
  * frees it after waiting for the device (0 or a hipError_t value; a later
  * call allocates again), and so does the thread's end. Calls through
