@@ -304,7 +304,8 @@ int launch_narrow(const Problem& p, int kt_count, hipStream_t stream) {
 // `swapped`: the caller's problem is N-thin and is computed as its transpose
 // (out^T = rhs * lhs^T): the kernel's rows are the caller's columns.
 template <Elem E, int RBC, int TM, int TN, int KSPLIT, int D>
-int launch_thin(const Problem& caller, bool swapped, hipStream_t stream, bool allow_k_slices = false) {
+int launch_thin(const Problem& caller, bool swapped, hipStream_t stream, bool allow_k_slices = false,
+                int max_k_slices = 8) {
   constexpr int OBYTES = ElemTraits<E>::Out::kOutBytes;
   Problem p = caller;
   if (swapped) {
@@ -383,7 +384,7 @@ int launch_thin(const Problem& caller, bool swapped, hipStream_t stream, bool al
     if (k_slices_override() > 0) {
       kslices = k_slices_override();
     } else if (cus > 0 && 2 * blocks <= cus) {
-      kslices = std::min<int64_t>(8, cus / blocks);
+      kslices = std::min<int64_t>(max_k_slices, cus / blocks);
     }
     kslices = std::max<int64_t>(1, std::min<int64_t>(kslices, a.steps / (4 * KSPLIT)));
     if (blocks * kslices >= (1ll << 31)) kslices = 1;
@@ -753,7 +754,14 @@ int launch_class(const Problem& p, int forced, hipStream_t stream, const char** 
     // Few 64x64 blocks and a long K: the barrier-free kernel with a 64x64
     // block per workgroup, whose four waves split K.
     if constexpr (RBC >= 8) {
-      int st = launch_thin<E, RBC, 4, 4, 4, 2>(p, false, stream);
+      // K over workgroups too where the 64x64 blocks are fewer than half the
+      // compute units and K is long: the meeting of the slices costs about 15
+      // us with blocks of this size, so only from 24 KB of K per row on (f16
+      // 128 x 128 x 65536, four blocks: 177 -> 52 us; 256 x 256 x 32768: 80 ->
+      // 35; 512 x 512 x 16384: 44 -> 27; with 8 KB of K per row, 384 x 384 x
+      // 4096, it loses: 16 -> 20 us).
+      const bool long_k = ((int64_t)p.K1 << p.lrb) >= 24576;
+      int st = launch_thin<E, RBC, 4, 4, 4, 2>(p, false, stream, long_k, 32);
       if (st >= 0) { *name = "mmt4d_mfma_64x64_ksplit"; return st; }
     }
     choice = 3;

@@ -178,3 +178,25 @@ def test_streamed_weights_hint_changes_no_result(gpu, tf, M0, N0, K0, n_thin):
         lib.set_k_slices(0)
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
     assert bool(outs[0].any())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tf,K0", [(uk.MMT4D_TYPE_S8S8S32, 16), (uk.MMT4D_TYPE_F16F16F32, 8)])
+def test_few_blocks_and_a_long_k_split_k_over_workgroups(gpu, oracle, tf, K0):
+    """A small output against a long K (144 x 130 outputs, 32 KB of K per row):
+    the 64x64 kernel, whose four waves already split K inside the workgroup,
+    splits it over workgroups as well. Against the oracle on the reference
+    tests' values (integers exact; float sums exact in any order), ACCUMULATE
+    off and on, and more than one slice reported."""
+    lib, torch = gpu
+    lib.set_kernel_mode(uk.KERNEL_MODE_AUTO)
+    bits = uk.MMT4D_TYPE_BITS[tf][0]
+    K1 = 32768 * 8 // bits // K0
+    for ci, c in enumerate(T.mmt4d_cases(tf, 16, 16, K0, seed=61, slack=16, shapes=((9, 9, K1),))):
+        lhs, rhs, out0 = T.make_mmt4d_buffers(c, np.random.default_rng(ci))
+        want = out0.copy()
+        G.run_mmt4d_case(oracle, c, lhs, rhs, want)
+        got = T.gpu_mmt4d(lib, torch, c, lhs, rhs, out0, allow_generic=False)
+        assert lib.last_kernel_name() == "mmt4d_mfma_64x64_ksplit", lib.last_kernel_name()
+        assert lib.last_k_slices() > 1
+        assert np.array_equal(got, want), c.label()
