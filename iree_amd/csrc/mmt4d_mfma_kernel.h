@@ -637,6 +637,18 @@ void mmt4d_mfma_kernel(Args a) {
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = TT::mfma(fb[tn], fa[tm], acc[tm][tn]);
   };
+  // The same sweep column by column (consecutive instructions share the RHS
+  // fragment): what the LDS-direct pipeline's compute phases issue. Measured
+  // against the row-by-row sweep in alternating processes on one box, three
+  // pairs: s8 8192^3 374.8 / 378.9 / 376.4 -> 371.7 / 371.7 / 375.2 us,
+  // 16x16x2 382.0 / 382.5 / 384.5 -> 378.5 / 379.4 / 382.2, f16 4096^3 91.2 /
+  // 91.3 / 91.3 -> 90.8 / 90.7 / 90.6, bf16 8192^3 unchanged.
+  auto mfmas_by_columns = [&](const v4i (&fa)[TM][HALVES], const v4i (&fb)[TN][HALVES]) {
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) acc[tm][tn] = TT::mfma(fb[tn], fa[tm], acc[tm][tn]);
+  };
   const int last = a.steps - 1;
   const bool has_tail = a.tail != 0;
 
@@ -1375,7 +1387,7 @@ void mmt4d_mfma_kernel(Args a) {
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
-        mfmas(fa, fb);
+        mfmas_by_columns(fa, fb);
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         if (group == 0) wait_vmem_in_flight<DU*(D - 2)>();   // the second half of step s + 1 has landed
@@ -1453,7 +1465,7 @@ void mmt4d_mfma_kernel(Args a) {
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
 #pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) mfmas(fa[kk], fb[kk]);
+        for (int kk = 0; kk < NKK; ++kk) mfmas_by_columns(fa[kk], fb[kk]);
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
