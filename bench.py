@@ -683,6 +683,16 @@ def main() -> int:
                                       "copy2d_frac": e["copy2d_ceiling"]["cold_frac"],
                                       "copy2d_unpack_frac": e["copy2d_ceiling_unpack"]["cold_frac"]},
                              "round_trip_bit_exact": e["parity"]["round_trip_bit_exact"]}
+        e = extra.get("pack_operand_forms")
+        if e:
+            ks = e["kernels"].values()
+            targets["pack_operand_forms"] = {
+                "kernels": sorted({k["kernel"] for k in ks}),
+                # launches on the same buffers (source in the memory-side cache) / that cache emptied before each
+                "frac_same_buffers": [round(min(k["frac"] for k in ks), 3), round(max(k["frac"] for k in ks), 3)],
+                "frac_cold": [round(min(k.get("cold_frac", float("nan")) for k in ks), 3),
+                              round(max(k.get("cold_frac", float("nan")) for k in ks), 3)],
+                "equals_reshape_permute": e["parity"]["ok"]}
         result["targets"] = targets
 
     R.close()
